@@ -1,0 +1,208 @@
+/*
+ * rstorch_hip.h - C ABI of the MI355X (gfx950) backend for the rstorch f64 training step.
+ *
+ * The reference crate is pure Rust and has no FFI of its own; its hot path sits behind the
+ * traits `Module` (src/module/mod.rs:42-56), `Loss` (src/loss/mod.rs:6-11) and `Optimizer`
+ * (src/optim/mod.rs:6-8).  These entry points are what a Rust (or C++/Python) implementation
+ * of those traits binds with `extern "C"`: plain pointers and sizes only.
+ *
+ * Conventions
+ *   - every matrix is dense row-major f64 without strides (the reference's Array2<f64>);
+ *     `double*` arguments are DEVICE pointers unless the name says `host`;
+ *   - every function returns an rst_status; on failure rst_last_error() gives a message for
+ *     the calling thread and rst_last_hip_error() the hipError_t, if HIP raised it.  The
+ *     reference panics in these situations (unwrap on a consumed cache, ndarray shape
+ *     mismatch, NaN in softmax); a binding turns the status into its own panic/exception;
+ *   - work is enqueued on the engine's stream and runs asynchronously; only the calls that
+ *     hand a value back to the host (downloads, the scalar loss) wait for it;
+ *   - one engine is used from one thread at a time (the reference is single-threaded,
+ *     nothing in it is Send/Sync).
+ */
+#ifndef RSTORCH_HIP_H
+#define RSTORCH_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum rst_status {
+  RST_OK = 0,
+  RST_ERR_INVALID_ARGUMENT = 1, /* null pointer, zero handle, bad enum */
+  RST_ERR_SHAPE = 2,            /* operand shapes do not agree (ndarray would panic) */
+  RST_ERR_STATE = 3,            /* backward before forward, step before backward, ... */
+  RST_ERR_HIP = 4,              /* a HIP call failed; see rst_last_hip_error() */
+  RST_ERR_NAN = 5,              /* NaN logits: the reference panics in softmax.rs:38 */
+  RST_ERR_OUT_OF_MEMORY = 6,
+  RST_ERR_UNSUPPORTED = 7
+} rst_status;
+
+typedef struct rst_engine rst_engine; /* one GPU + one stream + small scratch buffers */
+typedef struct rst_model rst_model;   /* a device-resident Sequential of Identity/Linear/ReLU */
+typedef struct rst_event rst_event;   /* a timestamp on the engine's stream */
+
+/* ---- errors ---------------------------------------------------------------------------- */
+const char* rst_last_error(void);
+int rst_last_hip_error(void);
+const char* rst_status_string(int status);
+
+/* ---- engine ---------------------------------------------------------------------------- */
+/* Opens device `device`, creates the stream every later call is ordered on. */
+int rst_engine_create(int device, rst_engine** out);
+int rst_engine_destroy(rst_engine* engine);
+/* Blocks until everything enqueued so far has finished. */
+int rst_engine_synchronize(rst_engine* engine);
+/* The hipStream_t, for callers that order their own HIP work against the engine's. */
+void* rst_engine_stream(rst_engine* engine);
+/* Device name and number of compute units (for reports). */
+int rst_engine_device_info(rst_engine* engine, char* name, size_t name_capacity,
+                           int* compute_units, size_t* total_memory_bytes);
+
+/* ---- device memory (counts are numbers of doubles) -------------------------------------- */
+int rst_malloc(rst_engine* engine, size_t count, double** out);
+int rst_free(rst_engine* engine, double* ptr);
+int rst_upload(rst_engine* engine, double* dst, const double* host_src, size_t count);
+int rst_download(rst_engine* engine, double* host_dst, const double* src, size_t count);
+int rst_copy(rst_engine* engine, double* dst, const double* src, size_t count);
+int rst_fill(rst_engine* engine, double* dst, size_t count, double value);
+
+/* ---- timing on the engine's stream ------------------------------------------------------ */
+int rst_event_create(rst_engine* engine, rst_event** out);
+int rst_event_destroy(rst_event* event);
+int rst_event_record(rst_event* event);
+/* Waits for `stop` and returns the time between the two records in milliseconds. */
+int rst_event_elapsed_ms(rst_event* start, rst_event* stop, double* host_ms);
+
+/* ---- Linear (replaces src/module/linear.rs:43-57 and :60-69) ----------------------------- */
+/* out[batch,out_features] = x[batch,in_features] . weight[out_features,in_features]^T, then
+ * + bias[1,out_features] (bias may be NULL).  With fuse_relu != 0 the ReLU that follows the
+ * layer (src/module/activation/relu.rs:19-22) is applied in the same kernel: out = max(z, 0). */
+int rst_linear_forward(rst_engine* engine, const double* x, const double* weight,
+                       const double* bias, double* out, size_t batch, size_t in_features,
+                       size_t out_features, int fuse_relu);
+/* n = batch.  grad_weight[out,in] = (grad^T . x) / n;  grad_bias[1,out] = colsum(grad) / n
+ * (NULL: skipped);  grad_input[batch,in] = grad . weight, not scaled (NULL: skipped).
+ * relu_mask_source (may be NULL) is the [batch,in] pre-activation or output of a ReLU that
+ * fed this layer: grad_input is then multiplied by (source > 0 ? 1 : 0), which is that ReLU's
+ * backward (src/module/activation/relu.rs:25-27) fused into the epilogue. */
+int rst_linear_backward(rst_engine* engine, const double* grad, const double* x,
+                        const double* weight, double* grad_weight, double* grad_bias,
+                        double* grad_input, const double* relu_mask_source, size_t batch,
+                        size_t in_features, size_t out_features);
+
+/* ---- ReLU, unfused (src/module/activation/relu.rs:19-27) --------------------------------- */
+int rst_relu_forward(rst_engine* engine, const double* x, double* out, size_t count);
+/* out = grad * (x > 0 ? 1 : 0); x may be the pre-activation or the ReLU output. */
+int rst_relu_backward(rst_engine* engine, const double* grad, const double* x, double* out,
+                      size_t count);
+
+/* ---- softmax over each row (src/module/activation/softmax.rs:45-53, axis 1) -------------- */
+/* Returns RST_ERR_NAN when a logit is NaN (checked when the call returns: this call waits). */
+int rst_softmax_rows(rst_engine* engine, const double* x, double* out, size_t rows, size_t cols);
+
+/* ---- CrossEntropyLoss (src/loss/cross_entropy.rs:34-47) ---------------------------------- */
+/* One pass: prob = softmax(pred); loss = -(sum truth*ln(prob)) / rows; grad_out = prob - truth
+ * (what `backward()` returns; NOT divided by rows).  prob_out may be NULL.  host_loss may be
+ * NULL, in which case nothing waits and the loss stays in the engine (rst_loss_value). */
+int rst_cross_entropy(rst_engine* engine, const double* pred, const double* truth,
+                      double* grad_out, double* prob_out, size_t rows, size_t cols,
+                      double* host_loss);
+/* The loss of the latest rst_cross_entropy on this engine; waits for it.  RST_ERR_NAN if a
+ * logit was NaN. */
+int rst_loss_value(rst_engine* engine, double* host_loss);
+
+/* ---- SGD (src/optim/sgd.rs:19-24) -------------------------------------------------------- */
+/* parm[i] = parm[i] - (lr * grad[i]) for every tensor in ONE launch: the product is rounded,
+ * then the difference (no fused multiply-add), as in the reference.  The arrays are HOST
+ * arrays of `tensor_count` device pointers / element counts. */
+int rst_sgd_step(rst_engine* engine, double* const* host_parm_ptrs,
+                 const double* const* host_grad_ptrs, const size_t* host_counts,
+                 size_t tensor_count, double lr);
+/* Same update over one contiguous range (a parameter arena). */
+int rst_sgd_step_flat(rst_engine* engine, double* parm, const double* grad, size_t count,
+                      double lr);
+
+/* ---- accuracy (src/utils.rs:44-65) ------------------------------------------------------- */
+/* Fraction of rows whose arg-max column (first maximum wins) agrees between pred and truth. */
+int rst_accuracy(rst_engine* engine, const double* pred, const double* truth, size_t rows,
+                 size_t cols, double* host_accuracy);
+
+/* ---- synthetic data and initialisers (src/module/init/{mod,he,xavier,sigma}.rs) ----------- */
+/* value(seed, stream, index) is a pure function (counter-based generator), so a tensor does
+ * not depend on launch geometry.  The reference draws from an unseedable thread RNG; these
+ * give the same distributions reproducibly: KaimingNormal is std = 1/sqrt(in_features). */
+int rst_fill_uniform(rst_engine* engine, double* dst, size_t count, uint64_t seed,
+                     uint64_t stream, double lo, double hi);
+int rst_fill_normal(rst_engine* engine, double* dst, size_t count, uint64_t seed,
+                    uint64_t stream, double mean, double std);
+/* dst[rows,cols] = one-hot rows with labels uniform over the columns (src/utils.rs:38-42). */
+int rst_fill_one_hot(rst_engine* engine, double* dst, size_t rows, size_t cols, uint64_t seed,
+                     uint64_t stream);
+
+/* ---- device-resident Sequential (src/module/sequential.rs:78-109) ------------------------ */
+enum { RST_LAYER_IDENTITY = 0, RST_LAYER_LINEAR = 1, RST_LAYER_RELU = 2 };
+
+/* kinds[i] is one of RST_LAYER_*; in_features/out_features are read for LINEAR entries.
+ * All weights, biases and their gradients live in two contiguous device arenas (parameters
+ * and gradients, same layout), zero-initialised. */
+int rst_model_create(rst_engine* engine, const int* kinds, const size_t* in_features,
+                     const size_t* out_features, size_t layer_count, rst_model** out);
+int rst_model_destroy(rst_model* model);
+/* Number of parameter tensors (2 per Linear) and total number of f64 parameters. */
+int rst_model_parameter_count(rst_model* model, size_t* tensor_count, size_t* element_count);
+/* Tensor `index` in the reference's order (per Linear in layer order: weight (out,in), then
+ * bias (1,out); src/module/linear.rs:71-78): device pointers of the parameter and its gradient. */
+int rst_model_parameter(rst_model* model, size_t index, double** parm, double** grad,
+                        size_t* rows, size_t* cols);
+/* KaimingNormal weights (std = 1/sqrt(in)), zero biases (src/module/init/mod.rs:15-17,
+ * he.rs:11-14); tensor i uses generator stream `first_stream + i`. */
+int rst_model_init_kaiming(rst_model* model, uint64_t seed, uint64_t first_stream);
+/* forward: x[batch, in] -> *logits (device pointer owned by the model, [batch, out]).
+ * Linear+ReLU pairs run as one kernel; the input is referenced, not copied, until backward. */
+int rst_model_forward(rst_model* model, const double* x, size_t batch, const double** logits);
+/* CrossEntropyLoss::forward on the logits of the last forward (truth[batch, classes], dense).
+ * host_loss may be NULL (no wait).  Keeps prob - truth for rst_model_backward. */
+int rst_model_loss(rst_model* model, const double* truth, double* host_loss);
+/* Sequential::backward.  grad == NULL: start from the gradient rst_model_loss kept
+ * (loss.backward()); otherwise from grad[batch, out].  need_input_grad == 0 skips the first
+ * Linear's input gradient, which the README loop discards; otherwise *input_grad receives it. */
+int rst_model_backward(rst_model* model, const double* grad, int need_input_grad,
+                       const double** input_grad);
+/* SGD::step over every parameter of the model (one launch over the arena). */
+int rst_model_sgd_step(rst_model* model, double lr);
+/* forward, loss, backward, step: the README loop body (README.md:64-74) without accuracy,
+ * i.e. what the reference's private BasicModel::step (src/model.rs:19-27) does.
+ * host_loss may be NULL: then the call returns without waiting for the GPU. */
+int rst_model_train_step(rst_model* model, const double* x, const double* truth, size_t batch,
+                         double lr, double* host_loss);
+/* Per-launch timing of the model's kernels: when enabled every launch is bracketed by events
+ * (this serialises nothing, the stream is already in order).  After a synchronising call,
+ * rst_model_profile_read returns up to `capacity` records of the latest step. */
+typedef struct rst_kernel_record {
+  int kind;          /* RST_KERNEL_* */
+  int layer;         /* layer index, -1 for loss / optimiser */
+  double ms;         /* launch duration */
+  double flops;      /* algorithmic flops (2*M*N*K for the contractions, else 0) */
+  double bytes;      /* algorithmic HBM bytes */
+} rst_kernel_record;
+enum {
+  RST_KERNEL_LINEAR_FORWARD = 0,
+  RST_KERNEL_GRAD_WEIGHT = 1,
+  RST_KERNEL_GRAD_BIAS = 2,
+  RST_KERNEL_GRAD_INPUT = 3,
+  RST_KERNEL_RELU_FORWARD = 4,
+  RST_KERNEL_RELU_BACKWARD = 5,
+  RST_KERNEL_CROSS_ENTROPY = 6,
+  RST_KERNEL_LOSS_REDUCE = 7,
+  RST_KERNEL_SGD = 8
+};
+int rst_model_profile_enable(rst_model* model, int enabled);
+int rst_model_profile_read(rst_model* model, rst_kernel_record* host_records, size_t capacity,
+                           size_t* count);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RSTORCH_HIP_H */

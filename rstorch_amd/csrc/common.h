@@ -1,0 +1,129 @@
+// Shared declarations of the gfx950 backend: engine state, error plumbing and the internal
+// launch functions that the C ABI (ops.hip, model.hip) is built from.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "../../include/rstorch_hip.h"
+
+namespace rst {
+
+// ---- error plumbing ------------------------------------------------------------------------
+int fail(int status, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int fail_hip(hipError_t err, const char* what, const char* file, int line);
+void clear_error();
+
+#define RST_HIP(expr)                                                          \
+  do {                                                                         \
+    hipError_t rst_hip_err_ = (expr);                                          \
+    if (rst_hip_err_ != hipSuccess)                                            \
+      return ::rst::fail_hip(rst_hip_err_, #expr, __FILE__, __LINE__);         \
+  } while (0)
+
+#define RST_TRY(expr)                      \
+  do {                                     \
+    int rst_status_ = (expr);              \
+    if (rst_status_ != RST_OK) return rst_status_; \
+  } while (0)
+
+// ---- epilogues of the contraction kernels ----------------------------------------------------
+enum Epilogue {
+  EPI_NONE = 0,
+  EPI_BIAS = 1,       // C = acc + bias[col]                       (Linear forward)
+  EPI_BIAS_RELU = 2,  // C = max(acc + bias[col], 0)               (Linear forward + ReLU)
+  EPI_DIVIDE = 3,     // C = acc / divisor                         (weight gradient)
+  EPI_MASK = 4,       // C = acc * (mask[row,col] > 0 ? 1 : 0)     (input gradient + ReLU backward)
+  EPI_RELU = 5        // C = max(acc, 0)                           (Linear without bias + ReLU)
+};
+
+// C[M,N] = sum_k A(i,k) * B(k,j), every matrix dense row-major.
+//   a_kc: A(i,k) = A[i*lda + k]  (contraction index contiguous), else A(i,k) = A[k*lda + i]
+//   b_kc: B(k,j) = B[j*ldb + k]  (contraction index contiguous), else B(k,j) = B[k*ldb + j]
+struct GemmDesc {
+  const double* A;
+  const double* B;
+  double* C;
+  int M, N, K;
+  long lda, ldb, ldc;
+  bool a_kc, b_kc;
+  int epilogue;
+  const double* bias;  // [N]
+  double divisor;
+  const double* mask;  // [M, ldmask]
+  long ldmask;
+};
+
+int launch_gemm(hipStream_t stream, const GemmDesc& d);
+
+// ---- streaming kernels -----------------------------------------------------------------------
+int launch_relu_forward(hipStream_t s, const double* x, double* out, size_t n);
+int launch_relu_backward(hipStream_t s, const double* g, const double* x, double* out, size_t n);
+int launch_fill(hipStream_t s, double* dst, size_t n, double value);
+// out[j] = (sum_r g[r, j]) / divisor, rows added in order inside fixed groups (deterministic)
+int launch_column_mean(hipStream_t s, const double* g, double* out, size_t rows, size_t cols,
+                       double divisor);
+int launch_sgd_flat(hipStream_t s, double* parm, const double* grad, size_t n, double lr);
+
+struct SgdTensor {
+  double* parm;
+  const double* grad;
+  unsigned long long count;
+  unsigned long long first_block;  // prefix of blocks, filled by the launcher
+};
+// table: device copy of `n_tensors` SgdTensor entries followed by a sentinel
+int launch_sgd_multi(hipStream_t s, const SgdTensor* device_table, size_t n_tensors,
+                     unsigned long long total_blocks, double lr);
+unsigned long long sgd_blocks_for(unsigned long long count);
+
+// softmax / cross entropy.  row_loss: [rows] scratch; flags[0] is set to 1 on a NaN logit.
+int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* grad_out,
+                      double* prob_out, double* row_loss, int* flags, size_t rows, size_t cols);
+// loss[0] = -(sum row_loss) / rows, fixed summation order
+int launch_loss_reduce(hipStream_t s, const double* row_loss, double* loss, size_t rows);
+// hits[0] = number of rows whose first arg-max agrees
+int launch_accuracy(hipStream_t s, const double* pred, const double* truth, size_t rows,
+                    size_t cols, unsigned long long* hits);
+
+int launch_fill_uniform(hipStream_t s, double* dst, size_t n, uint64_t seed, uint64_t stream,
+                        double lo, double hi);
+int launch_fill_normal(hipStream_t s, double* dst, size_t n, uint64_t seed, uint64_t stream,
+                       double mean, double std);
+int launch_fill_one_hot(hipStream_t s, double* dst, size_t rows, size_t cols, uint64_t seed,
+                        uint64_t stream);
+
+}  // namespace rst
+
+// ---- engine ------------------------------------------------------------------------------------
+struct rst_engine {
+  int device = 0;
+  hipStream_t stream = nullptr;
+  hipDeviceProp_t props;
+  // device-side scalars and their pinned host mirrors
+  double* d_loss = nullptr;
+  int* d_flags = nullptr;
+  unsigned long long* d_hits = nullptr;
+  double* h_loss = nullptr;  // pinned
+  int* h_flags = nullptr;    // pinned
+  unsigned long long* h_hits = nullptr;  // pinned
+  bool loss_valid = false;
+  // per-row loss scratch
+  double* d_row_loss = nullptr;
+  size_t row_loss_capacity = 0;
+  // SGD descriptor table cache
+  rst::SgdTensor* d_sgd_table = nullptr;
+  size_t sgd_table_capacity = 0;
+  std::vector<rst::SgdTensor> sgd_table_host;
+  unsigned long long sgd_total_blocks = 0;
+};
+
+namespace rst {
+int engine_activate(rst_engine* e);
+int engine_reserve_row_loss(rst_engine* e, size_t rows);
+int engine_cross_entropy(rst_engine* e, const double* pred, const double* truth, double* grad_out,
+                         double* prob_out, size_t rows, size_t cols, double* host_loss);
+}  // namespace rst

@@ -1,0 +1,495 @@
+// Device-resident Sequential of Identity / Linear / ReLU layers with CrossEntropyLoss and SGD:
+// the whole training step as an ordered list of launches on the engine's stream, weights,
+// gradients and activations staying in HBM between layers.
+//
+// Fusion plan (decided per call, so it follows whatever layer list the model was built with):
+//   forward : a Linear whose next non-Identity layer is a ReLU writes max(z, 0) directly;
+//   backward: a Linear whose input came out of a ReLU multiplies its input gradient by
+//             (input > 0) in the contraction epilogue, which is that ReLU's backward
+//             ([relu(z) > 0] == [z > 0], NaN included, both false);
+//   any ReLU not adjacent to a Linear runs the streaming kernels instead.
+#include <climits>
+#include <new>
+
+#include "common.h"
+
+using namespace rst;
+
+namespace {
+
+constexpr size_t kAlign = 32;  // doubles: every tensor starts on a 256-byte boundary
+
+size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+struct Layer {
+  int kind = RST_LAYER_IDENTITY;
+  size_t in = 0, out = 0;  // Linear only
+  size_t width_in = 0, width_out = 0;
+  // Linear parameters (into the arenas)
+  double *w = nullptr, *b = nullptr, *gw = nullptr, *gb = nullptr;
+  // forward
+  double* out_buf = nullptr;      // Linear: [batch,out]; unfused ReLU: [batch,width]
+  const double* input = nullptr;  // what the layer saw in forward (Linear: x; ReLU: pre-activation)
+  bool relu_fused = false;        // Linear: the following ReLU was applied in its epilogue
+  bool absorbed = false;          // ReLU: forward ran inside the preceding Linear
+  const double* mask_source = nullptr;  // ReLU: tensor whose sign gives the backward mask
+  // backward
+  double* grad_in_buf = nullptr;  // gradient w.r.t. the layer input
+  bool backward_absorbed = false; // ReLU: backward ran inside the following Linear's epilogue
+};
+
+struct ProfileSlot {
+  int kind, layer;
+  double flops, bytes;
+  hipEvent_t start, stop;
+};
+
+}  // namespace
+
+struct rst_model {
+  rst_engine* engine = nullptr;
+  std::vector<Layer> layers;
+  size_t in_width = 0, out_width = 0;
+  bool has_linear = false;
+  // arenas
+  double* parm_arena = nullptr;
+  double* grad_arena = nullptr;
+  size_t arena_count = 0;    // doubles, padding included
+  size_t element_count = 0;  // real parameters
+  size_t tensor_count = 0;
+  // activations
+  size_t batch_capacity = 0;
+  size_t batch = 0;
+  double* loss_grad = nullptr;  // [batch, out_width]
+  const double* logits = nullptr;
+  // state machine (mirrors the Option::take() caches of the reference)
+  bool forward_valid = false;
+  bool loss_grad_valid = false;
+  bool grads_valid = false;
+  // profiling
+  bool profiling = false;
+  std::vector<ProfileSlot> slots;
+  std::vector<hipEvent_t> event_pool;
+  size_t events_used = 0;
+};
+
+namespace {
+
+int free_activations(rst_model* m) {
+  for (auto& l : m->layers) {
+    if (l.out_buf) RST_HIP(hipFree(l.out_buf));
+    if (l.grad_in_buf) RST_HIP(hipFree(l.grad_in_buf));
+    l.out_buf = l.grad_in_buf = nullptr;
+  }
+  if (m->loss_grad) RST_HIP(hipFree(m->loss_grad));
+  m->loss_grad = nullptr;
+  m->batch_capacity = 0;
+  return RST_OK;
+}
+
+int reserve_activations(rst_model* m, size_t batch) {
+  if (batch <= m->batch_capacity) return RST_OK;
+  RST_HIP(hipStreamSynchronize(m->engine->stream));
+  RST_TRY(free_activations(m));
+  for (auto& l : m->layers) {
+    if (l.kind == RST_LAYER_IDENTITY) continue;
+    size_t n_out = batch * l.width_out, n_in = batch * l.width_in;
+    RST_HIP(hipMalloc(&l.out_buf, (n_out ? n_out : 1) * sizeof(double)));
+    RST_HIP(hipMalloc(&l.grad_in_buf, (n_in ? n_in : 1) * sizeof(double)));
+  }
+  size_t n = batch * m->out_width;
+  RST_HIP(hipMalloc(&m->loss_grad, (n ? n : 1) * sizeof(double)));
+  m->batch_capacity = batch;
+  return RST_OK;
+}
+
+// ---- profiling helpers --------------------------------------------------------------------
+int prof_begin(rst_model* m, int kind, int layer, double flops, double bytes) {
+  if (!m->profiling) return RST_OK;
+  while (m->event_pool.size() < m->events_used + 2) {
+    hipEvent_t ev;
+    RST_HIP(hipEventCreate(&ev));
+    m->event_pool.push_back(ev);
+  }
+  ProfileSlot s;
+  s.kind = kind; s.layer = layer; s.flops = flops; s.bytes = bytes;
+  s.start = m->event_pool[m->events_used++];
+  s.stop = m->event_pool[m->events_used++];
+  RST_HIP(hipEventRecord(s.start, m->engine->stream));
+  m->slots.push_back(s);
+  return RST_OK;
+}
+
+int prof_end(rst_model* m) {
+  if (!m->profiling) return RST_OK;
+  RST_HIP(hipEventRecord(m->slots.back().stop, m->engine->stream));
+  return RST_OK;
+}
+
+void prof_reset(rst_model* m) {
+  m->slots.clear();
+  m->events_used = 0;
+}
+
+int prev_non_identity(const rst_model* m, int i) {
+  for (int j = i - 1; j >= 0; --j)
+    if (m->layers[j].kind != RST_LAYER_IDENTITY) return j;
+  return -1;
+}
+int next_non_identity(const rst_model* m, int i) {
+  for (int j = i + 1; j < (int)m->layers.size(); ++j)
+    if (m->layers[j].kind != RST_LAYER_IDENTITY) return j;
+  return -1;
+}
+
+int do_forward(rst_model* m, const double* x, size_t batch) {
+  rst_engine* e = m->engine;
+  if (batch > (size_t)INT_MAX) return fail(RST_ERR_UNSUPPORTED, "batch too large");
+  RST_TRY(reserve_activations(m, batch));
+  m->batch = batch;
+  const double* cur = x;
+  const int n = (int)m->layers.size();
+  for (auto& l : m->layers) { l.absorbed = false; l.relu_fused = false; l.backward_absorbed = false; }
+  for (int i = 0; i < n; ++i) {
+    Layer& l = m->layers[i];
+    if (l.kind == RST_LAYER_IDENTITY) continue;  // identity.rs:17-19
+    if (l.kind == RST_LAYER_LINEAR) {
+      const int nx = next_non_identity(m, i);
+      const bool fuse = nx >= 0 && m->layers[nx].kind == RST_LAYER_RELU;
+      l.input = cur;  // linear.rs:56 keeps the input for backward
+      l.relu_fused = fuse;
+      GemmDesc d{};
+      d.A = cur; d.B = l.w; d.C = l.out_buf;
+      d.M = (int)batch; d.N = (int)l.out; d.K = (int)l.in;
+      d.lda = (long)l.in; d.ldb = (long)l.in; d.ldc = (long)l.out;
+      d.a_kc = true; d.b_kc = true;
+      d.epilogue = fuse ? EPI_BIAS_RELU : EPI_BIAS;
+      d.bias = l.b;
+      const double flops = 2.0 * (double)batch * (double)l.in * (double)l.out;
+      const double bytes = 8.0 * ((double)batch * l.in + (double)l.in * l.out + (double)batch * l.out);
+      RST_TRY(prof_begin(m, RST_KERNEL_LINEAR_FORWARD, i, flops, bytes));
+      RST_TRY(launch_gemm(e->stream, d));
+      RST_TRY(prof_end(m));
+      cur = l.out_buf;
+      if (fuse) {
+        Layer& r = m->layers[nx];
+        r.absorbed = true;
+        r.input = nullptr;
+        r.mask_source = l.out_buf;  // relu(z) > 0 == z > 0
+      }
+    } else {  // ReLU
+      if (l.absorbed) continue;  // its output already is `cur`
+      const size_t cnt = batch * l.width_in;
+      l.input = cur;        // relu.rs:20 keeps the pre-activation
+      l.mask_source = cur;
+      RST_TRY(prof_begin(m, RST_KERNEL_RELU_FORWARD, i, 0.0, 16.0 * (double)cnt));
+      RST_TRY(launch_relu_forward(e->stream, cur, l.out_buf, cnt));
+      RST_TRY(prof_end(m));
+      cur = l.out_buf;
+    }
+  }
+  m->logits = cur;
+  m->forward_valid = true;
+  m->loss_grad_valid = false;
+  return RST_OK;
+}
+
+int do_loss(rst_model* m, const double* truth, double* host_loss) {
+  rst_engine* e = m->engine;
+  if (!m->forward_valid) return fail(RST_ERR_STATE, "loss before forward");
+  if (!truth) return fail(RST_ERR_INVALID_ARGUMENT, "truth is null");
+  const size_t rows = m->batch, cols = m->out_width;
+  RST_TRY(prof_begin(m, RST_KERNEL_CROSS_ENTROPY, -1, 0.0, 24.0 * (double)rows * (double)cols));
+  RST_TRY(engine_cross_entropy(e, m->logits, truth, m->loss_grad, nullptr, rows, cols, nullptr));
+  RST_TRY(prof_end(m));
+  m->loss_grad_valid = true;
+  if (host_loss) return rst_loss_value(e, host_loss);
+  return RST_OK;
+}
+
+int do_backward(rst_model* m, const double* grad, int need_input_grad, const double** input_grad) {
+  rst_engine* e = m->engine;
+  if (!m->forward_valid)
+    return fail(RST_ERR_STATE, "backward without a forward (the reference panics on a consumed cache)");
+  if (!grad) {
+    if (!m->loss_grad_valid) return fail(RST_ERR_STATE, "backward from the loss before the loss was computed");
+    grad = m->loss_grad;
+  }
+  const size_t batch = m->batch;
+  const double n_rows = (double)batch;
+  const double* cur = grad;
+  const int n = (int)m->layers.size();
+  int first_linear = -1;
+  for (int i = 0; i < n; ++i)
+    if (m->layers[i].kind == RST_LAYER_LINEAR) { first_linear = i; break; }
+
+  for (int i = n - 1; i >= 0; --i) {
+    Layer& l = m->layers[i];
+    if (l.kind == RST_LAYER_IDENTITY) continue;  // identity.rs:22-24
+    if (l.kind == RST_LAYER_RELU) {
+      if (l.backward_absorbed) continue;
+      const size_t cnt = batch * l.width_in;
+      RST_TRY(prof_begin(m, RST_KERNEL_RELU_BACKWARD, i, 0.0, 24.0 * (double)cnt));
+      RST_TRY(launch_relu_backward(e->stream, cur, l.mask_source, l.grad_in_buf, cnt));
+      RST_TRY(prof_end(m));
+      cur = l.grad_in_buf;
+      continue;
+    }
+    // Linear: linear.rs:60-69
+    const double mnk = (double)batch * (double)l.in * (double)l.out;
+    {
+      GemmDesc d{};
+      d.A = cur; d.B = l.input; d.C = l.gw;
+      d.M = (int)l.out; d.N = (int)l.in; d.K = (int)batch;
+      d.lda = (long)l.out; d.ldb = (long)l.in; d.ldc = (long)l.in;
+      d.a_kc = false; d.b_kc = false;
+      d.epilogue = EPI_DIVIDE; d.divisor = n_rows;
+      const double bytes = 8.0 * ((double)batch * l.out + (double)batch * l.in + (double)l.in * l.out);
+      RST_TRY(prof_begin(m, RST_KERNEL_GRAD_WEIGHT, i, 2.0 * mnk, bytes));
+      RST_TRY(launch_gemm(e->stream, d));
+      RST_TRY(prof_end(m));
+    }
+    RST_TRY(prof_begin(m, RST_KERNEL_GRAD_BIAS, i, 0.0, 8.0 * ((double)batch * l.out + l.out)));
+    RST_TRY(launch_column_mean(e->stream, cur, l.gb, batch, l.out, n_rows));
+    RST_TRY(prof_end(m));
+
+    const bool wanted = need_input_grad || i != first_linear;
+    if (!wanted) { cur = nullptr; break; }
+    const int pv = prev_non_identity(m, i);
+    const bool mask = pv >= 0 && m->layers[pv].kind == RST_LAYER_RELU;
+    GemmDesc d{};
+    d.A = cur; d.B = l.w; d.C = l.grad_in_buf;
+    d.M = (int)batch; d.N = (int)l.in; d.K = (int)l.out;
+    d.lda = (long)l.out; d.ldb = (long)l.in; d.ldc = (long)l.in;
+    d.a_kc = true; d.b_kc = false;
+    d.epilogue = mask ? EPI_MASK : EPI_NONE;
+    d.mask = mask ? l.input : nullptr;  // the ReLU's output is this layer's input
+    d.ldmask = (long)l.in;
+    const double bytes = 8.0 * ((double)batch * l.out + (double)l.in * l.out +
+                                (double)batch * l.in * (mask ? 2.0 : 1.0));
+    RST_TRY(prof_begin(m, RST_KERNEL_GRAD_INPUT, i, 2.0 * mnk, bytes));
+    RST_TRY(launch_gemm(e->stream, d));
+    RST_TRY(prof_end(m));
+    if (mask) m->layers[pv].backward_absorbed = true;
+    cur = l.grad_in_buf;
+  }
+  if (input_grad) *input_grad = cur;
+  // the caches are consumed (Option::take in linear.rs:61, relu.rs:26, cross_entropy.rs:46)
+  m->forward_valid = false;
+  m->loss_grad_valid = false;
+  m->grads_valid = true;
+  return RST_OK;
+}
+
+int do_sgd(rst_model* m, double lr) {
+  if (!m->has_linear) return RST_OK;
+  if (!m->grads_valid)
+    return fail(RST_ERR_STATE, "optimizer step before any backward (the reference panics unwrapping the gradient)");
+  RST_TRY(prof_begin(m, RST_KERNEL_SGD, -1, 0.0, 24.0 * (double)m->element_count));
+  RST_TRY(launch_sgd_flat(m->engine->stream, m->parm_arena, m->grad_arena, m->arena_count, lr));
+  RST_TRY(prof_end(m));
+  return RST_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rst_model_create(rst_engine* e, const int* kinds, const size_t* in_features,
+                     const size_t* out_features, size_t layer_count, rst_model** out) {
+  RST_TRY(engine_activate(e));
+  if (!out) return fail(RST_ERR_INVALID_ARGUMENT, "out is null");
+  *out = nullptr;
+  if (layer_count && !kinds) return fail(RST_ERR_INVALID_ARGUMENT, "kinds is null");
+  rst_model* m = new (std::nothrow) rst_model();
+  if (!m) return fail(RST_ERR_OUT_OF_MEMORY, "host allocation failed");
+  m->engine = e;
+  m->layers.resize(layer_count);
+  size_t offset = 0;
+  size_t width = 0;
+  bool width_known = false;
+  for (size_t i = 0; i < layer_count; ++i) {
+    Layer& l = m->layers[i];
+    l.kind = kinds[i];
+    if (l.kind == RST_LAYER_LINEAR) {
+      if (!in_features || !out_features) { delete m; return fail(RST_ERR_INVALID_ARGUMENT, "feature arrays are null"); }
+      l.in = in_features[i];
+      l.out = out_features[i];
+      if (l.in > (size_t)INT_MAX || l.out > (size_t)INT_MAX) { delete m; return fail(RST_ERR_UNSUPPORTED, "layer too wide"); }
+      if (width_known && width != l.in) {
+        int status = fail(RST_ERR_SHAPE, "layer %zu expects %zu inputs but receives %zu", i, l.in, width);
+        delete m;
+        return status;
+      }
+      if (!m->has_linear) m->in_width = l.in;
+      m->has_linear = true;
+      width = l.out;
+      width_known = true;
+      offset = round_up(offset, kAlign) + l.in * l.out;
+      offset = round_up(offset, kAlign) + l.out;
+      m->element_count += l.in * l.out + l.out;
+      m->tensor_count += 2;
+    } else if (l.kind != RST_LAYER_IDENTITY && l.kind != RST_LAYER_RELU) {
+      int status = fail(RST_ERR_INVALID_ARGUMENT, "layer %zu has unknown kind %d", i, l.kind);
+      delete m;
+      return status;
+    }
+  }
+  if (!m->has_linear) {
+    delete m;
+    return fail(RST_ERR_UNSUPPORTED, "a device model needs at least one Linear layer to fix its width");
+  }
+  m->out_width = width;
+  // widths flowing through every layer
+  width = m->in_width;
+  for (auto& l : m->layers) {
+    l.width_in = width;
+    if (l.kind == RST_LAYER_LINEAR) width = l.out;
+    l.width_out = width;
+  }
+  m->arena_count = round_up(offset, kAlign);
+  hipError_t err = hipMalloc(&m->parm_arena, m->arena_count * sizeof(double));
+  if (err == hipSuccess) err = hipMalloc(&m->grad_arena, m->arena_count * sizeof(double));
+  if (err != hipSuccess) {
+    int status = fail_hip(err, "parameter arena allocation", __FILE__, __LINE__);
+    rst_model_destroy(m);
+    return status;
+  }
+  int status = launch_fill(e->stream, m->parm_arena, m->arena_count, 0.0);
+  if (status == RST_OK) status = launch_fill(e->stream, m->grad_arena, m->arena_count, 0.0);
+  if (status != RST_OK) { rst_model_destroy(m); return status; }
+  offset = 0;
+  for (auto& l : m->layers) {
+    if (l.kind != RST_LAYER_LINEAR) continue;
+    offset = round_up(offset, kAlign);
+    l.w = m->parm_arena + offset; l.gw = m->grad_arena + offset;
+    offset += l.in * l.out;
+    offset = round_up(offset, kAlign);
+    l.b = m->parm_arena + offset; l.gb = m->grad_arena + offset;
+    offset += l.out;
+  }
+  *out = m;
+  return RST_OK;
+}
+
+int rst_model_destroy(rst_model* m) {
+  if (!m) return RST_OK;
+  (void)hipSetDevice(m->engine->device);
+  (void)hipStreamSynchronize(m->engine->stream);
+  (void)free_activations(m);
+  if (m->parm_arena) (void)hipFree(m->parm_arena);
+  if (m->grad_arena) (void)hipFree(m->grad_arena);
+  for (hipEvent_t ev : m->event_pool) (void)hipEventDestroy(ev);
+  delete m;
+  return RST_OK;
+}
+
+int rst_model_parameter_count(rst_model* m, size_t* tensor_count, size_t* element_count) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  if (tensor_count) *tensor_count = m->tensor_count;
+  if (element_count) *element_count = m->element_count;
+  return RST_OK;
+}
+
+int rst_model_parameter(rst_model* m, size_t index, double** parm, double** grad, size_t* rows,
+                        size_t* cols) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  size_t k = 0;
+  for (auto& l : m->layers) {
+    if (l.kind != RST_LAYER_LINEAR) continue;
+    if (index == k || index == k + 1) {
+      const bool is_w = index == k;
+      if (parm) *parm = is_w ? l.w : l.b;
+      if (grad) *grad = is_w ? l.gw : l.gb;
+      if (rows) *rows = is_w ? l.out : 1;
+      if (cols) *cols = is_w ? l.in : l.out;
+      return RST_OK;
+    }
+    k += 2;
+  }
+  return fail(RST_ERR_INVALID_ARGUMENT, "parameter index %zu out of range (%zu tensors)", index, k);
+}
+
+int rst_model_init_kaiming(rst_model* m, uint64_t seed, uint64_t first_stream) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  RST_TRY(engine_activate(m->engine));
+  uint64_t stream = first_stream;
+  for (auto& l : m->layers) {
+    if (l.kind != RST_LAYER_LINEAR) continue;
+    const double sigma = 1.0 / sqrt((double)l.in);  // he.rs:12
+    RST_TRY(launch_fill_normal(m->engine->stream, l.w, l.in * l.out, seed, stream, 0.0, sigma));
+    RST_TRY(launch_fill(m->engine->stream, l.b, l.out, 0.0));  // init/mod.rs:15-17
+    stream += 2;
+  }
+  return RST_OK;
+}
+
+int rst_model_forward(rst_model* m, const double* x, size_t batch, const double** logits) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  RST_TRY(engine_activate(m->engine));
+  if (!x && batch) return fail(RST_ERR_INVALID_ARGUMENT, "x is null");
+  prof_reset(m);
+  RST_TRY(do_forward(m, x, batch));
+  if (logits) *logits = m->logits;
+  return RST_OK;
+}
+
+int rst_model_loss(rst_model* m, const double* truth, double* host_loss) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  RST_TRY(engine_activate(m->engine));
+  return do_loss(m, truth, host_loss);
+}
+
+int rst_model_backward(rst_model* m, const double* grad, int need_input_grad,
+                       const double** input_grad) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  RST_TRY(engine_activate(m->engine));
+  return do_backward(m, grad, need_input_grad, input_grad);
+}
+
+int rst_model_sgd_step(rst_model* m, double lr) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  RST_TRY(engine_activate(m->engine));
+  return do_sgd(m, lr);
+}
+
+int rst_model_train_step(rst_model* m, const double* x, const double* truth, size_t batch,
+                         double lr, double* host_loss) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  RST_TRY(engine_activate(m->engine));
+  if ((!x || !truth) && batch) return fail(RST_ERR_INVALID_ARGUMENT, "x or truth is null");
+  prof_reset(m);
+  RST_TRY(do_forward(m, x, batch));
+  RST_TRY(do_loss(m, truth, nullptr));
+  RST_TRY(do_backward(m, nullptr, 0, nullptr));
+  RST_TRY(do_sgd(m, lr));
+  if (host_loss) return rst_loss_value(m->engine, host_loss);
+  return RST_OK;
+}
+
+int rst_model_profile_enable(rst_model* m, int enabled) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->profiling = enabled != 0;
+  prof_reset(m);
+  return RST_OK;
+}
+
+int rst_model_profile_read(rst_model* m, rst_kernel_record* host_records, size_t capacity,
+                           size_t* count) {
+  if (!m || !count) return fail(RST_ERR_INVALID_ARGUMENT, "null argument");
+  RST_TRY(engine_activate(m->engine));
+  RST_HIP(hipStreamSynchronize(m->engine->stream));
+  *count = m->slots.size();
+  for (size_t i = 0; i < m->slots.size() && i < capacity && host_records; ++i) {
+    float ms = 0.f;
+    RST_HIP(hipEventElapsedTime(&ms, m->slots[i].start, m->slots[i].stop));
+    host_records[i].kind = m->slots[i].kind;
+    host_records[i].layer = m->slots[i].layer;
+    host_records[i].ms = (double)ms;
+    host_records[i].flops = m->slots[i].flops;
+    host_records[i].bytes = m->slots[i].bytes;
+  }
+  return RST_OK;
+}
+
+}  // extern "C"

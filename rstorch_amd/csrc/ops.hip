@@ -1,0 +1,229 @@
+// Operator-level C ABI: argument checking and dispatch onto the launch functions.  Each entry
+// point names the reference lines it replaces in include/rstorch_hip.h.
+#include <climits>
+#include <cstring>
+
+#include "common.h"
+
+using namespace rst;
+
+namespace rst {
+namespace {
+
+__global__ void reset_flags_kernel(int* flags) {
+  if (threadIdx.x < 4) flags[threadIdx.x] = 0;
+}
+
+int check_dim(size_t v, const char* what) {
+  if (v > (size_t)INT_MAX) return fail(RST_ERR_UNSUPPORTED, "%s = %zu exceeds 2^31-1", what, v);
+  return RST_OK;
+}
+
+}  // namespace
+
+int engine_cross_entropy(rst_engine* e, const double* pred, const double* truth, double* grad_out,
+                         double* prob_out, size_t rows, size_t cols, double* host_loss) {
+  RST_TRY(engine_reserve_row_loss(e, rows));
+  hipLaunchKernelGGL(reset_flags_kernel, dim3(1), dim3(64), 0, e->stream, e->d_flags);
+  RST_HIP(hipGetLastError());
+  RST_TRY(launch_softmax_ce(e->stream, pred, truth, grad_out, prob_out, e->d_row_loss, e->d_flags,
+                            rows, cols));
+  RST_TRY(launch_loss_reduce(e->stream, e->d_row_loss, e->d_loss, rows));
+  e->loss_valid = true;
+  if (host_loss) return rst_loss_value(e, host_loss);
+  return RST_OK;
+}
+
+}  // namespace rst
+
+extern "C" {
+
+int rst_linear_forward(rst_engine* e, const double* x, const double* weight, const double* bias,
+                       double* out, size_t batch, size_t in_features, size_t out_features,
+                       int fuse_relu) {
+  RST_TRY(engine_activate(e));
+  if (batch == 0 || out_features == 0) return RST_OK;
+  if (!out || !weight || (!x && in_features))
+    return fail(RST_ERR_INVALID_ARGUMENT, "linear_forward: null operand");
+  RST_TRY(check_dim(batch, "batch"));
+  RST_TRY(check_dim(in_features, "in_features"));
+  RST_TRY(check_dim(out_features, "out_features"));
+  GemmDesc d{};
+  d.A = x; d.B = weight; d.C = out;
+  d.M = (int)batch; d.N = (int)out_features; d.K = (int)in_features;
+  d.lda = (long)in_features; d.ldb = (long)in_features; d.ldc = (long)out_features;
+  d.a_kc = true; d.b_kc = true;
+  d.bias = bias;
+  if (bias) d.epilogue = fuse_relu ? EPI_BIAS_RELU : EPI_BIAS;
+  else d.epilogue = fuse_relu ? EPI_RELU : EPI_NONE;
+  return launch_gemm(e->stream, d);
+}
+
+int rst_linear_backward(rst_engine* e, const double* grad, const double* x, const double* weight,
+                        double* grad_weight, double* grad_bias, double* grad_input,
+                        const double* relu_mask_source, size_t batch, size_t in_features,
+                        size_t out_features) {
+  RST_TRY(engine_activate(e));
+  if (!grad || !x || !weight || !grad_weight)
+    return fail(RST_ERR_INVALID_ARGUMENT, "linear_backward: null operand");
+  RST_TRY(check_dim(batch, "batch"));
+  RST_TRY(check_dim(in_features, "in_features"));
+  RST_TRY(check_dim(out_features, "out_features"));
+  const double n = (double)batch;
+  {  // grad_weight[out,in] = (grad^T . x) / n
+    GemmDesc d{};
+    d.A = grad; d.B = x; d.C = grad_weight;
+    d.M = (int)out_features; d.N = (int)in_features; d.K = (int)batch;
+    d.lda = (long)out_features; d.ldb = (long)in_features; d.ldc = (long)in_features;
+    d.a_kc = false; d.b_kc = false;
+    d.epilogue = EPI_DIVIDE; d.divisor = n;
+    RST_TRY(launch_gemm(e->stream, d));
+  }
+  if (grad_bias) RST_TRY(launch_column_mean(e->stream, grad, grad_bias, batch, out_features, n));
+  if (grad_input) {  // grad_input[batch,in] = grad . weight
+    GemmDesc d{};
+    d.A = grad; d.B = weight; d.C = grad_input;
+    d.M = (int)batch; d.N = (int)in_features; d.K = (int)out_features;
+    d.lda = (long)out_features; d.ldb = (long)in_features; d.ldc = (long)in_features;
+    d.a_kc = true; d.b_kc = false;
+    d.epilogue = relu_mask_source ? EPI_MASK : EPI_NONE;
+    d.mask = relu_mask_source; d.ldmask = (long)in_features;
+    RST_TRY(launch_gemm(e->stream, d));
+  }
+  return RST_OK;
+}
+
+int rst_relu_forward(rst_engine* e, const double* x, double* out, size_t count) {
+  RST_TRY(engine_activate(e));
+  if (count && (!x || !out)) return fail(RST_ERR_INVALID_ARGUMENT, "relu_forward: null operand");
+  return launch_relu_forward(e->stream, x, out, count);
+}
+
+int rst_relu_backward(rst_engine* e, const double* grad, const double* x, double* out,
+                      size_t count) {
+  RST_TRY(engine_activate(e));
+  if (count && (!grad || !x || !out))
+    return fail(RST_ERR_INVALID_ARGUMENT, "relu_backward: null operand");
+  return launch_relu_backward(e->stream, grad, x, out, count);
+}
+
+int rst_softmax_rows(rst_engine* e, const double* x, double* out, size_t rows, size_t cols) {
+  RST_TRY(engine_activate(e));
+  if (rows == 0 || cols == 0) return RST_OK;
+  if (!x || !out) return fail(RST_ERR_INVALID_ARGUMENT, "softmax_rows: null operand");
+  hipLaunchKernelGGL(reset_flags_kernel, dim3(1), dim3(64), 0, e->stream, e->d_flags);
+  RST_HIP(hipGetLastError());
+  RST_TRY(launch_softmax_ce(e->stream, x, nullptr, nullptr, out, nullptr, e->d_flags, rows, cols));
+  RST_HIP(hipMemcpyAsync(e->h_flags, e->d_flags, sizeof(int), hipMemcpyDeviceToHost, e->stream));
+  RST_HIP(hipStreamSynchronize(e->stream));
+  if (e->h_flags[0] & 1)
+    return fail(RST_ERR_NAN, "softmax: NaN in the input (the reference panics in softmax.rs:38)");
+  return RST_OK;
+}
+
+int rst_cross_entropy(rst_engine* e, const double* pred, const double* truth, double* grad_out,
+                      double* prob_out, size_t rows, size_t cols, double* host_loss) {
+  RST_TRY(engine_activate(e));
+  if (!pred || !truth || !grad_out)
+    return fail(RST_ERR_INVALID_ARGUMENT, "cross_entropy: null operand");
+  return engine_cross_entropy(e, pred, truth, grad_out, prob_out, rows, cols, host_loss);
+}
+
+int rst_loss_value(rst_engine* e, double* host_loss) {
+  RST_TRY(engine_activate(e));
+  if (!host_loss) return fail(RST_ERR_INVALID_ARGUMENT, "host_loss is null");
+  if (!e->loss_valid) return fail(RST_ERR_STATE, "no loss has been computed on this engine");
+  RST_HIP(hipMemcpyAsync(e->h_loss, e->d_loss, sizeof(double), hipMemcpyDeviceToHost, e->stream));
+  RST_HIP(hipMemcpyAsync(e->h_flags, e->d_flags, sizeof(int), hipMemcpyDeviceToHost, e->stream));
+  RST_HIP(hipStreamSynchronize(e->stream));
+  *host_loss = *e->h_loss;
+  if (e->h_flags[0] & 1)
+    return fail(RST_ERR_NAN, "cross entropy: NaN logits (the reference panics in softmax.rs:38)");
+  return RST_OK;
+}
+
+int rst_sgd_step_flat(rst_engine* e, double* parm, const double* grad, size_t count, double lr) {
+  RST_TRY(engine_activate(e));
+  if (count && (!parm || !grad)) return fail(RST_ERR_INVALID_ARGUMENT, "sgd: null operand");
+  return launch_sgd_flat(e->stream, parm, grad, count, lr);
+}
+
+int rst_sgd_step(rst_engine* e, double* const* host_parm_ptrs, const double* const* host_grad_ptrs,
+                 const size_t* host_counts, size_t tensor_count, double lr) {
+  RST_TRY(engine_activate(e));
+  if (tensor_count == 0) return RST_OK;
+  if (!host_parm_ptrs || !host_grad_ptrs || !host_counts)
+    return fail(RST_ERR_INVALID_ARGUMENT, "sgd: null table");
+  std::vector<SgdTensor> table;
+  table.reserve(tensor_count);
+  unsigned long long blocks = 0;
+  for (size_t i = 0; i < tensor_count; ++i) {
+    if (host_counts[i] == 0) continue;
+    if (!host_parm_ptrs[i] || !host_grad_ptrs[i])
+      return fail(RST_ERR_INVALID_ARGUMENT, "sgd: tensor %zu has a null pointer", i);
+    SgdTensor t;
+    t.parm = host_parm_ptrs[i];
+    t.grad = host_grad_ptrs[i];
+    t.count = host_counts[i];
+    t.first_block = blocks;
+    blocks += sgd_blocks_for(t.count);
+    table.push_back(t);
+  }
+  if (table.empty()) return RST_OK;
+  const bool same = table.size() == e->sgd_table_host.size() &&
+                    std::memcmp(table.data(), e->sgd_table_host.data(),
+                                table.size() * sizeof(SgdTensor)) == 0;
+  if (!same) {
+    // an earlier launch may still be reading the device table
+    RST_HIP(hipStreamSynchronize(e->stream));
+    if (table.size() > e->sgd_table_capacity) {
+      if (e->d_sgd_table) RST_HIP(hipFree(e->d_sgd_table));
+      e->d_sgd_table = nullptr;
+      e->sgd_table_capacity = 0;
+      size_t cap = table.size() < 64 ? 64 : table.size() * 2;
+      RST_HIP(hipMalloc(&e->d_sgd_table, cap * sizeof(SgdTensor)));
+      e->sgd_table_capacity = cap;
+    }
+    RST_HIP(hipMemcpy(e->d_sgd_table, table.data(), table.size() * sizeof(SgdTensor),
+                      hipMemcpyHostToDevice));
+    e->sgd_table_host = table;
+    e->sgd_total_blocks = blocks;
+  }
+  return launch_sgd_multi(e->stream, e->d_sgd_table, table.size(), blocks, lr);
+}
+
+int rst_accuracy(rst_engine* e, const double* pred, const double* truth, size_t rows, size_t cols,
+                 double* host_accuracy) {
+  RST_TRY(engine_activate(e));
+  if (!pred || !truth || !host_accuracy)
+    return fail(RST_ERR_INVALID_ARGUMENT, "accuracy: null operand");
+  RST_TRY(launch_accuracy(e->stream, pred, truth, rows, cols, e->d_hits));
+  RST_HIP(hipMemcpyAsync(e->h_hits, e->d_hits, sizeof(unsigned long long), hipMemcpyDeviceToHost,
+                         e->stream));
+  RST_HIP(hipStreamSynchronize(e->stream));
+  *host_accuracy = (double)(*e->h_hits) / (double)rows;
+  return RST_OK;
+}
+
+int rst_fill_uniform(rst_engine* e, double* dst, size_t count, uint64_t seed, uint64_t stream,
+                     double lo, double hi) {
+  RST_TRY(engine_activate(e));
+  if (count && !dst) return fail(RST_ERR_INVALID_ARGUMENT, "fill_uniform: null destination");
+  return launch_fill_uniform(e->stream, dst, count, seed, stream, lo, hi);
+}
+
+int rst_fill_normal(rst_engine* e, double* dst, size_t count, uint64_t seed, uint64_t stream,
+                    double mean, double std) {
+  RST_TRY(engine_activate(e));
+  if (count && !dst) return fail(RST_ERR_INVALID_ARGUMENT, "fill_normal: null destination");
+  return launch_fill_normal(e->stream, dst, count, seed, stream, mean, std);
+}
+
+int rst_fill_one_hot(rst_engine* e, double* dst, size_t rows, size_t cols, uint64_t seed,
+                     uint64_t stream) {
+  RST_TRY(engine_activate(e));
+  if (rows && cols && !dst) return fail(RST_ERR_INVALID_ARGUMENT, "fill_one_hot: null destination");
+  return launch_fill_one_hot(e->stream, dst, rows, cols, seed, stream);
+}
+
+}  // extern "C"

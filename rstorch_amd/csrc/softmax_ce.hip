@@ -1,0 +1,259 @@
+// Row softmax and the fused softmax + cross-entropy forward/gradient kernel.
+//
+// Arithmetic follows the reference literally (src/module/activation/softmax.rs:45-53,
+// src/loss/cross_entropy.rs:34-47): m = max of the row folded from the lowest finite double,
+// e = exp(z - m), s = sum e, p = e / s (a true division), loss term = truth * ln(p),
+// gradient = -(truth - p).  Where truth is exactly 0 the term is 0 unless p is 0 or NaN
+// (0 * -inf = NaN in the reference), so ln is only evaluated where truth is non-zero.
+//
+// A row is kept in registers between the three phases, so each logit and each truth value is
+// read once and each gradient written once: 24 bytes per logit.
+#include <cfloat>
+
+#include "common.h"
+
+namespace rst {
+namespace {
+
+typedef double v2d __attribute__((ext_vector_type(2)));
+
+struct MaxOp {
+  __device__ static double apply(double a, double b) { return a < b ? b : a; }
+};
+struct SumOp {
+  __device__ static double apply(double a, double b) { return a + b; }
+};
+
+// Reduction over the TPR consecutive threads that share a row.  Every thread of the group
+// receives the same bits.  `scratch` needs TPR/64 doubles per row group when TPR > 64.
+template <int TPR, class Op>
+__device__ __forceinline__ double group_reduce(double v, double* scratch) {
+  constexpr int W = TPR < 64 ? TPR : 64;
+#pragma unroll
+  for (int off = W / 2; off > 0; off >>= 1) v = Op::apply(v, __shfl_xor(v, off));
+  if (TPR > 64) {
+    constexpr int NW = TPR / 64;
+    const int wave = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+    __syncthreads();
+    double r = scratch[0];
+#pragma unroll 1
+    for (int w = 1; w < NW; ++w) r = Op::apply(r, scratch[w]);
+    v = r;
+  }
+  return v;
+}
+
+__device__ __forceinline__ double loss_term(double truth, double p) {
+  if (truth == 0.0) return p > 0.0 ? 0.0 : __builtin_nan("");
+  return truth * log(p);
+}
+
+// Register-resident rows: TPR threads per row, IPT vectors of VEC doubles per thread.
+template <int TPR, int IPT, int VEC, bool CE>
+__global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
+    const double* __restrict__ z, const double* __restrict__ truth, double* __restrict__ grad,
+    double* __restrict__ prob, double* __restrict__ row_loss, int* __restrict__ flags, size_t rows,
+    size_t cols) {
+  constexpr int BLOCK = TPR > 256 ? TPR : 256;
+  constexpr int RPB = BLOCK / TPR;
+  __shared__ double red[3][TPR > 64 ? TPR / 64 : 1];
+
+  const int sub = threadIdx.x % TPR;
+  const size_t row = (size_t)blockIdx.x * RPB + threadIdx.x / TPR;
+  const bool row_ok = row < rows;
+  const size_t base = row * cols;
+
+  double x[IPT][VEC];
+  bool saw_nan = false;
+  double mx = -DBL_MAX;
+#pragma unroll
+  for (int i = 0; i < IPT; ++i) {
+    const size_t c = (size_t)(sub + i * TPR) * VEC;
+    const bool ok = row_ok && c < cols;
+    if (VEC == 2) {
+      v2d v = {0.0, 0.0};
+      if (ok) v = __builtin_nontemporal_load(reinterpret_cast<const v2d*>(z + base + c));
+      x[i][0] = v.x;
+      x[i][VEC - 1] = v.y;
+    } else {
+      x[i][0] = ok ? z[base + c] : 0.0;
+    }
+    if (ok) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        saw_nan |= (x[i][e] != x[i][e]);
+        mx = MaxOp::apply(mx, x[i][e]);
+      }
+    }
+  }
+  mx = group_reduce<TPR, MaxOp>(mx, red[0]);
+
+  double s = 0.0;
+#pragma unroll
+  for (int i = 0; i < IPT; ++i) {
+    const size_t c = (size_t)(sub + i * TPR) * VEC;
+    const bool ok = row_ok && c < cols;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      double ev = ok ? exp(x[i][e] - mx) : 0.0;
+      x[i][e] = ev;
+      s += ev;
+    }
+  }
+  s = group_reduce<TPR, SumOp>(s, red[1]);
+
+  double lsum = 0.0;
+#pragma unroll
+  for (int i = 0; i < IPT; ++i) {
+    const size_t c = (size_t)(sub + i * TPR) * VEC;
+    const bool ok = row_ok && c < cols;
+    if (!ok) continue;
+    double p[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) p[e] = x[i][e] / s;
+    if (CE) {
+      double t[VEC];
+      if (VEC == 2) {
+        v2d tv = __builtin_nontemporal_load(reinterpret_cast<const v2d*>(truth + base + c));
+        t[0] = tv.x;
+        t[VEC - 1] = tv.y;
+      } else {
+        t[0] = truth[base + c];
+      }
+      double g[VEC];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        lsum += loss_term(t[e], p[e]);
+        g[e] = -(t[e] - p[e]);
+      }
+      if (VEC == 2) {
+        v2d gv = {g[0], g[VEC - 1]};
+        __builtin_nontemporal_store(gv, reinterpret_cast<v2d*>(grad + base + c));
+      } else {
+        grad[base + c] = g[0];
+      }
+    }
+    if (prob) {
+      if (VEC == 2) {
+        v2d pv = {p[0], p[VEC - 1]};
+        *reinterpret_cast<v2d*>(prob + base + c) = pv;
+      } else {
+        prob[base + c] = p[0];
+      }
+    }
+  }
+  if (CE) {
+    lsum = group_reduce<TPR, SumOp>(lsum, red[2]);
+    if (sub == 0 && row_ok) row_loss[row] = lsum;
+  }
+  if (saw_nan) atomicOr(flags, 1);
+}
+
+// Rows too long for registers: one 1024-thread workgroup per row, three passes over memory.
+template <bool CE>
+__global__ __launch_bounds__(1024) void softmax_long_rows_kernel(
+    const double* __restrict__ z, const double* __restrict__ truth, double* __restrict__ grad,
+    double* __restrict__ prob, double* __restrict__ row_loss, int* __restrict__ flags, size_t rows,
+    size_t cols) {
+  constexpr int TPR = 1024;
+  __shared__ double red[3][TPR / 64];
+  const size_t row = blockIdx.x;
+  const size_t base = row * cols;
+  (void)rows;
+  bool saw_nan = false;
+  double mx = -DBL_MAX;
+  for (size_t c = threadIdx.x; c < cols; c += TPR) {
+    double v = z[base + c];
+    saw_nan |= (v != v);
+    mx = MaxOp::apply(mx, v);
+  }
+  mx = group_reduce<TPR, MaxOp>(mx, red[0]);
+  double s = 0.0;
+  for (size_t c = threadIdx.x; c < cols; c += TPR) s += exp(z[base + c] - mx);
+  s = group_reduce<TPR, SumOp>(s, red[1]);
+  double lsum = 0.0;
+  for (size_t c = threadIdx.x; c < cols; c += TPR) {
+    double p = exp(z[base + c] - mx) / s;
+    if (CE) {
+      double t = truth[base + c];
+      lsum += loss_term(t, p);
+      grad[base + c] = -(t - p);
+    }
+    if (prob) prob[base + c] = p;
+  }
+  if (CE) {
+    lsum = group_reduce<TPR, SumOp>(lsum, red[2]);
+    if (threadIdx.x == 0) row_loss[row] = lsum;
+  }
+  if (saw_nan) atomicOr(flags, 1);
+}
+
+// loss = -(sum of the per-row sums) / rows, one workgroup, fixed order.
+__global__ __launch_bounds__(1024) void loss_reduce_kernel(const double* __restrict__ row_loss,
+                                                          double* __restrict__ loss, size_t rows) {
+  __shared__ double red[1024 / 64];
+  double s = 0.0;
+  for (size_t r = threadIdx.x; r < rows; r += 1024) s += row_loss[r];
+  s = group_reduce<1024, SumOp>(s, red);
+  if (threadIdx.x == 0) loss[0] = -s / (double)rows;
+}
+
+template <int TPR, int IPT, int VEC>
+int launch_rows(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
+                double* row_loss, int* flags, size_t rows, size_t cols, bool ce) {
+  constexpr int BLOCK = TPR > 256 ? TPR : 256;
+  constexpr int RPB = BLOCK / TPR;
+  size_t blocks = (rows + RPB - 1) / RPB;
+  if (blocks > 0x7fffffffull) return fail(RST_ERR_UNSUPPORTED, "too many rows for one launch");
+  if (ce)
+    hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, true>), dim3((unsigned)blocks),
+                       dim3(BLOCK), 0, s, z, t, grad, prob, row_loss, flags, rows, cols);
+  else
+    hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, false>), dim3((unsigned)blocks),
+                       dim3(BLOCK), 0, s, z, t, grad, prob, row_loss, flags, rows, cols);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+template <int VEC>
+int dispatch(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
+             double* row_loss, int* flags, size_t rows, size_t cols, bool ce) {
+  const size_t units = cols / VEC;  // vectors per row
+  if (units <= 16 * 2) return launch_rows<16, 2, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
+  if (units <= 64 * 4) return launch_rows<64, 4, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
+  if (units <= 256 * 4) return launch_rows<256, 4, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
+  if (units <= 1024 * 4) return launch_rows<1024, 4, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
+  if (units <= 1024 * 16) return launch_rows<1024, 16, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
+  if (rows > 0x7fffffffull) return fail(RST_ERR_UNSUPPORTED, "too many rows for one launch");
+  if (ce)
+    hipLaunchKernelGGL(softmax_long_rows_kernel<true>, dim3((unsigned)rows), dim3(1024), 0, s, z, t,
+                       grad, prob, row_loss, flags, rows, cols);
+  else
+    hipLaunchKernelGGL(softmax_long_rows_kernel<false>, dim3((unsigned)rows), dim3(1024), 0, s, z, t,
+                       grad, prob, row_loss, flags, rows, cols);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+}  // namespace
+
+int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* grad_out,
+                      double* prob_out, double* row_loss, int* flags, size_t rows, size_t cols) {
+  if (rows == 0 || cols == 0) return RST_OK;
+  const bool ce = grad_out != nullptr;
+  const bool vec = cols % 2 == 0 && aligned16(z) && (!ce || (aligned16(t) && aligned16(grad_out))) &&
+                   (!prob_out || aligned16(prob_out));
+  if (vec) return dispatch<2>(s, z, t, grad_out, prob_out, row_loss, flags, rows, cols, ce);
+  return dispatch<1>(s, z, t, grad_out, prob_out, row_loss, flags, rows, cols, ce);
+}
+
+int launch_loss_reduce(hipStream_t s, const double* row_loss, double* loss, size_t rows) {
+  hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(1024), 0, s, row_loss, loss, rows);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+}  // namespace rst

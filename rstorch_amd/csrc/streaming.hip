@@ -1,0 +1,279 @@
+// HBM-bound streaming kernels: ReLU forward/backward (unfused form), fill, the bias-gradient
+// column mean, SGD and row arg-max accuracy.  All of them move each byte exactly once with
+// 16-byte accesses where alignment allows.
+#include "common.h"
+
+namespace rst {
+namespace {
+
+typedef double v2d __attribute__((ext_vector_type(2)));
+constexpr int kBlock = 256;
+
+inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+inline unsigned grid_for(size_t work_items, size_t per_block) {
+  size_t blocks = (work_items + per_block - 1) / per_block;
+  if (blocks < 1) blocks = 1;
+  return (unsigned)blocks;
+}
+
+// ---- ReLU -----------------------------------------------------------------------------------
+// forward: out = max(x, 0); fmax returns the non-NaN operand, like f64::max in the reference.
+__global__ __launch_bounds__(kBlock) void relu_forward_v2(const v2d* __restrict__ x,
+                                                         v2d* __restrict__ out, size_t n2) {
+  size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n2) {
+    v2d v = __builtin_nontemporal_load(x + i);
+    v.x = fmax(v.x, 0.0);
+    v.y = fmax(v.y, 0.0);
+    out[i] = v;
+  }
+}
+__global__ __launch_bounds__(kBlock) void relu_forward_s(const double* __restrict__ x,
+                                                        double* __restrict__ out, size_t n) {
+  size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) out[i] = fmax(x[i], 0.0);
+}
+// backward: out = g * (x > 0 ? 1 : 0), a real multiply so that inf * 0 stays NaN.
+__global__ __launch_bounds__(kBlock) void relu_backward_v2(const v2d* __restrict__ g,
+                                                          const v2d* __restrict__ x,
+                                                          v2d* __restrict__ out, size_t n2) {
+  size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n2) {
+    v2d gv = __builtin_nontemporal_load(g + i);
+    v2d xv = __builtin_nontemporal_load(x + i);
+    v2d r;
+    r.x = gv.x * (xv.x > 0.0 ? 1.0 : 0.0);
+    r.y = gv.y * (xv.y > 0.0 ? 1.0 : 0.0);
+    out[i] = r;
+  }
+}
+__global__ __launch_bounds__(kBlock) void relu_backward_s(const double* __restrict__ g,
+                                                         const double* __restrict__ x,
+                                                         double* __restrict__ out, size_t n) {
+  size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) out[i] = g[i] * (x[i] > 0.0 ? 1.0 : 0.0);
+}
+
+// ---- fill -----------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void fill_kernel(double* __restrict__ dst, size_t n,
+                                                     double value) {
+  size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  size_t stride = (size_t)gridDim.x * kBlock;
+  for (; i < n; i += stride) dst[i] = value;
+}
+
+// ---- column mean (bias gradient) -----------------------------------------------------------
+// 256 threads = 16 row groups x 16 columns; a thread adds rows rg, rg+16, ... of its column in
+// order, the 16 partial sums are combined through LDS in a fixed order, then divided.
+__global__ __launch_bounds__(kBlock) void column_mean_kernel(const double* __restrict__ g,
+                                                            double* __restrict__ out, size_t rows,
+                                                            size_t cols, double divisor) {
+  __shared__ double part[16][17];
+  const int c = threadIdx.x & 15, rg = threadIdx.x >> 4;
+  const size_t col = (size_t)blockIdx.x * 16 + c;
+  double s = 0.0;
+  if (col < cols)
+    for (size_t r = rg; r < rows; r += 16) s += g[r * cols + col];
+  part[rg][c] = s;
+  __syncthreads();
+  if (rg == 0 && col < cols) {
+    double t = 0.0;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) t += part[k][c];
+    out[col] = t / divisor;
+  }
+}
+
+// ---- SGD --------------------------------------------------------------------------------------
+// parm = parm - (lr * grad): __dmul_rn / __dsub_rn keep the two roundings of the reference
+// (no contraction into an FMA).  Streaming loads and stores bypass temporal caching.
+__device__ __forceinline__ v2d sgd_update(v2d w, v2d g, double lr) {
+  v2d r;
+  r.x = __dsub_rn(w.x, __dmul_rn(lr, g.x));
+  r.y = __dsub_rn(w.y, __dmul_rn(lr, g.y));
+  return r;
+}
+
+__global__ __launch_bounds__(kBlock) void sgd_flat_v2(v2d* __restrict__ w,
+                                                     const v2d* __restrict__ g, size_t n2,
+                                                     double lr) {
+  size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n2) {
+    v2d wv = __builtin_nontemporal_load(w + i);
+    v2d gv = __builtin_nontemporal_load(g + i);
+    __builtin_nontemporal_store(sgd_update(wv, gv, lr), w + i);
+  }
+}
+__global__ __launch_bounds__(kBlock) void sgd_flat_s(double* __restrict__ w,
+                                                    const double* __restrict__ g, size_t n,
+                                                    double lr) {
+  size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  if (i < n) w[i] = __dsub_rn(w[i], __dmul_rn(lr, g[i]));
+}
+
+constexpr unsigned long long kSgdPerBlock = 2ull * kBlock;  // doubles per workgroup
+
+// One launch over many tensors: the workgroup finds its tensor by bisection over the block
+// prefix in the descriptor table (uniform per workgroup, scalar loads).
+__global__ __launch_bounds__(kBlock) void sgd_multi_kernel(const SgdTensor* __restrict__ table,
+                                                          int n_tensors, double lr) {
+  const unsigned long long b = blockIdx.x;
+  int lo = 0, hi = n_tensors - 1;
+  while (lo < hi) {
+    int mid = (lo + hi + 1) >> 1;
+    if (table[mid].first_block <= b) lo = mid; else hi = mid - 1;
+  }
+  const SgdTensor t = table[lo];
+  const unsigned long long first = (b - t.first_block) * kSgdPerBlock + 2ull * threadIdx.x;
+  if (first >= t.count) return;
+  double* w = t.parm + first;
+  const double* g = t.grad + first;
+  const bool pair = first + 1 < t.count;
+  if (pair && ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(g)) % 16 == 0)) {
+    v2d wv = __builtin_nontemporal_load(reinterpret_cast<v2d*>(w));
+    v2d gv = __builtin_nontemporal_load(reinterpret_cast<const v2d*>(g));
+    __builtin_nontemporal_store(sgd_update(wv, gv, lr), reinterpret_cast<v2d*>(w));
+  } else {
+    w[0] = __dsub_rn(w[0], __dmul_rn(lr, g[0]));
+    if (pair) w[1] = __dsub_rn(w[1], __dmul_rn(lr, g[1]));
+  }
+}
+
+// ---- accuracy -----------------------------------------------------------------------------------
+// One wavefront per row: every lane scans a strided part keeping its first maximum, then the
+// lanes are combined preferring the larger value and, on ties, the smaller column - which is
+// the reference's "first maximum wins" (strict > replacement).  NaN never replaces.
+__device__ __forceinline__ void argmax_combine(double& v, unsigned& idx, double ov, unsigned oidx) {
+  if (oidx != 0xffffffffu && (idx == 0xffffffffu || ov > v || (ov == v && oidx < idx))) {
+    v = ov;
+    idx = oidx;
+  }
+}
+
+__device__ __forceinline__ unsigned row_argmax(const double* __restrict__ row, size_t cols,
+                                               int lane) {
+  // the reference starts from element 0 and replaces only when e > acc
+  double v = 0.0;
+  unsigned idx = 0xffffffffu;
+  for (size_t c = lane; c < cols; c += 64) {
+    double x = row[c];
+    // a NaN never wins a strict comparison, so it only counts when it is element 0 (the
+    // reference's initial accumulator), where it also can never be replaced
+    if (x != x && c != 0) continue;
+    if (idx == 0xffffffffu) { v = x; idx = (unsigned)c; }
+    else if (x > v) { v = x; idx = (unsigned)c; }
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    double ov = __shfl_xor(v, off);
+    unsigned oidx = __shfl_xor(idx, off);
+    argmax_combine(v, idx, ov, oidx);
+  }
+  return idx;
+}
+
+__global__ __launch_bounds__(kBlock) void accuracy_kernel(const double* __restrict__ pred,
+                                                         const double* __restrict__ truth,
+                                                         size_t rows, size_t cols,
+                                                         unsigned long long* hits) {
+  const int lane = threadIdx.x & 63;
+  const size_t row = (size_t)blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  unsigned a = row_argmax(pred + row * cols, cols, lane);
+  unsigned b = row_argmax(truth + row * cols, cols, lane);
+  if (lane == 0 && a == b) atomicAdd(hits, 1ull);
+}
+
+__global__ void zero_hits_kernel(unsigned long long* hits) { hits[0] = 0ull; }
+
+}  // namespace
+
+int launch_relu_forward(hipStream_t s, const double* x, double* out, size_t n) {
+  if (n == 0) return RST_OK;
+  if (n % 2 == 0 && aligned16(x) && aligned16(out)) {
+    hipLaunchKernelGGL(relu_forward_v2, dim3(grid_for(n / 2, kBlock)), dim3(kBlock), 0, s,
+                       reinterpret_cast<const v2d*>(x), reinterpret_cast<v2d*>(out), n / 2);
+  } else {
+    hipLaunchKernelGGL(relu_forward_s, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s, x, out, n);
+  }
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+int launch_relu_backward(hipStream_t s, const double* g, const double* x, double* out, size_t n) {
+  if (n == 0) return RST_OK;
+  if (n % 2 == 0 && aligned16(g) && aligned16(x) && aligned16(out)) {
+    hipLaunchKernelGGL(relu_backward_v2, dim3(grid_for(n / 2, kBlock)), dim3(kBlock), 0, s,
+                       reinterpret_cast<const v2d*>(g), reinterpret_cast<const v2d*>(x),
+                       reinterpret_cast<v2d*>(out), n / 2);
+  } else {
+    hipLaunchKernelGGL(relu_backward_s, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s, g, x, out, n);
+  }
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+int launch_fill(hipStream_t s, double* dst, size_t n, double value) {
+  if (n == 0) return RST_OK;
+  size_t blocks = (n + kBlock - 1) / kBlock;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(fill_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, s, dst, n, value);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+int launch_column_mean(hipStream_t s, const double* g, double* out, size_t rows, size_t cols,
+                       double divisor) {
+  if (cols == 0) return RST_OK;
+  hipLaunchKernelGGL(column_mean_kernel, dim3(grid_for(cols, 16)), dim3(kBlock), 0, s, g, out, rows,
+                     cols, divisor);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+int launch_sgd_flat(hipStream_t s, double* parm, const double* grad, size_t n, double lr) {
+  if (n == 0) return RST_OK;
+  if (aligned16(parm) && aligned16(grad)) {
+    size_t n2 = n / 2;
+    if (n2) {
+      if ((n2 + kBlock - 1) / kBlock > 0x7fffffffull)
+        return fail(RST_ERR_UNSUPPORTED, "parameter range too large for one launch");
+      hipLaunchKernelGGL(sgd_flat_v2, dim3(grid_for(n2, kBlock)), dim3(kBlock), 0, s,
+                         reinterpret_cast<v2d*>(parm), reinterpret_cast<const v2d*>(grad), n2, lr);
+    }
+    if (n & 1)
+      hipLaunchKernelGGL(sgd_flat_s, dim3(1), dim3(kBlock), 0, s, parm + (n - 1), grad + (n - 1),
+                         (size_t)1, lr);
+  } else {
+    hipLaunchKernelGGL(sgd_flat_s, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s, parm, grad, n, lr);
+  }
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+unsigned long long sgd_blocks_for(unsigned long long count) {
+  return (count + kSgdPerBlock - 1) / kSgdPerBlock;
+}
+
+int launch_sgd_multi(hipStream_t s, const SgdTensor* device_table, size_t n_tensors,
+                     unsigned long long total_blocks, double lr) {
+  if (n_tensors == 0 || total_blocks == 0) return RST_OK;
+  if (total_blocks > 0x7fffffffull)
+    return fail(RST_ERR_UNSUPPORTED, "too many parameters for one launch");
+  hipLaunchKernelGGL(sgd_multi_kernel, dim3((unsigned)total_blocks), dim3(kBlock), 0, s,
+                     device_table, (int)n_tensors, lr);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+int launch_accuracy(hipStream_t s, const double* pred, const double* truth, size_t rows,
+                    size_t cols, unsigned long long* hits) {
+  hipLaunchKernelGGL(zero_hits_kernel, dim3(1), dim3(1), 0, s, hits);
+  if (rows && cols)
+    hipLaunchKernelGGL(accuracy_kernel, dim3(grid_for(rows, kBlock / 64)), dim3(kBlock), 0, s, pred,
+                       truth, rows, cols, hits);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+}  // namespace rst

@@ -1,0 +1,304 @@
+"""Host-side mirror of the reference's ``module`` package over the HIP backend.
+
+Same names, argument meaning and failure behaviour as
+``src/module/{mod,linear,sequential}.rs`` and ``src/module/activation/{relu,identity}.rs``:
+``forward`` / ``backward`` / ``parameters`` / ``train`` / ``eval``; caches are consumed by
+``backward`` (a second ``backward`` raises, where the reference panics on ``unwrap``);
+gradients are overwritten, never accumulated.  Arrays are device-resident ``Array2``.
+"""
+import ctypes
+
+from . import _ffi
+from .engine import Array2, as_array2, default_engine
+from .init import InitParameters, KaimingNormal
+
+
+class Parameter:
+    """src/module/mod.rs:16-19: a parameter and its gradient (device arrays)."""
+
+    def __init__(self, parm, grad):
+        self.parm = parm
+        self.grad = grad
+
+
+class Parameters:
+    """src/module/mod.rs:21-40."""
+
+    def __init__(self, parms=None):
+        self.parms = list(parms or [])
+
+    def add(self, parm, grad):
+        self.parms.append(Parameter(parm, grad))
+        return self
+
+    def iter(self):
+        return iter(self.parms)
+
+    def __iter__(self):
+        return iter(self.parms)
+
+    def __len__(self):
+        return len(self.parms)
+
+
+class Module:
+    """src/module/mod.rs:42-56."""
+
+    def forward(self, input):
+        raise NotImplementedError
+
+    def backward(self, gradient):
+        raise NotImplementedError
+
+    def parameters(self):
+        return Parameters()
+
+    def train(self):
+        pass
+
+    def eval(self):
+        pass
+
+
+class Identity(Module):
+    """src/module/activation/identity.rs:15-29."""
+
+    @classmethod
+    def new(cls):
+        return cls()
+
+    def forward(self, input):
+        return input
+
+    def backward(self, gradient):
+        return gradient
+
+    def __repr__(self):
+        return "Identity"
+
+
+class ReLU(Module):
+    """src/module/activation/relu.rs:17-32."""
+
+    def __init__(self):
+        self.prev_input = None  # tensor whose sign gives the mask (pre-activation or output)
+
+    @classmethod
+    def new(cls):
+        return cls()
+
+    def forward(self, input):
+        x = as_array2(input)
+        out = x.engine.empty(x.rows, x.cols)
+        _ffi.check(x.engine.lib.rst_relu_forward(x.engine.handle, x.ptr, out.ptr, x.size))
+        self.prev_input = x
+        return out
+
+    def backward(self, gradient):
+        if self.prev_input is None:
+            raise _ffi.StateError(_ffi.RST_ERR_STATE, "ReLU.backward without a forward")
+        g = as_array2(gradient, self.prev_input.engine)
+        x, self.prev_input = self.prev_input, None  # take()
+        if g.shape != x.shape:
+            raise _ffi.ShapeError(_ffi.RST_ERR_SHAPE, "gradient %r vs input %r" % (g.shape, x.shape))
+        out = x.engine.empty(x.rows, x.cols)
+        _ffi.check(x.engine.lib.rst_relu_backward(x.engine.handle, g.ptr, x.ptr, out.ptr, x.size))
+        return out
+
+    # used by Sequential when the neighbouring Linear kernels do this layer's work
+    def _absorb_forward(self, activation):
+        self.prev_input = activation
+
+    def _absorb_backward(self):
+        if self.prev_input is None:
+            raise _ffi.StateError(_ffi.RST_ERR_STATE, "ReLU.backward without a forward")
+        self.prev_input = None
+
+    def __repr__(self):
+        return "ReLU"
+
+
+class Linear(Module):
+    """src/module/linear.rs:8-79.  weight (out, in), bias (1, out)."""
+
+    def __init__(self, input_size, output_size, init=None, engine=None):
+        init = init if init is not None else KaimingNormal()
+        eng = engine or default_engine()
+        self.engine = eng
+        self.input_size, self.output_size = int(input_size), int(output_size)
+        self.weight = as_array2(init.weight(self.input_size, self.output_size, eng), eng)
+        self.bias = as_array2(init.bias(self.input_size, self.output_size, eng), eng)
+        if self.weight.shape != (self.output_size, self.input_size):
+            raise _ffi.ShapeError(_ffi.RST_ERR_SHAPE, "init.weight returned %r" % (self.weight.shape,))
+        if self.bias.shape != (1, self.output_size):
+            raise _ffi.ShapeError(_ffi.RST_ERR_SHAPE, "init.bias returned %r" % (self.bias.shape,))
+        self.prev_input = None
+        self.grad_weight = None
+        self.grad_bias = None
+
+    @classmethod
+    def new(cls, input_size, output_size):
+        return cls(input_size, output_size)
+
+    @classmethod
+    def new_with_kernel(cls, input_size, output_size, init):
+        return cls(input_size, output_size, init)
+
+    def _forward(self, input, fuse_relu):
+        x = as_array2(input, self.engine)
+        if x.cols != self.input_size:
+            raise _ffi.ShapeError(_ffi.RST_ERR_SHAPE, "input has %d features, layer expects %d"
+                                  % (x.cols, self.input_size))
+        out = self.engine.empty(x.rows, self.output_size)
+        _ffi.check(self.engine.lib.rst_linear_forward(
+            self.engine.handle, x.ptr, self.weight.ptr, self.bias.ptr, out.ptr, x.rows,
+            self.input_size, self.output_size, 1 if fuse_relu else 0))
+        self.prev_input = x
+        return out
+
+    def forward(self, input):
+        return self._forward(input, False)
+
+    def _backward(self, gradient, mask_by_input, need_input_grad=True):
+        if self.prev_input is None:
+            raise _ffi.StateError(_ffi.RST_ERR_STATE, "Linear.backward without a forward")
+        g = as_array2(gradient, self.engine)
+        x, self.prev_input = self.prev_input, None  # take()
+        if g.shape != (x.rows, self.output_size):
+            raise _ffi.ShapeError(_ffi.RST_ERR_SHAPE, "gradient %r vs expected %r"
+                                  % (g.shape, (x.rows, self.output_size)))
+        if self.grad_weight is None:
+            self.grad_weight = self.engine.empty(self.output_size, self.input_size)
+            self.grad_bias = self.engine.empty(1, self.output_size)
+        gx = self.engine.empty(x.rows, self.input_size) if need_input_grad else None
+        _ffi.check(self.engine.lib.rst_linear_backward(
+            self.engine.handle, g.ptr, x.ptr, self.weight.ptr, self.grad_weight.ptr,
+            self.grad_bias.ptr, gx.ptr if gx is not None else None,
+            x.ptr if (mask_by_input and gx is not None) else None, x.rows, self.input_size,
+            self.output_size))
+        return gx
+
+    def backward(self, gradient):
+        return self._backward(gradient, False)
+
+    def parameters(self):
+        if self.grad_weight is None:
+            raise _ffi.StateError(_ffi.RST_ERR_STATE,
+                                  "Linear.parameters before any backward (no gradient yet)")
+        return Parameters().add(self.weight, self.grad_weight).add(self.bias, self.grad_bias)
+
+    def __repr__(self):
+        return "Linear(%d, %d)" % (self.input_size, self.output_size)
+
+
+class Sequential(Module):
+    """src/module/sequential.rs:11-110.  The layer list may change at any time; the
+    Linear/ReLU fusion is decided afresh on every call."""
+
+    def __init__(self, layers=None):
+        self.layers = list(layers or [])
+
+    @classmethod
+    def new(cls, layers):
+        return cls(layers)
+
+    def push(self, layer):
+        self.layers.append(layer)
+
+    push_box = push
+
+    def insert(self, index, layer):
+        self.layers.insert(index, layer)
+
+    insert_box = insert
+
+    def len(self):
+        return len(self.layers)
+
+    __len__ = len
+
+    def is_empty(self):
+        return not self.layers
+
+    def remove(self, index):
+        if index >= len(self.layers):
+            return None
+        return self.layers.pop(index)
+
+    def _next_real(self, i):
+        for j in range(i + 1, len(self.layers)):
+            if not isinstance(self.layers[j], Identity):
+                return j
+        return -1
+
+    def _prev_real(self, i):
+        for j in range(i - 1, -1, -1):
+            if not isinstance(self.layers[j], Identity):
+                return j
+        return -1
+
+    def forward(self, input):
+        x = input
+        skip = set()
+        for i, layer in enumerate(self.layers):
+            if i in skip:
+                continue
+            if type(layer) is Linear:
+                j = self._next_real(i)
+                if j >= 0 and type(self.layers[j]) is ReLU:
+                    x = layer._forward(x, True)
+                    self.layers[j]._absorb_forward(x)
+                    skip.add(j)
+                    continue
+            x = layer.forward(x)
+        return x
+
+    def backward(self, gradient):
+        g = gradient
+        skip = set()
+        for i in range(len(self.layers) - 1, -1, -1):
+            if i in skip:
+                continue
+            layer = self.layers[i]
+            if type(layer) is Linear:
+                j = self._prev_real(i)
+                if j >= 0 and type(self.layers[j]) is ReLU and \
+                        self.layers[j].prev_input is not None:
+                    g = layer._backward(g, True)
+                    self.layers[j]._absorb_backward()
+                    skip.add(j)
+                    continue
+            g = layer.backward(g)
+        return g
+
+    def train(self):
+        for layer in self.layers:
+            layer.train()
+
+    def eval(self):
+        for layer in self.layers:
+            layer.eval()
+
+    def parameters(self):
+        out = Parameters()
+        for layer in self.layers:
+            for p in layer.parameters():
+                out.parms.append(p)
+        return out
+
+    def __repr__(self):
+        return "Sequential(%s)" % ", ".join(repr(l) for l in self.layers)
+
+
+def sequential(*layers):
+    """The ``sequential!`` macro (src/module/sequential.rs:62-74): both spellings of the
+    reference are accepted - layer instances, or ``(LayerClass, arg, ...)`` tuples."""
+    built = []
+    for l in layers:
+        if isinstance(l, tuple):
+            built.append(l[0].new(*l[1:]))
+        elif isinstance(l, type):
+            built.append(l.new())
+        else:
+            built.append(l)
+    return Sequential.new(built)

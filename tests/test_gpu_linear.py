@@ -1,0 +1,133 @@
+"""Linear forward/backward on the GPU (through the C ABI) against the CPU oracle.
+
+Tolerance: max|got-want| / max|want| <= 1e-10 per tensor (the bound BASELINE.json states for
+logits and every dW/db); the contraction order differs from the oracle's, so results are not
+bit-identical."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-10
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")
+
+
+def _linear(rs, w, b):
+    return rs.Linear.new_with_kernel(w.shape[1], w.shape[0], rs.FromArrays(w, b))
+
+
+SHAPES = [
+    (1, 1, 1), (3, 2, 1), (2, 3, 10), (32, 784, 100), (32, 100, 100), (32, 100, 10),
+    (37, 101, 13), (5, 7, 3), (129, 17, 130), (64, 64, 64), (100, 300, 33),
+    (512, 256, 384), (1024, 128, 1000), (256, 1024, 1024), (2048, 100, 10),
+]
+
+
+@pytest.mark.parametrize("batch,k,n", SHAPES)
+@pytest.mark.parametrize("fuse_relu", [False, True])
+def test_forward_matches_oracle(engine, oracle, batch, k, n, fuse_relu):
+    import rstorch_amd as rs
+    rng = np.random.default_rng(batch * 1000003 + k * 1009 + n)
+    x = rng.standard_normal((batch, k))
+    w = rng.standard_normal((n, k)) / np.sqrt(k)
+    b = rng.standard_normal((1, n))
+    lin = _linear(rs, w, b)
+    got = lin._forward(x, fuse_relu).to_numpy()
+    want = oracle.linear_forward(x, w, b)
+    if fuse_relu:
+        want = oracle.relu_forward(want)
+    assert rel_err(got, want) <= TOL
+
+
+@pytest.mark.parametrize("batch,k,n", SHAPES)
+def test_backward_matches_oracle(engine, oracle, batch, k, n):
+    import rstorch_amd as rs
+    rng = np.random.default_rng(batch * 7919 + k * 31 + n)
+    x = rng.standard_normal((batch, k))
+    w = rng.standard_normal((n, k)) / np.sqrt(k)
+    b = rng.standard_normal((1, n))
+    g = rng.standard_normal((batch, n))
+    lin = _linear(rs, w, b)
+    lin.forward(x)
+    gx = lin.backward(g).to_numpy()
+    want_gw, want_gb, want_gx = oracle.linear_backward(g, x, w)
+    params = list(lin.parameters())
+    assert params[0].grad.shape == w.shape and params[1].grad.shape == b.shape
+    assert rel_err(params[0].grad.to_numpy(), want_gw) <= TOL
+    assert rel_err(params[1].grad.to_numpy(), want_gb) <= TOL
+    assert rel_err(gx, want_gx) <= TOL
+
+
+@pytest.mark.parametrize("batch,k,n", [(32, 100, 10), (130, 66, 34), (512, 256, 128)])
+def test_backward_with_fused_relu_mask(engine, oracle, batch, k, n):
+    """grad_input * (input > 0) in the epilogue == Linear.backward then ReLU.backward."""
+    import rstorch_amd as rs
+    rng = np.random.default_rng(5 + batch)
+    pre = rng.standard_normal((batch, k))
+    x = oracle.relu_forward(pre)  # the layer's input is a ReLU output
+    w = rng.standard_normal((n, k))
+    g = rng.standard_normal((batch, n))
+    lin = _linear(rs, w, np.zeros((1, n)))
+    lin.forward(x)
+    got = lin._backward(g, True).to_numpy()
+    _, _, gx = oracle.linear_backward(g, x, w)
+    want = oracle.relu_backward(gx, pre)
+    assert rel_err(got, want) <= TOL
+    assert np.all(got[pre <= 0] == 0.0)
+
+
+def test_reference_known_answers(engine):
+    """The reference's own Linear tests (src/module/linear.rs:97-131), exact small integers."""
+    import rstorch_amd as rs
+    kats = json.load(open(GOLDEN))
+    f = kats["linear_forward"]
+    lin = _linear(rs, np.array(f["weight"]), np.array(f["bias"]))
+    np.testing.assert_array_equal(lin.forward(np.array(f["input"])).to_numpy(), np.array(f["output"]))
+    b = kats["linear_backward"]
+    lin = _linear(rs, np.array(b["weight"]), np.array(b["bias"]))
+    lin.forward(np.array(b["input"]))
+    gx = lin.backward(np.array(b["gradient"])).to_numpy()
+    p = list(lin.parameters())
+    np.testing.assert_array_equal(p[0].grad.to_numpy(), np.array(b["grad_weight"]))
+    np.testing.assert_array_equal(p[1].grad.to_numpy(), np.array(b["grad_bias"]))
+    np.testing.assert_array_equal(gx, np.array(b["grad_input"]))
+    assert p[0].grad.shape == p[0].parm.shape and p[1].grad.shape == p[1].parm.shape
+
+
+def test_identity_weight_copies_input(engine):
+    """W = I reduces the contraction to a copy: bit-exact."""
+    import rstorch_amd as rs
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((70, 48))
+    lin = _linear(rs, np.eye(48), np.zeros((1, 48)))
+    np.testing.assert_array_equal(lin.forward(x).to_numpy(), x)
+
+
+def test_one_hot_input_selects_weight_rows(engine):
+    """One-hot rows select columns of W (exact), and dW = G^T X / n scatters G rows (exact
+    for a power-of-two batch)."""
+    import rstorch_amd as rs
+    rng = np.random.default_rng(4)
+    k, n, batch = 24, 19, 16
+    idx = rng.integers(0, k, size=batch)
+    x = np.zeros((batch, k)); x[np.arange(batch), idx] = 1.0
+    w = rng.standard_normal((n, k)); b = rng.standard_normal((1, n))
+    lin = _linear(rs, w, b)
+    np.testing.assert_array_equal(lin.forward(x).to_numpy(), w[:, idx].T + b)
+
+
+def test_backward_twice_raises(engine):
+    import rstorch_amd as rs
+    lin = _linear(rs, np.ones((2, 3)), np.zeros((1, 2)))
+    with pytest.raises(rs.StateError):
+        lin.parameters()  # no gradient yet (reference: unwrap on None, linear.rs:72)
+    lin.forward(np.ones((4, 3)))
+    lin.backward(np.ones((4, 2)))
+    with pytest.raises(rs.StateError):
+        lin.backward(np.ones((4, 2)))  # cache consumed (linear.rs:61)
+    with pytest.raises(rs.ShapeError):
+        lin.forward(np.ones((4, 5)))
