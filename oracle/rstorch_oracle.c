@@ -57,7 +57,7 @@ static void* xmalloc(size_t bytes) {
  * sequential, accumulators held in registers as 4-wide vectors. */
 typedef double v4d __attribute__((vector_size(32), aligned(8)));
 
-__attribute__((target_clones("fma", "default")))
+__attribute__((target_clones("fma", "default"), optimize("fp-contract=fast")))
 static void micro_kernel(size_t kc, const double* restrict ap, const double* restrict bp,
                          double* restrict c, size_t ldc, size_t mr, size_t nr, int first) {
   const v4d zero = {0.0, 0.0, 0.0, 0.0};

@@ -20,6 +20,8 @@ SOURCES = ["engine.hip", "gemm_f64.hip", "streaming.hip", "softmax_ce.hip", "rng
 
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    # a*b+c stays two roundings, as in the reference's element-wise ndarray expressions
+    "-ffp-contract=off",
     # packed FP32 instructions are not to be generated on this hardware pool
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function",

@@ -86,12 +86,20 @@ __global__ __launch_bounds__(kBlock) void column_mean_kernel(const double* __res
 }
 
 // ---- SGD --------------------------------------------------------------------------------------
-// parm = parm - (lr * grad): __dmul_rn / __dsub_rn keep the two roundings of the reference
-// (no contraction into an FMA).  Streaming loads and stores bypass temporal caching.
+// parm = parm - (lr * grad) with the two roundings of the reference: the product is rounded to
+// f64, then the difference.  Contraction into a fused multiply-add is switched off here (and for
+// the whole library on the compiler command line; the __dmul_rn intrinsic is a plain multiply
+// that the compiler would be free to fuse).  Streaming loads and stores bypass temporal caching.
+__device__ __forceinline__ double sgd_scalar(double w, double g, double lr) {
+#pragma clang fp contract(off)
+  const double step = lr * g;
+  return w - step;
+}
+
 __device__ __forceinline__ v2d sgd_update(v2d w, v2d g, double lr) {
   v2d r;
-  r.x = __dsub_rn(w.x, __dmul_rn(lr, g.x));
-  r.y = __dsub_rn(w.y, __dmul_rn(lr, g.y));
+  r.x = sgd_scalar(w.x, g.x, lr);
+  r.y = sgd_scalar(w.y, g.y, lr);
   return r;
 }
 
@@ -109,7 +117,7 @@ __global__ __launch_bounds__(kBlock) void sgd_flat_s(double* __restrict__ w,
                                                     const double* __restrict__ g, size_t n,
                                                     double lr) {
   size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
-  if (i < n) w[i] = __dsub_rn(w[i], __dmul_rn(lr, g[i]));
+  if (i < n) w[i] = sgd_scalar(w[i], g[i], lr);
 }
 
 constexpr unsigned long long kSgdPerBlock = 2ull * kBlock;  // doubles per workgroup
@@ -135,8 +143,8 @@ __global__ __launch_bounds__(kBlock) void sgd_multi_kernel(const SgdTensor* __re
     v2d gv = __builtin_nontemporal_load(reinterpret_cast<const v2d*>(g));
     __builtin_nontemporal_store(sgd_update(wv, gv, lr), reinterpret_cast<v2d*>(w));
   } else {
-    w[0] = __dsub_rn(w[0], __dmul_rn(lr, g[0]));
-    if (pair) w[1] = __dsub_rn(w[1], __dmul_rn(lr, g[1]));
+    w[0] = sgd_scalar(w[0], g[0], lr);
+    if (pair) w[1] = sgd_scalar(w[1], g[1], lr);
   }
 }
 

@@ -1,0 +1,198 @@
+"""ReLU, Identity, softmax and CrossEntropyLoss on the GPU against the oracle, the reference's
+known answers and closed forms.  ReLU/Identity are selections: bit-exact.  softmax / loss:
+max|got-want|/max|want| <= 1e-10 (exp/ln are the device library's, the oracle's are glibc's)."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+
+from conftest import rel_err
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-10
+KATS = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_kats.json")))
+
+
+def _softmax(engine, x):
+    import ctypes
+    from rstorch_amd import _ffi
+    a = engine.from_numpy(x)
+    out = engine.empty(a.rows, a.cols)
+    _ffi.check(engine.lib.rst_softmax_rows(engine.handle, a.ptr, out.ptr, a.rows, a.cols))
+    return out.to_numpy()
+
+
+# ---- ReLU / Identity --------------------------------------------------------------------------
+def test_relu_reference_known_answers(engine):
+    import rstorch_amd as rs
+    k = KATS["relu"]
+    m = rs.ReLU.new()
+    np.testing.assert_array_equal(m.forward(np.array(k["input"])).to_numpy(), np.array(k["forward"]))
+    np.testing.assert_array_equal(m.backward(np.array(k["gradient"])).to_numpy(), np.array(k["backward"]))
+    with pytest.raises(rs.StateError):
+        m.backward(np.array(k["gradient"]))  # cache consumed (relu.rs:26)
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (32, 100), (257, 129), (1024, 4096)])
+def test_relu_bit_exact(engine, oracle, shape):
+    import rstorch_amd as rs
+    rng = np.random.default_rng(shape[0] + shape[1])
+    x = rng.standard_normal(shape)
+    x[rng.random(shape) < 0.05] = 0.0
+    x.flat[0] = -0.0
+    g = rng.standard_normal(shape)
+    m = rs.ReLU.new()
+    np.testing.assert_array_equal(m.forward(x).to_numpy(), oracle.relu_forward(x))
+    np.testing.assert_array_equal(m.backward(g).to_numpy(), oracle.relu_backward(g, x))
+
+
+def test_relu_special_values(engine, oracle):
+    """NaN -> 0 forward (f64::max), mask false for NaN; inf gradient * 0 mask = NaN (a multiply)."""
+    import rstorch_amd as rs
+    x = np.array([[np.nan, -np.inf, np.inf, 0.0, -0.0, 1e-320, -1e-320, 2.0]])
+    g = np.array([[1.0, np.inf, np.inf, np.inf, 3.0, 4.0, 5.0, np.nan]])
+    m = rs.ReLU.new()
+    f = m.forward(x).to_numpy()
+    np.testing.assert_array_equal(f, oracle.relu_forward(x))
+    assert f[0, 0] == 0.0 and f[0, 2] == np.inf
+    b = m.backward(g).to_numpy()
+    np.testing.assert_array_equal(b, oracle.relu_backward(g, x))
+    assert np.isnan(b[0, 1]) and np.isnan(b[0, 3]) and b[0, 2] == np.inf
+
+
+def test_identity(engine):
+    import rstorch_amd as rs
+    x = np.array(KATS["identity"]["input"])
+    m = rs.Identity.new()
+    a = engine.from_numpy(x)
+    assert m.forward(a) is a and m.backward(a) is a
+    assert len(m.parameters()) == 0
+
+
+# ---- softmax ------------------------------------------------------------------------------------
+def test_softmax_reference_known_answer(engine):
+    k = KATS["softmax_axis1"]
+    p = _softmax(engine, np.array(k["input"]))
+    assert np.all(np.abs(p.sum(axis=1) - np.array(k["row_sums"])) <= k["row_sum_tolerance"])
+    assert p.sum() == k["total_exact"]  # the reference asserts exact equality (softmax.rs:92)
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1), (3, 2), (32, 10), (33, 11), (8, 64), (5, 100),
+                                       (17, 257), (64, 1000), (7, 1001), (4, 4096), (3, 8190),
+                                       (2, 32768), (2, 32770), (2, 40001)])
+def test_softmax_matches_oracle(engine, oracle, rows, cols):
+    rng = np.random.default_rng(rows * 65537 + cols)
+    x = rng.standard_normal((rows, cols)) * 3.0
+    got = _softmax(engine, x)
+    want = oracle.softmax(x)
+    assert rel_err(got, want) <= TOL
+    assert np.all(np.abs(got.sum(axis=1) - 1.0) <= 1e-12)
+
+
+def test_softmax_uniform_power_of_two_is_exact(engine):
+    for cols in (2, 16, 256, 4096):
+        p = _softmax(engine, np.full((3, cols), 0.37))
+        np.testing.assert_array_equal(p, np.full((3, cols), 1.0 / cols))
+
+
+def test_softmax_shift_invariance(engine):
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((9, 50))
+    np.testing.assert_array_equal(_softmax(engine, x + 64.0), _softmax(engine, (x + 64.0)))
+    # shifting by a power of two keeps x - max exact, so the result is bit-identical
+    np.testing.assert_array_equal(_softmax(engine, x), _softmax(engine, x + 0.0))
+    big = _softmax(engine, x * 1e3)  # huge logits do not overflow
+    assert np.all(np.isfinite(big)) and np.all(np.abs(big.sum(axis=1) - 1.0) <= 1e-12)
+
+
+def test_softmax_nan_is_an_error(engine):
+    import rstorch_amd as rs
+    x = np.zeros((4, 12)); x[2, 7] = np.nan
+    with pytest.raises(rs.NanError):
+        _softmax(engine, x)
+    # -inf is not NaN: partial_cmp succeeds and the maximum stays at the lowest finite double
+    y = np.zeros((2, 6)); y[0, 1] = -np.inf
+    p = _softmax(engine, y)
+    assert p[0, 1] == 0.0 and abs(p[0].sum() - 1.0) < 1e-15
+
+
+# ---- CrossEntropyLoss ---------------------------------------------------------------------------
+@pytest.mark.parametrize("rows,cols", [(1, 2), (32, 10), (33, 11), (64, 100), (128, 1000),
+                                       (16, 4096), (4, 32768), (3, 33000)])
+def test_cross_entropy_matches_oracle(engine, oracle, rows, cols):
+    import rstorch_amd as rs
+    rng = np.random.default_rng(rows + 17 * cols)
+    z = rng.standard_normal((rows, cols)) * 2.0
+    t = np.zeros((rows, cols)); t[np.arange(rows), rng.integers(0, cols, rows)] = 1.0
+    loss = rs.CrossEntropyLoss.new()
+    got = loss.forward(z, t)
+    want, prob = oracle.cross_entropy_forward(z, t)
+    assert abs(got - want) <= TOL * abs(want)
+    g = loss.backward().to_numpy()
+    assert rel_err(g, oracle.cross_entropy_backward(prob, t)) <= TOL
+    assert np.all(np.abs(g.sum(axis=1)) <= 1e-12)  # rows of prob - one_hot sum to 0
+    with pytest.raises(rs.StateError):
+        loss.backward()  # consumed (cross_entropy.rs:46)
+
+
+def test_cross_entropy_soft_labels(engine, oracle):
+    """truth need not be one-hot: every ln(prob) then contributes."""
+    import rstorch_amd as rs
+    rng = np.random.default_rng(21)
+    z = rng.standard_normal((19, 37))
+    t = rng.random((19, 37)); t /= t.sum(axis=1, keepdims=True)
+    loss = rs.CrossEntropyLoss.new()
+    got = loss.forward(z, t)
+    want, prob = oracle.cross_entropy_forward(z, t)
+    assert abs(got - want) <= TOL * abs(want)
+    assert rel_err(loss.backward().to_numpy(), prob - t) <= TOL
+
+
+def test_cross_entropy_closed_forms(engine):
+    import rstorch_amd as rs
+    rows, cols = 8, 64
+    t = np.zeros((rows, cols)); t[np.arange(rows), np.arange(rows)] = 1.0
+    # uniform logits: loss = ln C
+    got = rs.CrossEntropyLoss.new().forward(np.full((rows, cols), 1.25), t)
+    assert abs(got - math.log(cols)) <= 1e-14
+    # one-hot truth: loss = mean(logsumexp(z) - z[target])
+    rng = np.random.default_rng(2)
+    z = rng.standard_normal((rows, cols))
+    lse = np.log(np.exp(z - z.max(axis=1, keepdims=True)).sum(axis=1)) + z.max(axis=1)
+    want = np.mean(lse - z[np.arange(rows), np.arange(rows)])
+    got = rs.CrossEntropyLoss.new().forward(z, t)
+    assert abs(got - want) <= 1e-13 * abs(want)
+
+
+def test_cross_entropy_underflow_gives_nan_like_the_reference(engine, oracle):
+    """A probability that underflows to 0 where truth is 0 makes 0 * ln(0) = NaN in the reference
+    (cross_entropy.rs:38 takes ln of the probability); the kernel reproduces it."""
+    import rstorch_amd as rs
+    z = np.array([[0.0, -800.0, 1.0], [0.5, 0.25, 0.125]])
+    t = np.array([[1.0, 0.0, 0.0], [0.0, 1.0, 0.0]])
+    want, _ = oracle.cross_entropy_forward(z, t)
+    got = rs.CrossEntropyLoss.new().forward(z, t)
+    assert math.isnan(want) and math.isnan(got)
+
+
+def test_cross_entropy_nan_logits_is_an_error(engine):
+    import rstorch_amd as rs
+    z = np.zeros((4, 10)); z[1, 3] = np.nan
+    t = np.zeros((4, 10)); t[:, 0] = 1.0
+    with pytest.raises(rs.NanError):
+        rs.CrossEntropyLoss.new().forward(z, t)
+    with pytest.raises(rs.ShapeError):
+        rs.CrossEntropyLoss.new().forward(np.zeros((4, 10)), np.zeros((4, 9)))
+
+
+def test_accuracy_first_maximum_wins(engine, oracle):
+    import rstorch_amd as rs
+    rng = np.random.default_rng(8)
+    for rows, cols in [(32, 10), (100, 1000), (5, 70)]:
+        pred = rng.integers(0, 4, size=(rows, cols)).astype(np.float64)  # many ties
+        truth = np.zeros((rows, cols)); truth[np.arange(rows), rng.integers(0, cols, rows)] = 1.0
+        truth[0, :] = 0.0
+        truth[0, np.argmax(pred[0])] = 1.0
+        assert rs.accuracy(pred, truth) == oracle.accuracy(pred, truth)

@@ -1,0 +1,141 @@
+"""The fused device-resident step (rst_model_*) against the oracle, including the shapes of
+the benchmark configurations at sizes the oracle finishes in seconds."""
+import numpy as np
+import pytest
+
+from conftest import rel_err
+from test_gpu_sequential import README_MLP, batch_data, make_weights
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-10
+
+
+def pair(rs, oracle, spec, seed):
+    weights = make_weights(oracle, spec, seed)
+    dm = rs.DeviceModel(spec)
+    dm.load_parameters(weights)
+    ref = oracle.Model(spec)
+    for (p, _), w in zip(ref.parameters(), weights):
+        p[...] = w
+    return dm, ref
+
+
+CASES = [
+    ("C0_readme_b32", README_MLP, 32, False, 0.01),
+    ("C1_readme_b8192", README_MLP, 8192, False, 0.01),
+    ("C2_wide_reduced", [("linear", 1024, 4096), ("relu",), ("linear", 4096, 4096), ("relu",),
+                         ("linear", 4096, 1000)], 256, True, 0.01),
+    ("C4_deep_reduced", [("linear", 512, 512), ("relu",)] * 8 + [("linear", 512, 4096)], 128, True, 0.01),
+    ("ragged", [("identity",), ("linear", 33, 65), ("relu",), ("identity",), ("linear", 65, 129),
+                ("relu",), ("linear", 129, 7)], 67, True, 0.05),
+]
+
+
+@pytest.mark.parametrize("name,spec,batch,normal,lr", CASES, ids=[c[0] for c in CASES])
+def test_train_step_matches_oracle(engine, oracle, name, spec, batch, normal, lr):
+    import rstorch_amd as rs
+    dm, ref = pair(rs, oracle, spec, 0x5EED)
+    oracle.set_threads(8)
+    try:
+        n_in, n_out = dm.in_width, dm.out_width
+        x, y = batch_data(oracle, batch, n_in, n_out, 11, 0, normal)
+        # piecewise first, to compare logits / gradients
+        logits = dm.forward(x).to_numpy()
+        want_logits = ref.forward(x)
+        assert rel_err(logits, want_logits) <= TOL
+        got_loss = dm.loss(y)
+        want_loss, prob = oracle.cross_entropy_forward(want_logits, y)
+        assert abs(got_loss - want_loss) <= TOL * abs(want_loss)
+        gin = dm.backward(None, need_input_grad=True).to_numpy()
+        want_gin = ref.backward(oracle.cross_entropy_backward(prob, y))
+        assert rel_err(gin, want_gin) <= TOL
+        for (_, g), (_, rg) in zip(dm.parameters(), ref.parameters()):
+            assert g.shape == rg.shape and rel_err(g.to_numpy(), rg) <= TOL
+        dm.sgd_step(lr)
+        ref.sgd_step(lr)
+        for (p, _), (rp, _) in zip(dm.parameters(), ref.parameters()):
+            assert rel_err(p.to_numpy(), rp) <= TOL
+        # then the single-call step, twice
+        for step in (1, 2):
+            x, y = batch_data(oracle, batch, n_in, n_out, 11, step, normal)
+            got = dm.train_step(x, y, lr)
+            want = ref.train_step(x, y, lr)
+            assert abs(got - want) <= TOL * abs(want)
+        for (p, _), (rp, _) in zip(dm.parameters(), ref.parameters()):
+            assert rel_err(p.to_numpy(), rp) <= TOL
+    finally:
+        oracle.set_threads(1)
+
+
+def test_hundred_fused_steps(engine, oracle):
+    import rstorch_amd as rs
+    dm, ref = pair(rs, oracle, README_MLP, 5)
+    for step in range(100):
+        x, y = batch_data(oracle, 32, 784, 10, 13, step)
+        got = dm.train_step(x, y, 0.01)
+        want = ref.train_step(x, y, 0.01)
+        assert abs(got - want) <= 1e-8 * abs(want), "step %d" % step
+
+
+def test_basic_model_from_sequential(engine, oracle):
+    """BasicModel::step (src/model.rs:19-27) == the layer-by-layer README loop."""
+    import rstorch_amd as rs
+    spec = [("linear", 20, 30), ("relu",), ("linear", 30, 4)]
+    weights = make_weights(oracle, spec, 1)
+    def seq():
+        return rs.Sequential.new([rs.Linear.new_with_kernel(20, 30, rs.FromArrays(weights[0], weights[1])),
+                                  rs.ReLU.new(),
+                                  rs.Linear.new_with_kernel(30, 4, rs.FromArrays(weights[2], weights[3]))])
+    loop_model, loss, optim = seq(), rs.CrossEntropyLoss.new(), rs.SGD.new(0.1)
+    basic = rs.BasicModel.new(seq(), rs.CrossEntropyLoss.new(), rs.SGD.new(0.1))
+    for step in range(5):
+        x, y = batch_data(oracle, 16, 20, 4, 3, step, True)
+        l1 = loss.forward(loop_model.forward(x), y)
+        loop_model.backward(loss.backward())
+        optim.step(loop_model)
+        l2 = basic.step(x, y, want_loss=True)
+        assert l1 == l2  # same kernels, same order: bit-identical
+    for p, (q, _) in zip(loop_model.parameters(), basic.device.parameters()):
+        np.testing.assert_array_equal(p.parm.to_numpy(), q.to_numpy())
+    np.testing.assert_array_equal(basic.predict(x).to_numpy(), loop_model.forward(x).to_numpy())
+
+
+def test_state_machine_errors(engine):
+    """Misuse that panics in the reference returns RST_ERR_STATE / RST_ERR_SHAPE, never UB."""
+    import rstorch_amd as rs
+    dm = rs.DeviceModel([("linear", 4, 3)])
+    with pytest.raises(rs.StateError):
+        dm.sgd_step(0.1)                      # step before backward (linear.rs:72 unwrap)
+    with pytest.raises(rs.StateError):
+        dm.backward(None)                     # backward before forward
+    dm.forward(np.ones((2, 4)))
+    with pytest.raises(rs.StateError):
+        dm.backward(None)                     # loss gradient asked for before the loss
+    dm.loss(np.eye(3)[:2])
+    dm.backward(None)
+    with pytest.raises(rs.StateError):
+        dm.backward(None)                     # caches consumed
+    dm.sgd_step(0.1)
+    with pytest.raises(rs.ShapeError):
+        dm.forward(np.ones((2, 5)))
+    with pytest.raises(rs.ShapeError):
+        rs.DeviceModel([("linear", 4, 3), ("linear", 5, 2)])
+    z = np.zeros((2, 4)); z[0, 0] = np.nan
+    with pytest.raises(rs.NanError):
+        dm.train_step(z, np.eye(3)[:2], 0.1)
+
+
+def test_profile_records_cover_every_launch(engine, oracle):
+    import rstorch_amd as rs
+    dm, _ = pair(rs, oracle, README_MLP, 2)
+    dm.profile_enable(True)
+    x, y = batch_data(oracle, 32, 784, 10, 1, 0)
+    dm.train_step(x, y, 0.01)
+    recs = dm.profile_read()
+    kinds = [r["kernel"] for r in recs]
+    assert kinds.count("linear_forward") == 3 and kinds.count("grad_weight") == 3
+    assert kinds.count("grad_input") == 2      # the first layer's input gradient is skipped
+    assert kinds.count("cross_entropy") == 1 and kinds.count("sgd") == 1
+    assert "relu_forward" not in kinds and "relu_backward" not in kinds  # fused away
+    assert all(r["ms"] > 0 for r in recs)
+    dm.profile_enable(False)
