@@ -1,0 +1,255 @@
+#!/usr/bin/env python3
+"""Benchmark of the rstorch f64 training step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+
+Workload (BASELINE.json configs[4], the one the target sentence is quoted on): the deep MLP
+(Linear(4096,4096)+ReLU) x 8 -> Linear(4096,32768), f64, batch 1024, CrossEntropyLoss,
+SGD lr=0.01; weights N(0, 1/fan_in), inputs N(0,1), one-hot labels uniform over 32768 classes,
+all generated on the device by the counter-based generator.  One step = forward, loss,
+backward, SGD through the C ABI (rst_model_train_step), inputs resident in HBM.
+
+Prints ONE JSON line.  `roofline` is for the FP64-MFMA contraction kernel instantiation with the
+largest share of the step; per-launch durations come from HIP events recorded on the engine's
+stream around every launch of the timed steps.  `cpu_baseline` is the CPU restatement (oracle)
+timed on this host: a bounded sample of the same network at a reduced batch, extrapolated.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP64_MFMA_TFLOPS = 78.6
+PEAK_HBM_GBPS = 8000.0
+
+C4_SPEC = [("linear", 4096, 4096), ("relu",)] * 8 + [("linear", 4096, 32768)]
+C4_BATCH = 1024
+C2_SPEC = [("linear", 1024, 4096), ("relu",), ("linear", 4096, 4096), ("relu",),
+           ("linear", 4096, 1000)]
+C01_SPEC = [("identity",), ("linear", 784, 100), ("relu",), ("linear", 100, 100), ("relu",),
+            ("linear", 100, 10)]
+LR = 0.01
+SEED = 0x5EED
+
+
+def log(msg):
+    print(msg, file=sys.stderr, flush=True)
+
+
+def make_model(rs, eng, spec, batch, normal_inputs):
+    dm = rs.DeviceModel(spec, eng)
+    dm.init_kaiming(SEED, 0)
+    n_in, n_out = dm.in_width, dm.out_width
+    x = eng.normal(batch, n_in, SEED, 1000) if normal_inputs else eng.uniform(batch, n_in, SEED, 1000)
+    y = eng.one_hot(batch, n_out, SEED, 1001)
+    return dm, x, y
+
+
+def time_steps(eng, dm, x, y, steps, warmup, profile):
+    for _ in range(warmup):
+        dm.train_step(x, y, LR, want_loss=False)
+    eng.synchronize()
+    if profile:
+        dm.profile_enable(True)
+    ev0, ev1 = eng.event(), eng.event()
+    t0 = time.perf_counter()
+    ev0.record()
+    for _ in range(steps):
+        dm.train_step(x, y, LR, want_loss=False)
+    ev1.record()
+    eng.synchronize()
+    wall = time.perf_counter() - t0
+    dev_ms = ev0.elapsed_ms(ev1)
+    loss = dm.last_loss()
+    recs = dm.profile_read() if profile else []
+    if profile:
+        dm.profile_enable(False)
+    return wall, dev_ms, loss, recs
+
+
+def summarise(recs, steps):
+    """Per kernel class: launches per step, mean launch ms, achieved rate vs its roof."""
+    groups = {}
+    for r in recs:
+        g = groups.setdefault(r["kernel"], {"ms": 0.0, "flops": 0.0, "bytes": 0.0, "n": 0})
+        g["ms"] += r["ms"]; g["flops"] += r["flops"]; g["bytes"] += r["bytes"]; g["n"] += 1
+    out = {}
+    for k, g in groups.items():
+        e = {"launches_per_step": g["n"] / steps, "avg_launch_ms": g["ms"] / g["n"],
+             "ms_per_step": g["ms"] / steps}
+        if g["flops"] > 0:
+            e["bound"] = "mfma"
+            e["achieved_tflops"] = g["flops"] / (g["ms"] * 1e-3) / 1e12
+            e["frac"] = e["achieved_tflops"] / PEAK_FP64_MFMA_TFLOPS
+        else:
+            e["bound"] = "hbm"
+            e["achieved_gbps"] = g["bytes"] / (g["ms"] * 1e-3) / 1e9
+            e["frac"] = e["achieved_gbps"] / PEAK_HBM_GBPS
+        out[k] = e
+    return out
+
+
+def bench_sgd_c3(rs, eng, iters=20):
+    """configs[3]: SGD::step alone over 64 x (Linear(2048,2048) weight + bias), ~268.6M params."""
+    import ctypes
+    from rstorch_amd import _ffi
+    shapes = [(2048, 2048), (1, 2048)] * 64
+    total = sum(r * c for r, c in shapes)
+    parm = eng.normal(1, total, SEED, 2000, 0.0, 0.02)
+    grad = eng.normal(1, total, SEED, 2001, 0.0, 1e-3)
+    res = {"parameters": total, "bytes_per_step": 24 * total}
+    # (a) one launch over the 128 tensors (descriptor table)
+    n = len(shapes)
+    offs, o = [], 0
+    for r, c in shapes:
+        offs.append(o); o += r * c
+    pp = (ctypes.c_void_p * n)(*[parm.ptr + 8 * f for f in offs])
+    gp = (ctypes.c_void_p * n)(*[grad.ptr + 8 * f for f in offs])
+    cnt = (ctypes.c_size_t * n)(*[r * c for r, c in shapes])
+    for name, call in (
+            ("tensor_list", lambda: _ffi.check(eng.lib.rst_sgd_step(eng.handle, pp, gp, cnt, n, LR))),
+            ("arena", lambda: _ffi.check(eng.lib.rst_sgd_step_flat(eng.handle, parm.ptr, grad.ptr, total, LR)))):
+        for _ in range(3):
+            call()
+        eng.synchronize()
+        ev0, ev1 = eng.event(), eng.event()
+        ev0.record()
+        for _ in range(iters):
+            call()
+        ev1.record()
+        ms = ev0.elapsed_ms(ev1) / iters
+        res[name] = {"ms_per_step": ms, "steps_per_s": 1e3 / ms,
+                     "achieved_gbps": 24.0 * total / (ms * 1e-3) / 1e9,
+                     "frac_of_hbm_peak": 24.0 * total / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS}
+    return res
+
+
+def bench_small(rs, eng, spec, batch, normal, steps, warmup):
+    dm, x, y = make_model(rs, eng, spec, batch, normal)
+    wall, dev_ms, loss, _ = time_steps(eng, dm, x, y, steps, warmup, False)
+    dm.close()
+    return {"batch": batch, "steps": steps, "ms_per_step": wall * 1e3 / steps,
+            "steps_per_s": steps / wall, "samples_per_s": steps / wall * batch, "final_loss": loss}
+
+
+def cpu_baseline(sample_batch=64):
+    """The oracle (CPU restatement of the reference) on the C4 network at batch `sample_batch`.
+    Contraction and loss time scale linearly with the batch, SGD does not, so
+    t(1024) = t_sgd + (1024 / sample_batch) * (t_step(sample_batch) - t_sgd)."""
+    import numpy as np
+    import oracle
+    oracle.build()
+    # the GPU box grants a share of the host's cores; OMP_NUM_THREADS carries it
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16")))
+    ref = oracle.Model(C4_SPEC)
+    for i, (p, _) in enumerate(ref.parameters()):
+        if p.shape[0] > 1:
+            a = np.sqrt(3.0 / p.shape[1])  # uniform with the variance of N(0, 1/fan_in)
+            p[...] = oracle.fill_uniform(p.shape, SEED, i, -a, a)
+    x = oracle.fill_normal((sample_batch, 4096), SEED, 1000)
+    y = oracle.fill_one_hot(sample_batch, 32768, SEED, 1001)
+    out = {}
+    for label, threads in (("single", 1), ("all", cores)):
+        oracle.set_threads(threads)
+        if label == "all":
+            ref.train_step(x, y, LR)  # warm the thread pool
+        t0 = time.perf_counter(); ref.train_step(x, y, LR); t_step = time.perf_counter() - t0
+        t0 = time.perf_counter(); ref.sgd_step(LR); t_sgd = time.perf_counter() - t0
+        scale = C4_BATCH / float(sample_batch)
+        t_full = t_sgd + scale * max(t_step - t_sgd, 0.0)
+        out[label] = {"threads": threads, "t_step_sample_s": t_step, "t_sgd_s": t_sgd,
+                      "t_full_step_s": t_full, "steps_per_s": 1.0 / t_full}
+    oracle.set_threads(1)
+    del ref
+    return out, sample_batch, cores
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this backend runs the training step on ONE GPU; --gpus %d is not "
+                 "supported (no collectives are part of this build)" % args.gpus)
+
+    import rstorch_amd as rs
+    eng = rs.default_engine()
+    info = eng.device_info()
+    log("device: %s, %d CUs" % (info["name"], info["compute_units"]))
+
+    dm, x, y = make_model(rs, eng, C4_SPEC, C4_BATCH, True)
+    tensors, params = dm.parameter_count()
+    wall, dev_ms, loss, recs = time_steps(eng, dm, x, y, args.steps, args.warmup, True)
+    ms_per_step = wall * 1e3 / args.steps
+    kernels = summarise(recs, args.steps)
+    dm.close()
+    log("C4: %.3f ms/step, loss %.6f" % (ms_per_step, loss))
+
+    gemm_kinds = [k for k in ("linear_forward", "grad_weight", "grad_input") if k in kernels]
+    dominant = max(gemm_kinds, key=lambda k: kernels[k]["ms_per_step"])
+    d = kernels[dominant]
+    launches = [r for r in recs if r["kernel"] == dominant]
+    flops_per_launch = sum(r["flops"] for r in launches) / len(launches)
+    roofline = {"kernel": "gemm_f64_mfma (" + dominant + ")", "bound": "mfma",
+                "achieved": d["achieved_tflops"], "peak": PEAK_FP64_MFMA_TFLOPS, "unit": "TFLOP/s",
+                "frac": d["frac"], "traffic": None,
+                "avg_launch_ms": d["avg_launch_ms"], "flops_per_launch": flops_per_launch}
+    gemm_ms = sum(kernels[k]["ms_per_step"] for k in gemm_kinds)
+    gemm_flops = sum(r["flops"] for r in recs if r["kernel"] in gemm_kinds) / args.steps
+    all_gemm = {"tflops": gemm_flops / (gemm_ms * 1e-3) / 1e12,
+                "frac": gemm_flops / (gemm_ms * 1e-3) / 1e12 / PEAK_FP64_MFMA_TFLOPS,
+                "flops_per_step": gemm_flops, "ms_per_step": gemm_ms,
+                "first_layer_input_gradient": "skipped (the README loop discards it)"}
+
+    result = {
+        "metric": "training_steps_per_s", "value": args.steps / wall, "unit": "steps/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f64",
+        "data": "synthetic",
+        "config": {"workload": "C4 deep MLP: (Linear(4096,4096)+ReLU)x8 -> Linear(4096,32768), "
+                               "batch 1024, CrossEntropyLoss, SGD lr=0.01 (BASELINE.json configs[4])",
+                   "batch": C4_BATCH, "parameters": params, "samples_per_s": args.steps / wall * C4_BATCH,
+                   "device": info["name"], "device_ms_per_step": dev_ms / args.steps,
+                   "final_loss": loss, "per_launch_events": True},
+        "roofline": roofline,
+        "contractions": all_gemm,
+        "kernels": kernels,
+    }
+
+    if not args.no_extra:
+        log("SGD alone (configs[3]) ...")
+        result["sgd_c3"] = bench_sgd_c3(rs, eng)
+        log("other configurations ...")
+        result["other_configs"] = {
+            "C0_readme_b32": bench_small(rs, eng, C01_SPEC, 32, False, 2000, 100),
+            "C1_readme_b8192": bench_small(rs, eng, C01_SPEC, 8192, False, 200, 20),
+            "C2_wide_b2048": bench_small(rs, eng, C2_SPEC, 2048, True, 20, 3),
+        }
+
+    if not args.no_cpu:
+        log("CPU baseline (oracle) ...")
+        cpu, sample_batch, cores = cpu_baseline()
+        result["cpu_baseline"] = {
+            "value": cpu["single"]["steps_per_s"], "unit": "steps/s", "cores": 1, "kind": "port",
+            "sample": "oracle (C restatement of the reference, single thread like the reference) on "
+                      "the same C4 network at batch %d: one full step timed, contraction+loss time "
+                      "scaled x%d to batch 1024, SGD time added unscaled" % (sample_batch, C4_BATCH // sample_batch),
+            "detail": cpu["single"],
+        }
+        result["cpu_baseline_all_cores"] = {
+            "value": cpu["all"]["steps_per_s"], "unit": "steps/s", "cores": cores, "kind": "port",
+            "sample": "same sample, OpenMP over the oracle's contraction blocks", "detail": cpu["all"],
+        }
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -178,8 +178,9 @@ int rst_model_sgd_step(rst_model* model, double lr);
 int rst_model_train_step(rst_model* model, const double* x, const double* truth, size_t batch,
                          double lr, double* host_loss);
 /* Per-launch timing of the model's kernels: when enabled every launch is bracketed by events
- * (this serialises nothing, the stream is already in order).  After a synchronising call,
- * rst_model_profile_read returns up to `capacity` records of the latest step. */
+ * on the engine's stream (this serialises nothing, the stream is already in order).  Records
+ * accumulate over calls (up to 65536) until rst_model_profile_read, which waits for the stream,
+ * copies up to `capacity` of them (host_records == NULL: only counts) and clears the list. */
 typedef struct rst_kernel_record {
   int kind;          /* RST_KERNEL_* */
   int layer;         /* layer index, -1 for loss / optimiser */

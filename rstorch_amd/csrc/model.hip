@@ -68,6 +68,7 @@ struct rst_model {
   bool grads_valid = false;
   // profiling
   bool profiling = false;
+  bool slot_open = false;
   std::vector<ProfileSlot> slots;
   std::vector<hipEvent_t> event_pool;
   size_t events_used = 0;
@@ -104,8 +105,11 @@ int reserve_activations(rst_model* m, size_t batch) {
 }
 
 // ---- profiling helpers --------------------------------------------------------------------
+constexpr size_t kMaxProfileSlots = 1u << 16;  // records kept between two reads
+
 int prof_begin(rst_model* m, int kind, int layer, double flops, double bytes) {
-  if (!m->profiling) return RST_OK;
+  m->slot_open = false;
+  if (!m->profiling || m->slots.size() >= kMaxProfileSlots) return RST_OK;
   while (m->event_pool.size() < m->events_used + 2) {
     hipEvent_t ev;
     RST_HIP(hipEventCreate(&ev));
@@ -117,11 +121,13 @@ int prof_begin(rst_model* m, int kind, int layer, double flops, double bytes) {
   s.stop = m->event_pool[m->events_used++];
   RST_HIP(hipEventRecord(s.start, m->engine->stream));
   m->slots.push_back(s);
+  m->slot_open = true;
   return RST_OK;
 }
 
 int prof_end(rst_model* m) {
-  if (!m->profiling) return RST_OK;
+  if (!m->slot_open) return RST_OK;
+  m->slot_open = false;
   RST_HIP(hipEventRecord(m->slots.back().stop, m->engine->stream));
   return RST_OK;
 }
@@ -428,7 +434,6 @@ int rst_model_forward(rst_model* m, const double* x, size_t batch, const double*
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
   RST_TRY(engine_activate(m->engine));
   if (!x && batch) return fail(RST_ERR_INVALID_ARGUMENT, "x is null");
-  prof_reset(m);
   RST_TRY(do_forward(m, x, batch));
   if (logits) *logits = m->logits;
   return RST_OK;
@@ -458,7 +463,6 @@ int rst_model_train_step(rst_model* m, const double* x, const double* truth, siz
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
   RST_TRY(engine_activate(m->engine));
   if ((!x || !truth) && batch) return fail(RST_ERR_INVALID_ARGUMENT, "x or truth is null");
-  prof_reset(m);
   RST_TRY(do_forward(m, x, batch));
   RST_TRY(do_loss(m, truth, nullptr));
   RST_TRY(do_backward(m, nullptr, 0, nullptr));
@@ -489,6 +493,7 @@ int rst_model_profile_read(rst_model* m, rst_kernel_record* host_records, size_t
     host_records[i].flops = m->slots[i].flops;
     host_records[i].bytes = m->slots[i].bytes;
   }
+  prof_reset(m);  // reading consumes the records; their events go back to the pool
   return RST_OK;
 }
 

@@ -161,8 +161,8 @@ class DeviceModel:
     def profile_enable(self, on=True):
         _ffi.check(self.engine.lib.rst_model_profile_enable(self.handle, 1 if on else 0))
 
-    def profile_read(self):
-        cap = 4 * len(self.spec) + 16
+    def profile_read(self, capacity=65536):
+        cap = int(capacity)
         recs = (_ffi.KernelRecord * cap)()
         n = ctypes.c_size_t()
         _ffi.check(self.engine.lib.rst_model_profile_read(self.handle, recs, cap, ctypes.byref(n)))
