@@ -35,63 +35,83 @@ struct GemmParams {
   double divisor;
   const double* mask;
   long ldmask;
-  int a_vec, b_vec;  // 16-byte global loads are legal for the operand
   int tiles_m, tiles_n;
 };
 
 // LDS geometry of one operand tile of EXT rows/cols by BK contraction steps.
-//   contraction-contiguous: [EXT][BK + 2]   (stride 18 doubles: fragment reads hit 32 distinct
-//                                            8-byte banks per half wave)
-//   output-contiguous:      [BK][EXT + 16]  (stride = 16 mod 32 doubles, same property)
+//   contraction-contiguous: [EXT][BK], element (e, k) at e*BK + (k ^ (e & 15)).  The XOR spreads
+//       the 16 rows that one MFMA fragment read touches over all sixteen 8-byte bank pairs, for
+//       any k, without padding; an aligned pair (k, k+1) stays inside one 16-byte slot.
+//   output-contiguous:      [BK][EXT + 16], element (e, k) at k*(EXT+16) + e.  A fragment read
+//       takes 16 consecutive doubles per k, and the stride is 16 mod 32 doubles so that two
+//       neighbouring k rows fall into different halves of the banks.
 template <int EXT, bool KC>
 struct TileGeom {
-  static constexpr int stride = KC ? (BK + 2) : (EXT + 16);
-  static constexpr int size = KC ? EXT * (BK + 2) : BK * (EXT + 16);
-  static constexpr int loads = EXT * BK / 2 / kThreads;  // v2d loads per thread per tile
+  static constexpr int stride = KC ? BK : (EXT + 16);
+  static constexpr int size = KC ? EXT * BK : BK * (EXT + 16);
+  static constexpr int loads = EXT * BK / 2 / kThreads;  // 16-byte loads per thread per tile
   static_assert(EXT * BK / 2 % kThreads == 0, "tile must split evenly over the block");
 };
 
-// Copy one operand tile global -> registers.  `ext0` is the first row/col of the tile along
-// the output dimension (limit `ext_n`), `k0` the first contraction index (limit `k_n`).
-template <int EXT, bool KC>
-__device__ __forceinline__ void load_tile(v2d* __restrict__ reg,
-                                          const double* __restrict__ base, long ld, int ext0,
-                                          int ext_n, int k0, int k_n, int vec, int tid) {
+// Copy one operand tile global -> registers without any divergent branch.
+//   `ext0`/`ext_n`: first row (or column) of the tile along the output dimension and its limit;
+//   rows beyond the limit are clamped onto the last valid ones - they only feed output rows or
+//   columns that are never stored.
+//   `k0`/`k_n`: first contraction index and its limit.  TAIL = false promises k0 + BK <= k_n;
+//   TAIL = true clamps the address and zeroes what lies beyond the limit (both operands do, so
+//   no stray NaN or infinity meets a zero).
+//   VEC = true promises 16-byte alignment of every pair (even leading dimension, even extent).
+template <int EXT, bool KC, bool VEC, bool TAIL>
+__device__ __forceinline__ void load_tile(v2d* __restrict__ reg, const double* __restrict__ base,
+                                          long ld, int ext0, int ext_n, int k0, int k_n, int tid) {
   constexpr int L = TileGeom<EXT, KC>::loads;
 #pragma unroll
   for (int u = 0; u < L; ++u) {
     const int q = tid + u * kThreads;
-    int e, k;        // element coordinates of the first of the two doubles
-    bool contiguous_is_k = KC;
+    int e, k;  // coordinates of the first of the two doubles
     if (KC) {
-      e = ext0 + (q >> 3);           // BK/2 = 8 pairs per row
+      e = ext0 + (q >> 3);  // BK/2 = 8 pairs per row
       k = k0 + 2 * (q & 7);
     } else {
       k = k0 + q / (EXT / 2);
       e = ext0 + 2 * (q % (EXT / 2));
     }
-    v2d v = {0.0, 0.0};
-    if (contiguous_is_k) {
-      if (e < ext_n) {
-        const double* p = base + (size_t)e * ld + k;
-        if (vec) {
-          if (k + 1 < k_n) v = *reinterpret_cast<const v2d*>(p);
-          else if (k < k_n) v.x = p[0];
-        } else {
-          if (k < k_n) v.x = p[0];
-          if (k + 1 < k_n) v.y = p[1];
-        }
+    v2d v;
+    if (KC) {
+      const int ec = e < ext_n ? e : ext_n - 1;
+      int ka = k, kb = k + 1;
+      if (TAIL) {
+        ka = ka < k_n ? ka : k_n - 1;
+        kb = kb < k_n ? kb : k_n - 1;
+      }
+      const double* row = base + (size_t)ec * ld;
+      if (VEC && !TAIL) {
+        v = *reinterpret_cast<const v2d*>(row + ka);
+      } else {
+        v.x = row[ka];
+        v.y = row[kb];
+      }
+      if (TAIL) {
+        v.x = k < k_n ? v.x : 0.0;
+        v.y = k + 1 < k_n ? v.y : 0.0;
       }
     } else {
-      if (k < k_n) {
-        const double* p = base + (size_t)k * ld + e;
-        if (vec) {
-          if (e + 1 < ext_n) v = *reinterpret_cast<const v2d*>(p);
-          else if (e < ext_n) v.x = p[0];
-        } else {
-          if (e < ext_n) v.x = p[0];
-          if (e + 1 < ext_n) v.y = p[1];
-        }
+      int kc = k;
+      if (TAIL) kc = kc < k_n ? kc : k_n - 1;
+      const double* row = base + (size_t)kc * ld;
+      if (VEC) {
+        const int ec = e + 1 < ext_n ? e : ext_n - 2;
+        v = *reinterpret_cast<const v2d*>(row + ec);
+      } else {
+        const int ea = e < ext_n ? e : ext_n - 1;
+        const int eb = e + 1 < ext_n ? e + 1 : ext_n - 1;
+        v.x = row[ea];
+        v.y = row[eb];
+      }
+      if (TAIL) {
+        const bool in = k < k_n;
+        v.x = in ? v.x : 0.0;
+        v.y = in ? v.y : 0.0;
       }
     }
     reg[u] = v;
@@ -107,10 +127,16 @@ __device__ __forceinline__ void store_tile(double* __restrict__ lds,
 #pragma unroll
   for (int u = 0; u < L; ++u) {
     const int q = tid + u * kThreads;
-    int off;
-    if (KC) off = (q >> 3) * S + 2 * (q & 7);
-    else off = (q / (EXT / 2)) * S + 2 * (q % (EXT / 2));
-    *reinterpret_cast<v2d*>(lds + off) = reg[u];
+    if (KC) {
+      const int e = q >> 3, k = 2 * (q & 7);
+      // slot of the pair: (k ^ (e & 14)); inside the slot the two doubles swap when e is odd
+      v2d v = reg[u];
+      if (e & 1) v = (v2d){v.y, v.x};
+      *reinterpret_cast<v2d*>(lds + e * S + (k ^ (e & 14))) = v;
+    } else {
+      const int off = (q / (EXT / 2)) * S + 2 * (q % (EXT / 2));
+      *reinterpret_cast<v2d*>(lds + off) = reg[u];
+    }
   }
 }
 
@@ -118,10 +144,10 @@ __device__ __forceinline__ void store_tile(double* __restrict__ lds,
 template <int EXT, bool KC>
 __device__ __forceinline__ double read_frag(const double* __restrict__ lds, int e, int k) {
   constexpr int S = TileGeom<EXT, KC>::stride;
-  return KC ? lds[e * S + k] : lds[k * S + e];
+  return KC ? lds[e * S + (k ^ (e & 15))] : lds[k * S + e];
 }
 
-template <int BM, int BN, bool A_KC, bool B_KC>
+template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
 __global__ __launch_bounds__(kThreads, 2) void gemm_f64_mfma(const GemmParams p) {
   using GA = TileGeom<BM, A_KC>;
   using GB = TileGeom<BN, B_KC>;
@@ -168,21 +194,31 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f64_mfma(const GemmParams p)
     for (int j = 0; j < TN; ++j) acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
 
   v2d ra[GA::loads], rb[GB::loads];
-  const int nk = (p.K + BK - 1) / BK;
+  const int nk_full = p.K / BK;                     // K steps that need no bounds handling
+  const int nk = nk_full + (p.K % BK != 0 ? 1 : 0);
 
-  load_tile<BM, A_KC>(ra, p.A, p.lda, m0, p.M, 0, p.K, p.a_vec, tid);
-  load_tile<BN, B_KC>(rb, p.B, p.ldb, n0, p.N, 0, p.K, p.b_vec, tid);
-  store_tile<BM, A_KC>(lds_a[0], ra, tid);
-  store_tile<BN, B_KC>(lds_b[0], rb, tid);
+  // Loads the operand tiles of K step `kt` into registers; only the last step can be partial.
+  auto fetch = [&](int kt) {
+    if (kt < nk_full) {
+      load_tile<BM, A_KC, VEC, false>(ra, p.A, p.lda, m0, p.M, kt * BK, p.K, tid);
+      load_tile<BN, B_KC, VEC, false>(rb, p.B, p.ldb, n0, p.N, kt * BK, p.K, tid);
+    } else {
+      load_tile<BM, A_KC, VEC, true>(ra, p.A, p.lda, m0, p.M, kt * BK, p.K, tid);
+      load_tile<BN, B_KC, VEC, true>(rb, p.B, p.ldb, n0, p.N, kt * BK, p.K, tid);
+    }
+  };
+
+  if (nk > 0) {
+    fetch(0);
+    store_tile<BM, A_KC>(lds_a[0], ra, tid);
+    store_tile<BN, B_KC>(lds_b[0], rb, tid);
+  }
   __syncthreads();
 
   for (int kt = 0; kt < nk; ++kt) {
     const int cur = kt & 1;
     const bool more = kt + 1 < nk;
-    if (more) {
-      load_tile<BM, A_KC>(ra, p.A, p.lda, m0, p.M, (kt + 1) * BK, p.K, p.a_vec, tid);
-      load_tile<BN, B_KC>(rb, p.B, p.ldb, n0, p.N, (kt + 1) * BK, p.K, p.b_vec, tid);
-    }
+    if (more) fetch(kt + 1);  // in flight while this step is multiplied
     const double* __restrict__ sa = lds_a[cur];
     const double* __restrict__ sb = lds_b[cur];
 #pragma unroll
@@ -233,28 +269,28 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f64_mfma(const GemmParams p)
   }
 }
 
-template <int BM, int BN, bool A_KC, bool B_KC>
+template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
 int launch_one(hipStream_t stream, GemmParams p) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const long long blocks = (long long)p.tiles_m * p.tiles_n;
   if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
-  hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, A_KC, B_KC>), dim3((unsigned)blocks), dim3(kThreads), 0,
-                     stream, p);
+  hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, A_KC, B_KC, VEC>), dim3((unsigned)blocks),
+                     dim3(kThreads), 0, stream, p);
   RST_HIP(hipGetLastError());
   return RST_OK;
 }
 
-template <bool A_KC, bool B_KC>
+template <bool A_KC, bool B_KC, bool VEC>
 int launch_layout(hipStream_t stream, const GemmParams& p) {
   // Largest tile that still gives the 256 compute units about two workgroups each; small
   // problems fall through to smaller tiles for parallelism.
   auto tiles = [&](int bm, int bn) {
     return (long long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
   };
-  if (tiles(128, 128) >= 256) return launch_one<128, 128, A_KC, B_KC>(stream, p);
-  if (tiles(64, 64) >= 256) return launch_one<64, 64, A_KC, B_KC>(stream, p);
-  return launch_one<32, 32, A_KC, B_KC>(stream, p);
+  if (tiles(128, 128) >= 256) return launch_one<128, 128, A_KC, B_KC, VEC>(stream, p);
+  if (tiles(64, 64) >= 256) return launch_one<64, 64, A_KC, B_KC, VEC>(stream, p);
+  return launch_one<32, 32, A_KC, B_KC, VEC>(stream, p);
 }
 
 }  // namespace
@@ -271,13 +307,16 @@ int launch_gemm(hipStream_t stream, const GemmDesc& d) {
     return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && (ld % 2 == 0) &&
            (contiguous_extent % 2 == 0);
   };
-  p.a_vec = vec_ok(d.A, d.lda, d.a_kc ? d.K : d.M) ? 1 : 0;
-  p.b_vec = vec_ok(d.B, d.ldb, d.b_kc ? d.K : d.N) ? 1 : 0;
+  // 16-byte loads need both operands aligned with even leading dimensions and extents
+  const bool vec = vec_ok(d.A, d.lda, d.a_kc ? d.K : d.M) && vec_ok(d.B, d.ldb, d.b_kc ? d.K : d.N);
   p.tiles_m = p.tiles_n = 0;
-  if (d.a_kc && d.b_kc) return launch_layout<true, true>(stream, p);
-  if (!d.a_kc && !d.b_kc) return launch_layout<false, false>(stream, p);
-  if (d.a_kc && !d.b_kc) return launch_layout<true, false>(stream, p);
-  return launch_layout<false, true>(stream, p);
+  if (d.a_kc && d.b_kc)
+    return vec ? launch_layout<true, true, true>(stream, p) : launch_layout<true, true, false>(stream, p);
+  if (!d.a_kc && !d.b_kc)
+    return vec ? launch_layout<false, false, true>(stream, p) : launch_layout<false, false, false>(stream, p);
+  if (d.a_kc && !d.b_kc)
+    return vec ? launch_layout<true, false, true>(stream, p) : launch_layout<true, false, false>(stream, p);
+  return vec ? launch_layout<false, true, true>(stream, p) : launch_layout<false, true, false>(stream, p);
 }
 
 }  // namespace rst
