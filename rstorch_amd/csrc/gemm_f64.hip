@@ -21,7 +21,6 @@ namespace {
 typedef double v4d __attribute__((ext_vector_type(4)));
 typedef double v2d __attribute__((ext_vector_type(2)));
 
-constexpr int kThreads = 256;
 constexpr int BK = 16;
 
 struct GemmParams {
@@ -45,12 +44,12 @@ struct GemmParams {
 //   output-contiguous:      [BK][EXT + 16], element (e, k) at k*(EXT+16) + e.  A fragment read
 //       takes 16 consecutive doubles per k, and the stride is 16 mod 32 doubles so that two
 //       neighbouring k rows fall into different halves of the banks.
-template <int EXT, bool KC>
+template <int EXT, bool KC, int THREADS>
 struct TileGeom {
   static constexpr int stride = KC ? BK : (EXT + 16);
   static constexpr int size = KC ? EXT * BK : BK * (EXT + 16);
-  static constexpr int loads = EXT * BK / 2 / kThreads;  // 16-byte loads per thread per tile
-  static_assert(EXT * BK / 2 % kThreads == 0, "tile must split evenly over the block");
+  static constexpr int loads = EXT * BK / 2 / THREADS;  // 16-byte loads per thread per tile
+  static_assert(EXT * BK / 2 % THREADS == 0, "tile must split evenly over the block");
 };
 
 // Copy one operand tile global -> registers without any divergent branch.
@@ -61,13 +60,13 @@ struct TileGeom {
 //   TAIL = true clamps the address and zeroes what lies beyond the limit (both operands do, so
 //   no stray NaN or infinity meets a zero).
 //   VEC = true promises 16-byte alignment of every pair (even leading dimension, even extent).
-template <int EXT, bool KC, bool VEC, bool TAIL>
+template <int EXT, bool KC, bool VEC, bool TAIL, int THREADS>
 __device__ __forceinline__ void load_tile(v2d* __restrict__ reg, const double* __restrict__ base,
                                           long ld, int ext0, int ext_n, int k0, int k_n, int tid) {
-  constexpr int L = TileGeom<EXT, KC>::loads;
+  constexpr int L = TileGeom<EXT, KC, THREADS>::loads;
 #pragma unroll
   for (int u = 0; u < L; ++u) {
-    const int q = tid + u * kThreads;
+    const int q = tid + u * THREADS;
     int e, k;  // coordinates of the first of the two doubles
     if (KC) {
       e = ext0 + (q >> 3);  // BK/2 = 8 pairs per row
@@ -119,14 +118,14 @@ __device__ __forceinline__ void load_tile(v2d* __restrict__ reg, const double* _
 }
 
 // Registers -> LDS stage.
-template <int EXT, bool KC>
+template <int EXT, bool KC, int THREADS>
 __device__ __forceinline__ void store_tile(double* __restrict__ lds,
                                            const v2d* __restrict__ reg, int tid) {
-  constexpr int L = TileGeom<EXT, KC>::loads;
-  constexpr int S = TileGeom<EXT, KC>::stride;
+  constexpr int L = TileGeom<EXT, KC, THREADS>::loads;
+  constexpr int S = TileGeom<EXT, KC, THREADS>::stride;
 #pragma unroll
   for (int u = 0; u < L; ++u) {
-    const int q = tid + u * kThreads;
+    const int q = tid + u * THREADS;
     if (KC) {
       const int e = q >> 3, k = 2 * (q & 7);
       // slot of the pair: (k ^ (e & 14)); inside the slot the two doubles swap when e is odd
@@ -143,15 +142,17 @@ __device__ __forceinline__ void store_tile(double* __restrict__ lds,
 // LDS -> MFMA fragment: element (e, k) of the tile, e = output index inside the tile.
 template <int EXT, bool KC>
 __device__ __forceinline__ double read_frag(const double* __restrict__ lds, int e, int k) {
-  constexpr int S = TileGeom<EXT, KC>::stride;
+  constexpr int S = TileGeom<EXT, KC, 64>::stride;
   return KC ? lds[e * S + (k ^ (e & 15))] : lds[k * S + e];
 }
 
-template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
-__global__ __launch_bounds__(kThreads, 2) void gemm_f64_mfma(const GemmParams p) {
-  using GA = TileGeom<BM, A_KC>;
-  using GB = TileGeom<BN, B_KC>;
-  constexpr int WM = BM / 2, WN = BN / 2;    // per-wavefront block
+template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
+__global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm_f64_mfma(
+    const GemmParams p) {
+  constexpr int kThreads = WGM * WGN * 64;
+  using GA = TileGeom<BM, A_KC, kThreads>;
+  using GB = TileGeom<BN, B_KC, kThreads>;
+  constexpr int WM = BM / WGM, WN = BN / WGN;  // per-wavefront block
   constexpr int TM = WM / 16, TN = WN / 16;  // MFMA tiles per wavefront
   static_assert(WM % 16 == 0 && WN % 16 == 0, "wave block must be whole MFMA tiles");
 
@@ -184,7 +185,7 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f64_mfma(const GemmParams p)
 
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
   const int lr = lane & 15, lk = lane >> 4;
 
   v4d acc[TM][TN];
@@ -200,18 +201,18 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f64_mfma(const GemmParams p)
   // Loads the operand tiles of K step `kt` into registers; only the last step can be partial.
   auto fetch = [&](int kt) {
     if (kt < nk_full) {
-      load_tile<BM, A_KC, VEC, false>(ra, p.A, p.lda, m0, p.M, kt * BK, p.K, tid);
-      load_tile<BN, B_KC, VEC, false>(rb, p.B, p.ldb, n0, p.N, kt * BK, p.K, tid);
+      load_tile<BM, A_KC, VEC, false, kThreads>(ra, p.A, p.lda, m0, p.M, kt * BK, p.K, tid);
+      load_tile<BN, B_KC, VEC, false, kThreads>(rb, p.B, p.ldb, n0, p.N, kt * BK, p.K, tid);
     } else {
-      load_tile<BM, A_KC, VEC, true>(ra, p.A, p.lda, m0, p.M, kt * BK, p.K, tid);
-      load_tile<BN, B_KC, VEC, true>(rb, p.B, p.ldb, n0, p.N, kt * BK, p.K, tid);
+      load_tile<BM, A_KC, VEC, true, kThreads>(ra, p.A, p.lda, m0, p.M, kt * BK, p.K, tid);
+      load_tile<BN, B_KC, VEC, true, kThreads>(rb, p.B, p.ldb, n0, p.N, kt * BK, p.K, tid);
     }
   };
 
   if (nk > 0) {
     fetch(0);
-    store_tile<BM, A_KC>(lds_a[0], ra, tid);
-    store_tile<BN, B_KC>(lds_b[0], rb, tid);
+    store_tile<BM, A_KC, kThreads>(lds_a[0], ra, tid);
+    store_tile<BN, B_KC, kThreads>(lds_b[0], rb, tid);
   }
   __syncthreads();
 
@@ -235,8 +236,8 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f64_mfma(const GemmParams p)
           acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[i], fb[j], acc[i][j], 0, 0, 0);
     }
     if (more) {
-      store_tile<BM, A_KC>(lds_a[cur ^ 1], ra, tid);
-      store_tile<BN, B_KC>(lds_b[cur ^ 1], rb, tid);
+      store_tile<BM, A_KC, kThreads>(lds_a[cur ^ 1], ra, tid);
+      store_tile<BN, B_KC, kThreads>(lds_b[cur ^ 1], rb, tid);
     }
     __syncthreads();
   }
@@ -269,14 +270,215 @@ __global__ __launch_bounds__(kThreads, 2) void gemm_f64_mfma(const GemmParams p)
   }
 }
 
-template <int BM, int BN, bool A_KC, bool B_KC, bool VEC>
+// ---- 128x128 tiles fed by direct global -> LDS loads ------------------------------------------
+// The main path for large, aligned problems (K a multiple of 16, 16-byte aligned operands).
+// global_load_lds_dwordx4 moves 16 bytes per lane straight into LDS (lane l lands at
+// base + 16*l), so no staging registers and no ds_write instructions are spent on the operand
+// tiles; a wavefront moves one 1 KiB chunk of a tile per instruction:
+//   contraction-contiguous operand: a chunk is 8 rows x 16 doubles; lane l fetches, for row
+//       l/8, the pair k = 2*((l%8) ^ ((row>>1)&7)), i.e. the XOR swizzle is applied by choosing
+//       the global address, and fragment reads undo it (read_frag_kc16);
+//   output-contiguous operand: a chunk is one k row of 128 doubles; rows sit 144 doubles apart.
+// STAGES LDS stages form a ring, tile kt+DIST is requested while tile kt is multiplied; the
+// wait before the barrier only covers the tile needed next.
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
+
+__device__ __forceinline__ void dma16(const double* g, double* lds_wave_base) {
+  // every lane moves 16 bytes; lane l lands at lds_wave_base + 16*l
+  __builtin_amdgcn_global_load_lds((gbl_ptr_t)g, (lds_ptr_t)(uintptr_t)lds_wave_base, 16, 0, 0);
+}
+
+// contraction-contiguous tile for DMA: [EXT][16], 16-byte slot j of row e holds the pair
+// k = 2*(j ^ ((e >> 1) & 7)), unswapped.
+__device__ __forceinline__ double read_frag_kc16(const double* __restrict__ lds, int e, int k) {
+  return lds[e * BK + 2 * ((k >> 1) ^ ((e >> 1) & 7)) + (k & 1)];
+}
+
+
+__device__ __forceinline__ void wait_vmcnt(int n) {
+  // s_waitcnt with only the vector-memory counter constrained (gfx9 encoding)
+  switch (n) {
+    case 0: __builtin_amdgcn_s_waitcnt(0x0F70 | 0); break;
+    case 1: __builtin_amdgcn_s_waitcnt(0x0F70 | 1); break;
+    case 2: __builtin_amdgcn_s_waitcnt(0x0F70 | 2); break;
+    case 3: __builtin_amdgcn_s_waitcnt(0x0F70 | 3); break;
+    case 4: __builtin_amdgcn_s_waitcnt(0x0F70 | 4); break;
+    case 6: __builtin_amdgcn_s_waitcnt(0x0F70 | 6); break;
+    case 8: __builtin_amdgcn_s_waitcnt(0x0F70 | 8); break;
+    case 12: __builtin_amdgcn_s_waitcnt(0x0F70 | 12); break;
+    default: __builtin_amdgcn_s_waitcnt(0x0F70 | 0); break;
+  }
+}
+
+template <bool A_KC, bool B_KC, int WGM, int WGN, int STAGES, int DIST>
+__global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const GemmParams p) {
+  constexpr int BM = 128, BN = 128, NW = WGM * WGN;
+  constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 16, TN = WN / 16;
+  constexpr int CH = 16 / NW;  // 1 KiB chunks of each operand tile moved by one wavefront
+  static_assert(16 % NW == 0 && CH >= 1, "chunks must split over the wavefronts");
+  constexpr int A_SIZE = A_KC ? BM * BK : BK * (BM + 16);
+  constexpr int B_SIZE = B_KC ? BN * BK : BK * (BN + 16);
+  __shared__ __attribute__((aligned(1024))) double lds_a[STAGES][A_SIZE];
+  __shared__ __attribute__((aligned(1024))) double lds_b[STAGES][B_SIZE];
+
+  const int n_blocks = gridDim.x;
+  int logical;
+  {
+    const int pid = blockIdx.x;
+    const int xcd = pid & 7, local = pid >> 3;
+    const int base = n_blocks >> 3, rem = n_blocks & 7;
+    logical = xcd * base + (xcd < rem ? xcd : rem) + local;
+  }
+  int tile_m, tile_n;
+  {
+    constexpr int GROUP = 8;
+    const int group_size = GROUP * p.tiles_n;
+    const int group = logical / group_size;
+    const int first_m = group * GROUP;
+    const int gm = (p.tiles_m - first_m) < GROUP ? (p.tiles_m - first_m) : GROUP;
+    const int in_group = logical - group * group_size;
+    tile_m = first_m + in_group % gm;
+    tile_n = in_group / gm;
+  }
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+  const int lr = lane & 15, lk = lane >> 4;
+
+  const double* ga[CH];
+  const double* gb[CH];
+  int la[CH], lb[CH];
+#pragma unroll
+  for (int h = 0; h < CH; ++h) {
+    const int c = wave + NW * h;
+    if (A_KC) {
+      const int row = 8 * c + (lane >> 3);
+      int gr = m0 + row; gr = gr < p.M ? gr : p.M - 1;
+      ga[h] = p.A + (size_t)gr * p.lda + 2 * ((lane & 7) ^ ((row >> 1) & 7));
+      la[h] = c * 128;
+    } else {
+      int ge = m0 + 2 * lane; ge = ge + 1 < p.M ? ge : p.M - 2;
+      ga[h] = p.A + (size_t)c * p.lda + ge;
+      la[h] = c * (BM + 16);
+    }
+    if (B_KC) {
+      const int row = 8 * c + (lane >> 3);
+      int gr = n0 + row; gr = gr < p.N ? gr : p.N - 1;
+      gb[h] = p.B + (size_t)gr * p.ldb + 2 * ((lane & 7) ^ ((row >> 1) & 7));
+      lb[h] = c * 128;
+    } else {
+      int ge = n0 + 2 * lane; ge = ge + 1 < p.N ? ge : p.N - 2;
+      gb[h] = p.B + (size_t)c * p.ldb + ge;
+      lb[h] = c * (BN + 16);
+    }
+  }
+  const long a_step = A_KC ? BK : (long)BK * p.lda;
+  const long b_step = B_KC ? BK : (long)BK * p.ldb;
+
+  v4d acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
+
+  const int nk = p.K / BK;
+  auto issue = [&](int stage) {
+#pragma unroll
+    for (int h = 0; h < CH; ++h) {
+      dma16(ga[h], &lds_a[stage][la[h]]);
+      dma16(gb[h], &lds_b[stage][lb[h]]);
+      ga[h] += a_step;
+      gb[h] += b_step;
+    }
+  };
+  // prologue: tiles 0 .. DIST-1 in flight, tile 0 landed
+#pragma unroll
+  for (int d = 0; d < DIST; ++d)
+    if (d < nk) issue(d);
+  if (nk >= DIST) wait_vmcnt((DIST - 1) * 2 * CH); else wait_vmcnt(0);
+  __builtin_amdgcn_s_barrier();
+
+  int cur = 0, nxt = DIST % STAGES;
+  for (int kt = 0; kt < nk; ++kt) {
+    if (kt + DIST < nk) issue(nxt);
+    const double* __restrict__ sa = lds_a[cur];
+    const double* __restrict__ sb = lds_b[cur];
+#pragma unroll
+    for (int ks = 0; ks < BK / 4; ++ks) {
+      double fa[TM], fb[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int e = wm * WM + i * 16 + lr, k = ks * 4 + lk;
+        fa[i] = A_KC ? read_frag_kc16(sa, e, k) : sa[k * (BM + 16) + e];
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int e = wn * WN + j * 16 + lr, k = ks * 4 + lk;
+        fb[j] = B_KC ? read_frag_kc16(sb, e, k) : sb[k * (BN + 16) + e];
+      }
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    }
+    // tile kt+1 must have landed: at most DIST-1 younger tiles may still be in flight
+    if (kt + DIST < nk) wait_vmcnt((DIST - 1) * 2 * CH); else wait_vmcnt(0);
+    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS reads of `cur` are done
+    __builtin_amdgcn_s_barrier();
+    cur = cur + 1 == STAGES ? 0 : cur + 1;
+    nxt = nxt + 1 == STAGES ? 0 : nxt + 1;
+  }
+
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = n0 + wn * WN + j * 16 + lr;
+      if (col >= p.N) continue;
+      double bias = 0.0;
+      if (p.epilogue == EPI_BIAS || p.epilogue == EPI_BIAS_RELU) bias = p.bias[col];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = m0 + wm * WM + i * 16 + 4 * r + lk;
+        if (row >= p.M) continue;
+        double v = acc[i][j][r];
+        switch (p.epilogue) {
+          case EPI_BIAS: v = v + bias; break;
+          case EPI_BIAS_RELU: v = fmax(v + bias, 0.0); break;
+          case EPI_RELU: v = fmax(v, 0.0); break;
+          case EPI_DIVIDE: v = v / p.divisor; break;
+          case EPI_MASK: v = v * (p.mask[(size_t)row * p.ldmask + col] > 0.0 ? 1.0 : 0.0); break;
+          default: break;
+        }
+        p.C[(size_t)row * p.ldc + col] = v;
+      }
+    }
+  }
+}
+
+template <bool A_KC, bool B_KC>
+int launch_dma(hipStream_t stream, GemmParams p) {
+  p.tiles_m = (p.M + 127) / 128;
+  p.tiles_n = (p.N + 127) / 128;
+  const long long blocks = (long long)p.tiles_m * p.tiles_n;
+  if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
+  hipLaunchKernelGGL((gemm_f64_mfma_dma<A_KC, B_KC, 2, 4, 2, 1>), dim3((unsigned)blocks),
+                     dim3(512), 0, stream, p);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
 int launch_one(hipStream_t stream, GemmParams p) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   const long long blocks = (long long)p.tiles_m * p.tiles_n;
   if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
-  hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, A_KC, B_KC, VEC>), dim3((unsigned)blocks),
-                     dim3(kThreads), 0, stream, p);
+  hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, WGM, WGN, A_KC, B_KC, VEC>), dim3((unsigned)blocks),
+                     dim3(WGM * WGN * 64), 0, stream, p);
   RST_HIP(hipGetLastError());
   return RST_OK;
 }
@@ -288,9 +490,12 @@ int launch_layout(hipStream_t stream, const GemmParams& p) {
   auto tiles = [&](int bm, int bn) {
     return (long long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
   };
-  if (tiles(128, 128) >= 256) return launch_one<128, 128, A_KC, B_KC, VEC>(stream, p);
-  if (tiles(64, 64) >= 256) return launch_one<64, 64, A_KC, B_KC, VEC>(stream, p);
-  return launch_one<32, 32, A_KC, B_KC, VEC>(stream, p);
+  if (tiles(128, 128) >= 256) {
+    if (VEC && p.K % BK == 0 && p.K > 0 && p.M >= 2 && p.N >= 2) return launch_dma<A_KC, B_KC>(stream, p);
+    return launch_one<128, 128, 2, 4, A_KC, B_KC, VEC>(stream, p);
+  }
+  if (tiles(64, 64) >= 256) return launch_one<64, 64, 2, 2, A_KC, B_KC, VEC>(stream, p);
+  return launch_one<32, 32, 2, 2, A_KC, B_KC, VEC>(stream, p);
 }
 
 }  // namespace

@@ -24,6 +24,9 @@ SHAPES = [
     (1, 1, 1), (3, 2, 1), (2, 3, 10), (32, 784, 100), (32, 100, 100), (32, 100, 10),
     (37, 101, 13), (5, 7, 3), (129, 17, 130), (64, 64, 64), (100, 300, 33),
     (512, 256, 384), (1024, 128, 1000), (256, 1024, 1024), (2048, 100, 10),
+    # >= 256 tiles of 128x128 with ragged edges: the direct-to-LDS kernels (K % 16 == 0) and the
+    # register-staged kernel with a K tail, for each of the three operand layouts
+    (2050, 64, 2046), (2064, 2046, 2046), (2050, 2046, 2048),
 ]
 
 
