@@ -61,8 +61,11 @@ int rst_engine_device_info(rst_engine* engine, char* name, size_t name_capacity,
                            int* compute_units, size_t* total_memory_bytes);
 
 /* ---- device memory (counts are numbers of doubles) -------------------------------------- */
+/* rst_free keeps the block in a per-engine cache for the next rst_malloc of the same size (no
+ * device synchronisation on either call); rst_engine_trim returns the cache to the driver. */
 int rst_malloc(rst_engine* engine, size_t count, double** out);
 int rst_free(rst_engine* engine, double* ptr);
+int rst_engine_trim(rst_engine* engine);
 int rst_upload(rst_engine* engine, double* dst, const double* host_src, size_t count);
 int rst_download(rst_engine* engine, double* host_dst, const double* src, size_t count);
 int rst_copy(rst_engine* engine, double* dst, const double* src, size_t count);
@@ -177,6 +180,10 @@ int rst_model_sgd_step(rst_model* model, double lr);
  * host_loss may be NULL: then the call returns without waiting for the GPU. */
 int rst_model_train_step(rst_model* model, const double* x, const double* truth, size_t batch,
                          double lr, double* host_loss);
+/* rst_model_train_step records its launches into a HIP graph the first time it sees a given
+ * (x, truth, batch, lr) and replays the graph afterwards; a different argument re-records.
+ * enabled == 0 switches to plain launches (profiling does so by itself).  Default: enabled. */
+int rst_model_graph_enable(rst_model* model, int enabled);
 /* Per-launch timing of the model's kernels: when enabled every launch is bracketed by events
  * on the engine's stream (this serialises nothing, the stream is already in order).  Records
  * accumulate over calls (up to 65536) until rst_model_profile_read, which waits for the stream,

@@ -63,6 +63,7 @@ SIGNATURES = {
     "rst_engine_create": [_i32, c_void_pp],
     "rst_engine_destroy": [_vp],
     "rst_engine_synchronize": [_vp],
+    "rst_engine_trim": [_vp],
     "rst_engine_device_info": [_vp, ctypes.c_char_p, _sz, ctypes.POINTER(_i32), c_size_p],
     "rst_malloc": [_vp, _sz, c_void_pp],
     "rst_free": [_vp, _dp],
@@ -98,6 +99,7 @@ SIGNATURES = {
     "rst_model_sgd_step": [_vp, _dbl],
     "rst_model_train_step": [_vp, _dp, _dp, _sz, _dbl, c_double_p],
     "rst_model_profile_enable": [_vp, _i32],
+    "rst_model_graph_enable": [_vp, _i32],
     "rst_model_profile_read": [_vp, ctypes.POINTER(KernelRecord), _sz, c_size_p],
 }
 _SPECIAL = {

@@ -1,0 +1,117 @@
+// The reference's unit tests for the hot path (src/module/linear.rs:97-131, relu.rs:38-57,
+// identity.rs:35-51, sequential.rs:119-172, optim/sgd.rs:34-43) written against the C++ mirror.
+#include <cmath>
+#include <cstdio>
+#include <vector>
+
+#include "rstorch.hpp"
+
+using namespace rstorch;
+
+static int failures = 0;
+#define EXPECT(cond)                                                        \
+  do {                                                                      \
+    if (!(cond)) { std::printf("FAILED %s:%d  %s\n", __FILE__, __LINE__, #cond); ++failures; } \
+  } while (0)
+
+// assert_array_eq! of the reference (src/lib.rs:27-49): shape + absolute tolerance 1e-6
+static bool array_eq(const Array2& a, const Array2& b, double tol = 1e-6) {
+  if (!a.same_shape(b)) return false;
+  auto x = a.to_host(), y = b.to_host();
+  for (size_t i = 0; i < x.size(); ++i)
+    if (!(std::fabs(x[i] - y[i]) <= tol)) return false;
+  return true;
+}
+
+struct FixedInit : InitParameters {
+  Array2 weight(size_t, size_t) const override { return Array2{{1.0, 0.5}}; }
+  Array2 bias(size_t, size_t) const override { return Array2{{10.0}}; }
+};
+
+template <class F> static bool panics(F f) {
+  try { f(); } catch (const Panic&) { return true; }
+  return false;
+}
+
+int main() {
+  try {
+    {  // linear.rs:97-105
+      Linear m = Linear::new_with_kernel(2, 1, FixedInit());
+      Array2 out = m.forward(Array2{{1.0, 2.0}, {3.0, -4.0}, {-5.0, -6.0}});
+      EXPECT(array_eq(out, Array2{{12.0}, {11.0}, {2.0}}));
+    }
+    {  // linear.rs:107-131
+      Linear m = Linear::new_with_kernel(2, 1, FixedInit());
+      m.forward(Array2{{1.0, 2.0}, {3.0, -4.0}, {-5.0, -6.0}, {-7.0, 8.0}});
+      Array2 gx = m.backward(Array2::ones(4, 1));
+      EXPECT(m.grad_weight().same_shape(m.weight()) && m.grad_bias().same_shape(m.bias()));
+      EXPECT(array_eq(m.grad_weight(), Array2{{-2.0, 0.0}}));
+      EXPECT(array_eq(m.grad_bias(), Array2{{1.0}}));
+      EXPECT(array_eq(gx, Array2{{1.0, 0.5}, {1.0, 0.5}, {1.0, 0.5}, {1.0, 0.5}}));
+      EXPECT(panics([&] { m.backward(Array2::ones(4, 1)); }));  // cache consumed (linear.rs:61)
+    }
+    {  // relu.rs:38-57
+      ReLU m;
+      EXPECT(array_eq(m.forward(Array2{{1.0, 2.0}, {3.0, -4.0}, {-5.0, -6.0}}),
+                      Array2{{1.0, 2.0}, {3.0, 0.0}, {0.0, 0.0}}));
+      EXPECT(array_eq(m.backward(Array2::ones(3, 2)), Array2{{1.0, 1.0}, {1.0, 0.0}, {0.0, 0.0}}));
+      EXPECT(panics([&] { m.backward(Array2::ones(3, 2)); }));
+    }
+    {  // identity.rs:35-51
+      Identity m;
+      Array2 d{{1.0, 2.0}, {3.0, 4.0}, {5.0, 6.0}};
+      EXPECT(array_eq(m.forward(d), d) && array_eq(m.backward(d), d));
+    }
+    {  // sgd.rs:34-43
+      SGD optim(0.1);
+      Linear linear(2, 2);
+      auto w0 = linear.weight().to_host();
+      EXPECT(panics([&] { optim.step(linear); }));  // no gradient yet (linear.rs:72)
+      linear.forward(Array2::zeros(2, 2));
+      linear.backward(Array2::zeros(2, 2));
+      optim.step(linear);
+      EXPECT(linear.weight().to_host() == w0);
+    }
+    {  // sequential.rs:119-172 plus the container operations
+      Sequential module = sequential(Linear(3, 10), ReLU(), Linear(10, 100), ReLU(), Linear(100, 2));
+      EXPECT(module.len() == 5 && !module.is_empty());
+      Array2 out = module.forward(Array2{{1.0, 2.0, 3.0}, {-4.0, -5.0, -6.0}});
+      EXPECT(out.nrows() == 2 && out.ncols() == 2);
+      Array2 gin = module.backward(Array2{{1.0, 2.0}, {3.0, -4.0}});
+      EXPECT(gin.nrows() == 2 && gin.ncols() == 3);
+      EXPECT(module.parameters().size() == 6);
+      EXPECT(module.remove(9) == nullptr);
+      module.insert(0, Identity());
+      module.push(ReLU());
+      EXPECT(module.len() == 7);
+      EXPECT(module.forward(Array2{{1.0, 2.0, 3.0}}).ncols() == 2);
+    }
+    {  // fused Sequential == layer-by-layer calls, bit for bit, and the loss/accuracy path
+      Linear a(20, 30), b(30, 4);
+      Linear a2 = a, b2 = b;  // shares the device weights (read-only here)
+      Array2 x = Array2::normal(16, 20, 1, 1, 0.0, 1.0), y = Array2::one_hot(16, 4, 1, 2);
+      ReLU r;
+      Array2 manual = b.forward(r.forward(a.forward(x)));
+      Sequential s;
+      s.push(std::move(a2)); s.push(ReLU()); s.push(std::move(b2));
+      Array2 fused = s.forward(x);
+      EXPECT(manual.to_host() == fused.to_host());
+      CrossEntropyLoss l1, l2;
+      double v1 = l1.forward(manual.clone(), y.clone()), v2 = l2.forward(fused.clone(), y.clone());
+      EXPECT(v1 == v2 && std::isfinite(v1));
+      EXPECT(rstorch::utils::accuracy(manual, y) == rstorch::utils::accuracy(fused, y));
+      Array2 g1 = a.backward(r.backward(b.backward(l1.backward())));
+      Array2 g2 = s.backward(l2.backward());
+      EXPECT(g1.to_host() == g2.to_host());
+      EXPECT(panics([&] { l1.backward(); }));
+      EXPECT(panics([&] { CrossEntropyLoss().forward(Array2::zeros(2, 3), Array2::zeros(2, 4)); }));
+      Array2 bad = Array2::full(2, 3, std::nan(""));
+      EXPECT(panics([&] { CrossEntropyLoss().forward(bad, Array2::zeros(2, 3)); }));
+    }
+  } catch (const Panic& p) {
+    std::printf("unexpected panic: %s\n", p.what());
+    return 2;
+  }
+  if (failures == 0) std::printf("all mirror tests passed\n");
+  return failures == 0 ? 0 : 1;
+}

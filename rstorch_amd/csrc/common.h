@@ -7,6 +7,7 @@
 #include <cstddef>
 #include <cstdint>
 #include <string>
+#include <unordered_map>
 #include <vector>
 
 #include "../../include/rstorch_hip.h"
@@ -56,6 +57,13 @@ struct GemmDesc {
   double divisor;
   const double* mask;  // [M, ldmask]
   long ldmask;
+  // only with a_kc == false (weight gradient): colsum[i] = (sum_k A(i,k)) / colsum_div, i.e.
+  // the bias gradient, computed by the workgroups of the first tile column.  NULL: not wanted.
+  double* colsum;
+  double colsum_div;
+  // scratch for split-K partial products (small outputs with a long contraction); NULL: never split
+  double* workspace;
+  size_t workspace_count;
 };
 
 int launch_gemm(hipStream_t stream, const GemmDesc& d);
@@ -80,11 +88,16 @@ int launch_sgd_multi(hipStream_t s, const SgdTensor* device_table, size_t n_tens
                      unsigned long long total_blocks, double lr);
 unsigned long long sgd_blocks_for(unsigned long long count);
 
-// softmax / cross entropy.  row_loss: [rows] scratch; flags[0] is set to 1 on a NaN logit.
+// softmax / cross entropy.  grad_out != NULL: cross entropy (row kernel + a one-workgroup
+// reduction) - row_loss is [rows] scratch, loss[0] receives -(sum)/rows, flags[1] the NaN flag of
+// this call (flags[0] is a working word left at zero).  grad_out == NULL: softmax only, prob_out
+// is written and flags[2] is set on a NaN input.
 int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* grad_out,
-                      double* prob_out, double* row_loss, int* flags, size_t rows, size_t cols);
-// loss[0] = -(sum row_loss) / rows, fixed summation order
-int launch_loss_reduce(hipStream_t s, const double* row_loss, double* loss, size_t rows);
+                      double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
+                      size_t cols);
+int launch_softmax_rows(hipStream_t s, const double* z, const double* t, double* grad_out,
+                        double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
+                        size_t cols);
 // hits[0] = number of rows whose first arg-max agrees
 int launch_accuracy(hipStream_t s, const double* pred, const double* truth, size_t rows,
                     size_t cols, unsigned long long* hits);
@@ -111,9 +124,16 @@ struct rst_engine {
   int* h_flags = nullptr;    // pinned
   unsigned long long* h_hits = nullptr;  // pinned
   bool loss_valid = false;
+  // split-K scratch of the contraction kernels (fixed size, allocated with the engine)
+  double* d_gemm_ws = nullptr;
+  size_t gemm_ws_count = 0;
   // per-row loss scratch
   double* d_row_loss = nullptr;
   size_t row_loss_capacity = 0;
+  // rst_malloc / rst_free block cache (bytes -> free blocks) and the live allocations
+  std::unordered_map<size_t, std::vector<void*>> free_blocks;
+  std::unordered_map<void*, size_t> live_blocks;
+  size_t cached_bytes = 0;
   // SGD descriptor table cache
   rst::SgdTensor* d_sgd_table = nullptr;
   size_t sgd_table_capacity = 0;

@@ -97,6 +97,8 @@ int rst_engine_create(int device, rst_engine** out) {
   if (err == hipSuccess) err = hipMalloc(&e->d_loss, sizeof(double));
   if (err == hipSuccess) err = hipMalloc(&e->d_flags, 4 * sizeof(int));
   if (err == hipSuccess) err = hipMalloc(&e->d_hits, sizeof(unsigned long long));
+  e->gemm_ws_count = (size_t)4 << 20;  // 4 Mi doubles = 32 MiB
+  if (err == hipSuccess) err = hipMalloc(&e->d_gemm_ws, e->gemm_ws_count * sizeof(double));
   if (err == hipSuccess) err = hipHostMalloc(&e->h_loss, sizeof(double), hipHostMallocDefault);
   if (err == hipSuccess) err = hipHostMalloc(&e->h_flags, 4 * sizeof(int), hipHostMallocDefault);
   if (err == hipSuccess)
@@ -116,9 +118,13 @@ int rst_engine_destroy(rst_engine* e) {
   if (!e) return RST_OK;
   (void)hipSetDevice(e->device);
   if (e->stream) (void)hipStreamSynchronize(e->stream);
+  for (auto& kv : e->free_blocks)
+    for (void* p : kv.second) (void)hipFree(p);
+  for (auto& kv : e->live_blocks) (void)hipFree(kv.first);
   if (e->d_loss) (void)hipFree(e->d_loss);
   if (e->d_flags) (void)hipFree(e->d_flags);
   if (e->d_hits) (void)hipFree(e->d_hits);
+  if (e->d_gemm_ws) (void)hipFree(e->d_gemm_ws);
   if (e->d_row_loss) (void)hipFree(e->d_row_loss);
   if (e->d_sgd_table) (void)hipFree(e->d_sgd_table);
   if (e->h_loss) (void)hipHostFree(e->h_loss);
@@ -149,20 +155,55 @@ int rst_engine_device_info(rst_engine* e, char* name, size_t name_capacity, int*
   return RST_OK;
 }
 
+// Allocation goes through a per-engine cache of freed blocks keyed by size: the layer-by-layer
+// API allocates an output array per call (the reference allocates a fresh Array2 per expression
+// too), and hipMalloc / hipFree would synchronise the device every time.  A cached block is
+// only ever reused by work enqueued later on the engine's single stream, so reuse needs no wait.
 int rst_malloc(rst_engine* e, size_t count, double** out) {
   RST_TRY(engine_activate(e));
   if (!out) return fail(RST_ERR_INVALID_ARGUMENT, "out is null");
   *out = nullptr;
-  size_t bytes = (count ? count : 1) * sizeof(double);
-  RST_HIP(hipMalloc(out, bytes));
+  size_t bytes = ((count ? count : 1) * sizeof(double) + 255) / 256 * 256;
+  auto it = e->free_blocks.find(bytes);
+  if (it != e->free_blocks.end() && !it->second.empty()) {
+    *out = static_cast<double*>(it->second.back());
+    it->second.pop_back();
+    e->cached_bytes -= bytes;
+  } else {
+    void* p = nullptr;
+    hipError_t err = hipMalloc(&p, bytes);
+    if (err == hipErrorOutOfMemory && e->cached_bytes) {  // give the cache back and retry
+      (void)hipGetLastError();
+      RST_TRY(rst_engine_trim(e));
+      err = hipMalloc(&p, bytes);
+    }
+    if (err != hipSuccess) return fail_hip(err, "hipMalloc", __FILE__, __LINE__);
+    *out = static_cast<double*>(p);
+  }
+  e->live_blocks[*out] = bytes;
   return RST_OK;
 }
 
 int rst_free(rst_engine* e, double* ptr) {
-  RST_TRY(engine_activate(e));
+  if (!e) return fail(RST_ERR_INVALID_ARGUMENT, "engine is null");
   if (!ptr) return RST_OK;
+  auto it = e->live_blocks.find(ptr);
+  if (it == e->live_blocks.end())
+    return fail(RST_ERR_INVALID_ARGUMENT, "rst_free: pointer was not allocated by rst_malloc on this engine");
+  const size_t bytes = it->second;
+  e->live_blocks.erase(it);
+  e->free_blocks[bytes].push_back(ptr);
+  e->cached_bytes += bytes;
+  return RST_OK;
+}
+
+int rst_engine_trim(rst_engine* e) {
+  RST_TRY(engine_activate(e));
   RST_HIP(hipStreamSynchronize(e->stream));
-  RST_HIP(hipFree(ptr));
+  for (auto& kv : e->free_blocks)
+    for (void* p : kv.second) RST_HIP(hipFree(p));
+  e->free_blocks.clear();
+  e->cached_bytes = 0;
   return RST_OK;
 }
 

@@ -34,7 +34,17 @@ struct GemmParams {
   double divisor;
   const double* mask;
   long ldmask;
+  double* colsum;        // weight-gradient launches only: colsum[i] = (sum_k A(i,k)) / colsum_div
+  double colsum_div;
   int tiles_m, tiles_n;
+  // split-K (small outputs with a long contraction): slice s of the K steps is multiplied by
+  // workgroups [s*tiles, (s+1)*tiles) and lands, without epilogue, in ws[s][M][N] (and its
+  // column sums in ws_colsum[s][M]); split_reduce_kernel adds the slices in order afterwards.
+  int split_k;           // number of slices, 1 = off
+  int steps_per_split;   // K steps (of BK) per slice
+  double* ws;
+  double* ws_colsum;
+  size_t ws_capacity;    // doubles available at ws
 };
 
 // LDS geometry of one operand tile of EXT rows/cols by BK contraction steps.
@@ -146,6 +156,36 @@ __device__ __forceinline__ double read_frag(const double* __restrict__ lds, int 
   return KC ? lds[e * S + (k ^ (e & 15))] : lds[k * S + e];
 }
 
+// Bias gradient inside the weight-gradient contraction (output-contiguous A = grad^T): the
+// workgroups of tile column 0 also add up their A tile over the contraction index.  Thread t
+// owns output row t % BM and every (THREADS/BM)-th contraction row; partial sums are combined
+// through LDS in a fixed order at the end, so the result is reproducible.
+template <int BM, int THREADS>
+__device__ __forceinline__ void colsum_accumulate(double& partial, const double* __restrict__ lds_a_stage,
+                                                  int tid) {
+  constexpr int G = THREADS / BM;      // contraction-row groups
+  constexpr int S = BM + 16;           // LDS stride of an output-contiguous tile
+  const int e = tid % BM, kg = tid / BM;
+#pragma unroll
+  for (int k = kg; k < BK; k += G) partial += lds_a_stage[k * S + e];
+}
+
+template <int BM, int THREADS>
+__device__ __forceinline__ void colsum_finish(double partial, double* __restrict__ scratch, int tid,
+                                              int m0, int split, const GemmParams& p) {
+  constexpr int G = THREADS / BM;
+  const int e = tid % BM, kg = tid / BM;
+  scratch[kg * BM + e] = partial;
+  __syncthreads();
+  if (kg == 0 && m0 + e < p.M) {
+    double t = 0.0;
+#pragma unroll
+    for (int g = 0; g < G; ++g) t += scratch[g * BM + e];
+    if (p.split_k > 1) p.ws_colsum[(size_t)split * p.M + m0 + e] = t;  // slice sum, reduced later
+    else p.colsum[m0 + e] = t / p.colsum_div;
+  }
+}
+
 template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
 __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm_f64_mfma(
     const GemmParams p) {
@@ -162,10 +202,11 @@ __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm
   // Workgroups are handed to the 8 XCDs round-robin; renumber them so that each XCD (and
   // its private L2) works on one compact patch of the tile grid, then walk the patch in
   // groups of 8 tile rows so that concurrently resident workgroups share operand panels.
-  const int n_blocks = gridDim.x;
+  const int n_blocks = p.tiles_m * p.tiles_n;
+  const int split = blockIdx.x / n_blocks;  // K slice of this workgroup (0 without split-K)
   int logical;
   {
-    const int pid = blockIdx.x;
+    const int pid = blockIdx.x - split * n_blocks;
     const int xcd = pid & 7, local = pid >> 3;
     const int base = n_blocks >> 3, rem = n_blocks & 7;
     logical = xcd * base + (xcd < rem ? xcd : rem) + local;
@@ -196,7 +237,10 @@ __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm
 
   v2d ra[GA::loads], rb[GB::loads];
   const int nk_full = p.K / BK;                     // K steps that need no bounds handling
-  const int nk = nk_full + (p.K % BK != 0 ? 1 : 0);
+  const int nk_all = nk_full + (p.K % BK != 0 ? 1 : 0);
+  const int kt0 = split * p.steps_per_split;        // this workgroup's K steps: [kt0, nk)
+  const int nk = (p.split_k > 1 && kt0 + p.steps_per_split < nk_all) ? kt0 + p.steps_per_split
+                                                                      : nk_all;
 
   // Loads the operand tiles of K step `kt` into registers; only the last step can be partial.
   auto fetch = [&](int kt) {
@@ -209,19 +253,25 @@ __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm
     }
   };
 
-  if (nk > 0) {
-    fetch(0);
+  if (nk > kt0) {
+    fetch(kt0);
     store_tile<BM, A_KC, kThreads>(lds_a[0], ra, tid);
     store_tile<BN, B_KC, kThreads>(lds_b[0], rb, tid);
   }
   __syncthreads();
 
-  for (int kt = 0; kt < nk; ++kt) {
-    const int cur = kt & 1;
+  const bool do_colsum = !A_KC && p.colsum != nullptr && tile_n == 0;
+  double colsum_partial = 0.0;
+
+  for (int kt = kt0; kt < nk; ++kt) {
+    const int cur = (kt - kt0) & 1;
     const bool more = kt + 1 < nk;
     if (more) fetch(kt + 1);  // in flight while this step is multiplied
     const double* __restrict__ sa = lds_a[cur];
     const double* __restrict__ sb = lds_b[cur];
+    if (!A_KC) {
+      if (do_colsum) colsum_accumulate<BM, kThreads>(colsum_partial, sa, tid);
+    }
 #pragma unroll
     for (int ks = 0; ks < BK / 4; ++ks) {
       double fa[TM], fb[TN];
@@ -241,8 +291,26 @@ __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm
     }
     __syncthreads();
   }
+  if (!A_KC) {
+    if (do_colsum) colsum_finish<BM, kThreads>(colsum_partial, lds_b[0], tid, m0, split, p);
+  }
 
   // Epilogue: accumulator register r of this lane is row 4*r + lk, column lr of its tile.
+  if (p.split_k > 1) {  // raw partial products of this K slice; the reduction applies the epilogue
+    double* __restrict__ out = p.ws + (size_t)split * p.M * p.N;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wn * WN + j * 16 + lr;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = m0 + wm * WM + i * 16 + 4 * r + lk;
+          if (row < p.M && col < p.N) out[(size_t)row * p.N + col] = acc[i][j][r];
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -400,11 +468,17 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
   if (nk >= DIST) wait_vmcnt((DIST - 1) * 2 * CH); else wait_vmcnt(0);
   __builtin_amdgcn_s_barrier();
 
+  const bool do_colsum = !A_KC && p.colsum != nullptr && tile_n == 0;
+  double colsum_partial = 0.0;
+
   int cur = 0, nxt = DIST % STAGES;
   for (int kt = 0; kt < nk; ++kt) {
     if (kt + DIST < nk) issue(nxt);
     const double* __restrict__ sa = lds_a[cur];
     const double* __restrict__ sb = lds_b[cur];
+    if (!A_KC) {
+      if (do_colsum) colsum_accumulate<BM, NW * 64>(colsum_partial, sa, tid);
+    }
 #pragma unroll
     for (int ks = 0; ks < BK / 4; ++ks) {
       double fa[TM], fb[TN];
@@ -430,6 +504,9 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
     __builtin_amdgcn_s_barrier();
     cur = cur + 1 == STAGES ? 0 : cur + 1;
     nxt = nxt + 1 == STAGES ? 0 : nxt + 1;
+  }
+  if (!A_KC) {
+    if (do_colsum) colsum_finish<BM, NW * 64>(colsum_partial, lds_b[0], tid, m0, 0, p);
   }
 
 #pragma unroll
@@ -463,6 +540,7 @@ template <bool A_KC, bool B_KC>
 int launch_dma(hipStream_t stream, GemmParams p) {
   p.tiles_m = (p.M + 127) / 128;
   p.tiles_n = (p.N + 127) / 128;
+  p.split_k = 1;
   const long long blocks = (long long)p.tiles_m * p.tiles_n;
   if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
   hipLaunchKernelGGL((gemm_f64_mfma_dma<A_KC, B_KC, 2, 4, 2, 1>), dim3((unsigned)blocks),
@@ -471,22 +549,72 @@ int launch_dma(hipStream_t stream, GemmParams p) {
   return RST_OK;
 }
 
+// Adds the K slices of a split contraction in slice order and applies the epilogue.
+__global__ __launch_bounds__(256) void split_reduce_kernel(const GemmParams p) {
+  const size_t mn = (size_t)p.M * p.N;
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < mn) {
+    double v = 0.0;
+#pragma unroll 8
+    for (int s = 0; s < p.split_k; ++s) v += p.ws[(size_t)s * mn + i];
+    const int row = (int)(i / p.N), col = (int)(i - (size_t)row * p.N);
+    switch (p.epilogue) {
+      case EPI_BIAS: v = v + p.bias[col]; break;
+      case EPI_BIAS_RELU: v = fmax(v + p.bias[col], 0.0); break;
+      case EPI_RELU: v = fmax(v, 0.0); break;
+      case EPI_DIVIDE: v = v / p.divisor; break;
+      case EPI_MASK: v = v * (p.mask[(size_t)row * p.ldmask + col] > 0.0 ? 1.0 : 0.0); break;
+      default: break;
+    }
+    p.C[(size_t)row * p.ldc + col] = v;
+  }
+  if (p.colsum != nullptr && i < (size_t)p.M) {
+    double t = 0.0;
+    for (int s = 0; s < p.split_k; ++s) t += p.ws_colsum[(size_t)s * p.M + i];
+    p.colsum[i] = t / p.colsum_div;
+  }
+}
+
 template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
 int launch_one(hipStream_t stream, GemmParams p) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
-  const long long blocks = (long long)p.tiles_m * p.tiles_n;
+  long long blocks = (long long)p.tiles_m * p.tiles_n;
+  // Few output tiles but a long contraction: cut K into slices so that the chip fills up.
+  const int nk = (p.K + BK - 1) / BK;
+  p.split_k = 1;
+  p.steps_per_split = nk;
+  if (blocks < 256 && nk >= 8 && p.ws != nullptr) {
+    long long want = (2048 + blocks - 1) / blocks;           // about eight workgroups per CU
+    if (want > 64) want = 64;                                // keep the ordered reduction short
+    long long max_by_steps = nk / 4;                         // at least 4 K steps per slice
+    long long max_by_ws = (long long)(p.ws_capacity / ((size_t)p.M * p.N + (size_t)p.M));
+    long long s = want < max_by_steps ? want : max_by_steps;
+    if (s > max_by_ws) s = max_by_ws;
+    if (s > 1) {
+      p.steps_per_split = (int)((nk + s - 1) / s);
+      p.split_k = (nk + p.steps_per_split - 1) / p.steps_per_split;
+      p.ws_colsum = p.ws + (size_t)p.split_k * p.M * p.N;
+      blocks *= p.split_k;
+    }
+  }
   if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
   hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, WGM, WGN, A_KC, B_KC, VEC>), dim3((unsigned)blocks),
                      dim3(WGM * WGN * 64), 0, stream, p);
   RST_HIP(hipGetLastError());
+  if (p.split_k > 1) {
+    const size_t mn = (size_t)p.M * p.N;
+    hipLaunchKernelGGL(split_reduce_kernel, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, stream, p);
+    RST_HIP(hipGetLastError());
+  }
   return RST_OK;
 }
 
 template <bool A_KC, bool B_KC, bool VEC>
 int launch_layout(hipStream_t stream, const GemmParams& p) {
-  // Largest tile that still gives the 256 compute units about two workgroups each; small
-  // problems fall through to smaller tiles for parallelism.
+  // 128x128 tiles once they fill the 256 compute units, 64x64 while that still leaves about
+  // four workgroups per CU to overlap each other's load latency, else 32x32 (which cuts the
+  // contraction into slices when even that gives too few workgroups).
   auto tiles = [&](int bm, int bn) {
     return (long long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
   };
@@ -494,7 +622,7 @@ int launch_layout(hipStream_t stream, const GemmParams& p) {
     if (VEC && p.K % BK == 0 && p.K > 0 && p.M >= 2 && p.N >= 2) return launch_dma<A_KC, B_KC>(stream, p);
     return launch_one<128, 128, 2, 4, A_KC, B_KC, VEC>(stream, p);
   }
-  if (tiles(64, 64) >= 256) return launch_one<64, 64, 2, 2, A_KC, B_KC, VEC>(stream, p);
+  if (tiles(64, 64) >= 1024) return launch_one<64, 64, 2, 2, A_KC, B_KC, VEC>(stream, p);
   return launch_one<32, 32, 2, 2, A_KC, B_KC, VEC>(stream, p);
 }
 
@@ -508,6 +636,10 @@ int launch_gemm(hipStream_t stream, const GemmDesc& d) {
   p.lda = d.lda; p.ldb = d.ldb; p.ldc = d.ldc;
   p.epilogue = d.epilogue;
   p.bias = d.bias; p.divisor = d.divisor; p.mask = d.mask; p.ldmask = d.ldmask;
+  p.colsum = (!d.a_kc) ? d.colsum : nullptr;
+  p.colsum_div = d.colsum_div;
+  p.split_k = 1; p.steps_per_split = 0;
+  p.ws = d.workspace; p.ws_colsum = nullptr; p.ws_capacity = d.workspace ? d.workspace_count : 0;
   auto vec_ok = [](const double* ptr, long ld, int contiguous_extent) {
     return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && (ld % 2 == 0) &&
            (contiguous_extent % 2 == 0);

@@ -66,6 +66,13 @@ struct rst_model {
   bool forward_valid = false;
   bool loss_grad_valid = false;
   bool grads_valid = false;
+  // the captured training step (one graph launch instead of ~10 kernel launches)
+  bool graph_enabled = true;
+  hipGraphExec_t graph_exec = nullptr;
+  const double* graph_x = nullptr;
+  const double* graph_truth = nullptr;
+  size_t graph_batch = 0;
+  double graph_lr = 0.0;
   // profiling
   bool profiling = false;
   bool slot_open = false;
@@ -76,7 +83,13 @@ struct rst_model {
 
 namespace {
 
+void drop_graph(rst_model* m) {
+  if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
+  m->graph_exec = nullptr;
+}
+
 int free_activations(rst_model* m) {
+  drop_graph(m);  // it holds the addresses of these buffers
   for (auto& l : m->layers) {
     if (l.out_buf) RST_HIP(hipFree(l.out_buf));
     if (l.grad_in_buf) RST_HIP(hipFree(l.grad_in_buf));
@@ -174,6 +187,7 @@ int do_forward(rst_model* m, const double* x, size_t batch) {
       const double flops = 2.0 * (double)batch * (double)l.in * (double)l.out;
       const double bytes = 8.0 * ((double)batch * l.in + (double)l.in * l.out + (double)batch * l.out);
       RST_TRY(prof_begin(m, RST_KERNEL_LINEAR_FORWARD, i, flops, bytes));
+      d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
       RST_TRY(launch_gemm(e->stream, d));
       RST_TRY(prof_end(m));
       cur = l.out_buf;
@@ -250,14 +264,21 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
       d.lda = (long)l.out; d.ldb = (long)l.in; d.ldc = (long)l.in;
       d.a_kc = false; d.b_kc = false;
       d.epilogue = EPI_DIVIDE; d.divisor = n_rows;
+      // the bias gradient (linear.rs:65-67) is accumulated by the same launch
+      const bool fused_bias = l.in > 0 && batch > 0;
+      d.colsum = fused_bias ? l.gb : nullptr;
+      d.colsum_div = n_rows;
       const double bytes = 8.0 * ((double)batch * l.out + (double)batch * l.in + (double)l.in * l.out);
       RST_TRY(prof_begin(m, RST_KERNEL_GRAD_WEIGHT, i, 2.0 * mnk, bytes));
+      d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
       RST_TRY(launch_gemm(e->stream, d));
       RST_TRY(prof_end(m));
+      if (!fused_bias) {
+        RST_TRY(prof_begin(m, RST_KERNEL_GRAD_BIAS, i, 0.0, 8.0 * ((double)batch * l.out + l.out)));
+        RST_TRY(launch_column_mean(e->stream, cur, l.gb, batch, l.out, n_rows));
+        RST_TRY(prof_end(m));
+      }
     }
-    RST_TRY(prof_begin(m, RST_KERNEL_GRAD_BIAS, i, 0.0, 8.0 * ((double)batch * l.out + l.out)));
-    RST_TRY(launch_column_mean(e->stream, cur, l.gb, batch, l.out, n_rows));
-    RST_TRY(prof_end(m));
 
     const bool wanted = need_input_grad || i != first_linear;
     if (!wanted) { cur = nullptr; break; }
@@ -274,7 +295,8 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
     const double bytes = 8.0 * ((double)batch * l.out + (double)l.in * l.out +
                                 (double)batch * l.in * (mask ? 2.0 : 1.0));
     RST_TRY(prof_begin(m, RST_KERNEL_GRAD_INPUT, i, 2.0 * mnk, bytes));
-    RST_TRY(launch_gemm(e->stream, d));
+    d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
+      RST_TRY(launch_gemm(e->stream, d));
     RST_TRY(prof_end(m));
     if (mask) m->layers[pv].backward_absorbed = true;
     cur = l.grad_in_buf;
@@ -383,6 +405,7 @@ int rst_model_destroy(rst_model* m) {
   (void)hipSetDevice(m->engine->device);
   (void)hipStreamSynchronize(m->engine->stream);
   (void)free_activations(m);
+  drop_graph(m);
   if (m->parm_arena) (void)hipFree(m->parm_arena);
   if (m->grad_arena) (void)hipFree(m->grad_arena);
   for (hipEvent_t ev : m->event_pool) (void)hipEventDestroy(ev);
@@ -458,18 +481,84 @@ int rst_model_sgd_step(rst_model* m, double lr) {
   return do_sgd(m, lr);
 }
 
-int rst_model_train_step(rst_model* m, const double* x, const double* truth, size_t batch,
-                         double lr, double* host_loss) {
-  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
-  RST_TRY(engine_activate(m->engine));
-  if ((!x || !truth) && batch) return fail(RST_ERR_INVALID_ARGUMENT, "x or truth is null");
+}  // extern "C"
+
+namespace {
+
+int run_step(rst_model* m, const double* x, const double* truth, size_t batch, double lr) {
   RST_TRY(do_forward(m, x, batch));
   RST_TRY(do_loss(m, truth, nullptr));
   RST_TRY(do_backward(m, nullptr, 0, nullptr));
   RST_TRY(do_sgd(m, lr));
-  if (host_loss) return rst_loss_value(m->engine, host_loss);
   return RST_OK;
 }
+
+// Records the launches of one step into a graph.  Everything the step allocates lazily is
+// reserved first, because allocation is not allowed while the stream is capturing.  The graph
+// holds kernel nodes only (no memset nodes).
+int capture_step(rst_model* m, const double* x, const double* truth, size_t batch, double lr) {
+  rst_engine* e = m->engine;
+  drop_graph(m);
+  RST_TRY(reserve_activations(m, batch));
+  RST_TRY(engine_reserve_row_loss(e, batch));
+  RST_HIP(hipStreamBeginCapture(e->stream, hipStreamCaptureModeThreadLocal));
+  const int status = run_step(m, x, truth, batch, lr);
+  hipGraph_t graph = nullptr;
+  const hipError_t end = hipStreamEndCapture(e->stream, &graph);
+  if (status != RST_OK) {
+    if (graph) (void)hipGraphDestroy(graph);
+    return status;
+  }
+  if (end != hipSuccess) return fail_hip(end, "hipStreamEndCapture", __FILE__, __LINE__);
+  const hipError_t inst = hipGraphInstantiate(&m->graph_exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (inst != hipSuccess) {
+    m->graph_exec = nullptr;
+    return fail_hip(inst, "hipGraphInstantiate", __FILE__, __LINE__);
+  }
+  m->graph_x = x; m->graph_truth = truth; m->graph_batch = batch; m->graph_lr = lr;
+  return RST_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int rst_model_train_step(rst_model* m, const double* x, const double* truth, size_t batch,
+                         double lr, double* host_loss) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  rst_engine* e = m->engine;
+  RST_TRY(engine_activate(e));
+  if (!x || !truth) return fail(RST_ERR_INVALID_ARGUMENT, "x or truth is null");
+  if (batch == 0) return fail(RST_ERR_SHAPE, "training step on an empty batch");
+  if (m->graph_enabled && !m->profiling) {
+    const bool hit = m->graph_exec && m->graph_x == x && m->graph_truth == truth &&
+                     m->graph_batch == batch && m->graph_lr == lr;
+    if (!hit) RST_TRY(capture_step(m, x, truth, batch, lr));
+    RST_HIP(hipGraphLaunch(m->graph_exec, e->stream));
+    // the state the eager calls leave behind
+    m->batch = batch;
+    m->forward_valid = false;
+    m->loss_grad_valid = false;
+    m->grads_valid = true;
+    e->loss_valid = true;
+  } else {
+    RST_TRY(run_step(m, x, truth, batch, lr));
+  }
+  if (host_loss) return rst_loss_value(e, host_loss);
+  return RST_OK;
+}
+
+int rst_model_graph_enable(rst_model* m, int enabled) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->graph_enabled = enabled != 0;
+  if (!m->graph_enabled) drop_graph(m);
+  return RST_OK;
+}
+
+}  // extern "C"
+
+extern "C" {
 
 int rst_model_profile_enable(rst_model* m, int enabled) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");

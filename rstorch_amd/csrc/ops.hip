@@ -10,9 +10,7 @@ using namespace rst;
 namespace rst {
 namespace {
 
-__global__ void reset_flags_kernel(int* flags) {
-  if (threadIdx.x < 4) flags[threadIdx.x] = 0;
-}
+__global__ void reset_softmax_flag_kernel(int* flags) { flags[2] = 0; }
 
 int check_dim(size_t v, const char* what) {
   if (v > (size_t)INT_MAX) return fail(RST_ERR_UNSUPPORTED, "%s = %zu exceeds 2^31-1", what, v);
@@ -24,11 +22,9 @@ int check_dim(size_t v, const char* what) {
 int engine_cross_entropy(rst_engine* e, const double* pred, const double* truth, double* grad_out,
                          double* prob_out, size_t rows, size_t cols, double* host_loss) {
   RST_TRY(engine_reserve_row_loss(e, rows));
-  hipLaunchKernelGGL(reset_flags_kernel, dim3(1), dim3(64), 0, e->stream, e->d_flags);
-  RST_HIP(hipGetLastError());
-  RST_TRY(launch_softmax_ce(e->stream, pred, truth, grad_out, prob_out, e->d_row_loss, e->d_flags,
-                            rows, cols));
-  RST_TRY(launch_loss_reduce(e->stream, e->d_row_loss, e->d_loss, rows));
+  if (rows == 0 || cols == 0) return fail(RST_ERR_SHAPE, "cross entropy of an empty batch");
+  RST_TRY(launch_softmax_ce(e->stream, pred, truth, grad_out, prob_out, e->d_row_loss, e->d_loss,
+                            e->d_flags, rows, cols));
   e->loss_valid = true;
   if (host_loss) return rst_loss_value(e, host_loss);
   return RST_OK;
@@ -56,6 +52,7 @@ int rst_linear_forward(rst_engine* e, const double* x, const double* weight, con
   d.bias = bias;
   if (bias) d.epilogue = fuse_relu ? EPI_BIAS_RELU : EPI_BIAS;
   else d.epilogue = fuse_relu ? EPI_RELU : EPI_NONE;
+  d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
   return launch_gemm(e->stream, d);
 }
 
@@ -77,9 +74,14 @@ int rst_linear_backward(rst_engine* e, const double* grad, const double* x, cons
     d.lda = (long)out_features; d.ldb = (long)in_features; d.ldc = (long)in_features;
     d.a_kc = false; d.b_kc = false;
     d.epilogue = EPI_DIVIDE; d.divisor = n;
-    RST_TRY(launch_gemm(e->stream, d));
+    // grad_bias[1,out] = colsum(grad) / n rides along in the same launch
+    d.colsum = (in_features > 0 && batch > 0) ? grad_bias : nullptr;
+    d.colsum_div = n;
+    d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
+      RST_TRY(launch_gemm(e->stream, d));
+    if (grad_bias && !d.colsum)
+      RST_TRY(launch_column_mean(e->stream, grad, grad_bias, batch, out_features, n));
   }
-  if (grad_bias) RST_TRY(launch_column_mean(e->stream, grad, grad_bias, batch, out_features, n));
   if (grad_input) {  // grad_input[batch,in] = grad . weight
     GemmDesc d{};
     d.A = grad; d.B = weight; d.C = grad_input;
@@ -88,7 +90,8 @@ int rst_linear_backward(rst_engine* e, const double* grad, const double* x, cons
     d.a_kc = true; d.b_kc = false;
     d.epilogue = relu_mask_source ? EPI_MASK : EPI_NONE;
     d.mask = relu_mask_source; d.ldmask = (long)in_features;
-    RST_TRY(launch_gemm(e->stream, d));
+    d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
+      RST_TRY(launch_gemm(e->stream, d));
   }
   return RST_OK;
 }
@@ -111,12 +114,13 @@ int rst_softmax_rows(rst_engine* e, const double* x, double* out, size_t rows, s
   RST_TRY(engine_activate(e));
   if (rows == 0 || cols == 0) return RST_OK;
   if (!x || !out) return fail(RST_ERR_INVALID_ARGUMENT, "softmax_rows: null operand");
-  hipLaunchKernelGGL(reset_flags_kernel, dim3(1), dim3(64), 0, e->stream, e->d_flags);
+  hipLaunchKernelGGL(reset_softmax_flag_kernel, dim3(1), dim3(1), 0, e->stream, e->d_flags);
   RST_HIP(hipGetLastError());
-  RST_TRY(launch_softmax_ce(e->stream, x, nullptr, nullptr, out, nullptr, e->d_flags, rows, cols));
-  RST_HIP(hipMemcpyAsync(e->h_flags, e->d_flags, sizeof(int), hipMemcpyDeviceToHost, e->stream));
+  RST_TRY(launch_softmax_ce(e->stream, x, nullptr, nullptr, out, nullptr, nullptr, e->d_flags, rows,
+                            cols));
+  RST_HIP(hipMemcpyAsync(e->h_flags, e->d_flags, 4 * sizeof(int), hipMemcpyDeviceToHost, e->stream));
   RST_HIP(hipStreamSynchronize(e->stream));
-  if (e->h_flags[0] & 1)
+  if (e->h_flags[2] & 1)
     return fail(RST_ERR_NAN, "softmax: NaN in the input (the reference panics in softmax.rs:38)");
   return RST_OK;
 }
@@ -134,10 +138,10 @@ int rst_loss_value(rst_engine* e, double* host_loss) {
   if (!host_loss) return fail(RST_ERR_INVALID_ARGUMENT, "host_loss is null");
   if (!e->loss_valid) return fail(RST_ERR_STATE, "no loss has been computed on this engine");
   RST_HIP(hipMemcpyAsync(e->h_loss, e->d_loss, sizeof(double), hipMemcpyDeviceToHost, e->stream));
-  RST_HIP(hipMemcpyAsync(e->h_flags, e->d_flags, sizeof(int), hipMemcpyDeviceToHost, e->stream));
+  RST_HIP(hipMemcpyAsync(e->h_flags, e->d_flags, 4 * sizeof(int), hipMemcpyDeviceToHost, e->stream));
   RST_HIP(hipStreamSynchronize(e->stream));
   *host_loss = *e->h_loss;
-  if (e->h_flags[0] & 1)
+  if (e->h_flags[1] & 1)
     return fail(RST_ERR_NAN, "cross entropy: NaN logits (the reference panics in softmax.rs:38)");
   return RST_OK;
 }

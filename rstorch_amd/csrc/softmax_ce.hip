@@ -53,8 +53,8 @@ __device__ __forceinline__ double loss_term(double truth, double p) {
 template <int TPR, int IPT, int VEC, bool CE>
 __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
     const double* __restrict__ z, const double* __restrict__ truth, double* __restrict__ grad,
-    double* __restrict__ prob, double* __restrict__ row_loss, int* __restrict__ flags, size_t rows,
-    size_t cols) {
+    double* __restrict__ prob, double* __restrict__ row_loss, double* __restrict__ loss,
+    int* __restrict__ flags, size_t rows, size_t cols) {
   constexpr int BLOCK = TPR > 256 ? TPR : 256;
   constexpr int RPB = BLOCK / TPR;
   __shared__ double red[3][TPR > 64 ? TPR / 64 : 1];
@@ -146,16 +146,18 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
   if (CE) {
     lsum = group_reduce<TPR, SumOp>(lsum, red[2]);
     if (sub == 0 && row_ok) row_loss[row] = lsum;
+    if (saw_nan) atomicOr(&flags[0], 1);
+  } else {
+    if (saw_nan) atomicOr(&flags[2], 1);
   }
-  if (saw_nan) atomicOr(flags, 1);
 }
 
 // Rows too long for registers: one 1024-thread workgroup per row, three passes over memory.
 template <bool CE>
 __global__ __launch_bounds__(1024) void softmax_long_rows_kernel(
     const double* __restrict__ z, const double* __restrict__ truth, double* __restrict__ grad,
-    double* __restrict__ prob, double* __restrict__ row_loss, int* __restrict__ flags, size_t rows,
-    size_t cols) {
+    double* __restrict__ prob, double* __restrict__ row_loss, double* __restrict__ loss,
+    int* __restrict__ flags, size_t rows, size_t cols) {
   constexpr int TPR = 1024;
   __shared__ double red[3][TPR / 64];
   const size_t row = blockIdx.x;
@@ -185,53 +187,62 @@ __global__ __launch_bounds__(1024) void softmax_long_rows_kernel(
   if (CE) {
     lsum = group_reduce<TPR, SumOp>(lsum, red[2]);
     if (threadIdx.x == 0) row_loss[row] = lsum;
+    if (saw_nan) atomicOr(&flags[0], 1);
+  } else {
+    if (saw_nan) atomicOr(&flags[2], 1);
   }
-  if (saw_nan) atomicOr(flags, 1);
 }
 
-// loss = -(sum of the per-row sums) / rows, one workgroup, fixed order.
+// Second (tiny) launch of a cross entropy: loss = -(sum of the per-row sums) / rows in a fixed
+// order, one workgroup.  It also latches the NaN flag of the launch into flags[1] and re-arms
+// flags[0], so no reset launch is needed.
 __global__ __launch_bounds__(1024) void loss_reduce_kernel(const double* __restrict__ row_loss,
-                                                          double* __restrict__ loss, size_t rows) {
+                                                          double* __restrict__ loss,
+                                                          int* __restrict__ flags, size_t rows) {
   __shared__ double red[1024 / 64];
   double s = 0.0;
   for (size_t r = threadIdx.x; r < rows; r += 1024) s += row_loss[r];
   s = group_reduce<1024, SumOp>(s, red);
-  if (threadIdx.x == 0) loss[0] = -s / (double)rows;
+  if (threadIdx.x == 0) {
+    loss[0] = -s / (double)rows;
+    flags[1] = flags[0];
+    flags[0] = 0;
+  }
 }
 
 template <int TPR, int IPT, int VEC>
 int launch_rows(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
-                double* row_loss, int* flags, size_t rows, size_t cols, bool ce) {
+                double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce) {
   constexpr int BLOCK = TPR > 256 ? TPR : 256;
   constexpr int RPB = BLOCK / TPR;
   size_t blocks = (rows + RPB - 1) / RPB;
   if (blocks > 0x7fffffffull) return fail(RST_ERR_UNSUPPORTED, "too many rows for one launch");
   if (ce)
     hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, true>), dim3((unsigned)blocks),
-                       dim3(BLOCK), 0, s, z, t, grad, prob, row_loss, flags, rows, cols);
+                       dim3(BLOCK), 0, s, z, t, grad, prob, row_loss, loss, flags, rows, cols);
   else
     hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, false>), dim3((unsigned)blocks),
-                       dim3(BLOCK), 0, s, z, t, grad, prob, row_loss, flags, rows, cols);
+                       dim3(BLOCK), 0, s, z, t, grad, prob, row_loss, loss, flags, rows, cols);
   RST_HIP(hipGetLastError());
   return RST_OK;
 }
 
 template <int VEC>
 int dispatch(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
-             double* row_loss, int* flags, size_t rows, size_t cols, bool ce) {
+             double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce) {
   const size_t units = cols / VEC;  // vectors per row
-  if (units <= 16 * 2) return launch_rows<16, 2, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
-  if (units <= 64 * 4) return launch_rows<64, 4, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
-  if (units <= 256 * 4) return launch_rows<256, 4, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
-  if (units <= 1024 * 4) return launch_rows<1024, 4, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
-  if (units <= 1024 * 16) return launch_rows<1024, 16, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
+  if (units <= 16 * 2) return launch_rows<16, 2, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
+  if (units <= 64 * 4) return launch_rows<64, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
+  if (units <= 256 * 4) return launch_rows<256, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
+  if (units <= 1024 * 4) return launch_rows<1024, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
+  if (units <= 1024 * 16) return launch_rows<1024, 16, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
   if (rows > 0x7fffffffull) return fail(RST_ERR_UNSUPPORTED, "too many rows for one launch");
   if (ce)
     hipLaunchKernelGGL(softmax_long_rows_kernel<true>, dim3((unsigned)rows), dim3(1024), 0, s, z, t,
-                       grad, prob, row_loss, flags, rows, cols);
+                       grad, prob, row_loss, loss, flags, rows, cols);
   else
     hipLaunchKernelGGL(softmax_long_rows_kernel<false>, dim3((unsigned)rows), dim3(1024), 0, s, z, t,
-                       grad, prob, row_loss, flags, rows, cols);
+                       grad, prob, row_loss, loss, flags, rows, cols);
   RST_HIP(hipGetLastError());
   return RST_OK;
 }
@@ -241,19 +252,26 @@ inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 1
 }  // namespace
 
 int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* grad_out,
-                      double* prob_out, double* row_loss, int* flags, size_t rows, size_t cols) {
+                      double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
+                      size_t cols) {
   if (rows == 0 || cols == 0) return RST_OK;
+  const bool ce = grad_out != nullptr;
+  RST_TRY(launch_softmax_rows(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols));
+  if (ce) {
+    hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(1024), 0, s, row_loss, loss, flags, rows);
+    RST_HIP(hipGetLastError());
+  }
+  return RST_OK;
+}
+
+int launch_softmax_rows(hipStream_t s, const double* z, const double* t, double* grad_out,
+                        double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
+                        size_t cols) {
   const bool ce = grad_out != nullptr;
   const bool vec = cols % 2 == 0 && aligned16(z) && (!ce || (aligned16(t) && aligned16(grad_out))) &&
                    (!prob_out || aligned16(prob_out));
-  if (vec) return dispatch<2>(s, z, t, grad_out, prob_out, row_loss, flags, rows, cols, ce);
-  return dispatch<1>(s, z, t, grad_out, prob_out, row_loss, flags, rows, cols, ce);
-}
-
-int launch_loss_reduce(hipStream_t s, const double* row_loss, double* loss, size_t rows) {
-  hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(1024), 0, s, row_loss, loss, rows);
-  RST_HIP(hipGetLastError());
-  return RST_OK;
+  if (vec) return dispatch<2>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce);
+  return dispatch<1>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce);
 }
 
 }  // namespace rst

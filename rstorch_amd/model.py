@@ -157,6 +157,10 @@ class DeviceModel:
         _ffi.check(self.engine.lib.rst_loss_value(self.engine.handle, ctypes.byref(v)))
         return v.value
 
+    def graph_enable(self, on=True):
+        """Replay the step as a HIP graph (default) or launch its kernels one by one."""
+        _ffi.check(self.engine.lib.rst_model_graph_enable(self.handle, 1 if on else 0))
+
     # -- per-kernel timing -------------------------------------------------------------------
     def profile_enable(self, on=True):
         _ffi.check(self.engine.lib.rst_model_profile_enable(self.handle, 1 if on else 0))

@@ -139,3 +139,31 @@ def test_profile_records_cover_every_launch(engine, oracle):
     assert "relu_forward" not in kinds and "relu_backward" not in kinds  # fused away
     assert all(r["ms"] > 0 for r in recs)
     dm.profile_enable(False)
+
+
+def test_graph_replay_equals_eager_launches(engine, oracle):
+    """The captured step must give bit-identical results on every replay, with other eager work
+    and synchronisations between replays, and must re-record when an argument changes."""
+    import rstorch_amd as rs
+    spec = README_MLP
+    weights = make_weights(oracle, spec, 21)
+    g = rs.DeviceModel(spec); g.load_parameters(weights)          # graph replay (default)
+    e = rs.DeviceModel(spec); e.load_parameters(weights); e.graph_enable(False)
+    other = rs.Linear.new(64, 64)
+    x0, y0 = batch_data(oracle, 32, 784, 10, 5, 0)
+    x1, y1 = batch_data(oracle, 32, 784, 10, 5, 1)
+    dx0, dy0, dx1, dy1 = (engine.from_numpy(a) for a in (x0, y0, x1, y1))
+    for step in range(12):
+        x, y = (dx0, dy0) if step < 8 else (dx1, dy1)      # the change of batch re-records
+        lr = 0.01 if step != 5 else 0.02                   # so does a change of lr
+        lg = g.train_step(x, y, lr)
+        other.forward(np.ones((8, 64)))                    # unrelated eager work on the stream
+        engine.synchronize()
+        le = e.train_step(x, y, lr)
+        assert lg == le, "step %d" % step
+    for (p, _), (q, _) in zip(g.parameters(), e.parameters()):
+        np.testing.assert_array_equal(p.to_numpy(), q.to_numpy())
+    # the graph path keeps the state machine of the eager path
+    with pytest.raises(rs.StateError):
+        g.backward(None)
+    g.sgd_step(0.0)  # gradients exist
