@@ -26,6 +26,16 @@ sys.path.insert(0, ROOT)
 PEAK_FP64_MFMA_TFLOPS = 78.6
 PEAK_HBM_GBPS = 8000.0
 
+# HBM-side bytes per launch of the C4 contraction kernels, averaged over the launches of one step
+# (8 hidden layers + the head).  Measured with two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE)
+# of this script, scaled by the same counters on a streaming kernel of known size
+# (--calibration-copy: FETCH x 2.0, WRITE x 1.0); the summary is kept under profiles/.
+C4_TRAFFIC_BYTES_PER_LAUNCH = {
+    "linear_forward": (8 * 436.5e6 + 4474.9e6) / 9,
+    "grad_weight": (8 * 516.5e6 + 4276.8e6) / 9,
+    "grad_input": 982.5e6,
+}
+
 C4_SPEC = [("linear", 4096, 4096), ("relu",)] * 8 + [("linear", 4096, 32768)]
 C4_BATCH = 1024
 C2_SPEC = [("linear", 1024, 4096), ("relu",), ("linear", 4096, 4096), ("relu",),
@@ -175,6 +185,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one streaming ReLU over 1 GiB (reads 1 GiB, writes 1 GiB): the "
+                         "known-size kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs the training step on ONE GPU; --gpus %d is not "
@@ -184,6 +197,15 @@ def main():
     eng = rs.default_engine()
     info = eng.device_info()
     log("device: %s, %d CUs" % (info["name"], info["compute_units"]))
+
+    if args.calibration_copy:
+        from rstorch_amd import _ffi
+        n = 1 << 27  # doubles = 1 GiB
+        src, dst = eng.normal(1, n, SEED, 3000), eng.empty(1, n)
+        for _ in range(2):
+            _ffi.check(eng.lib.rst_relu_forward(eng.handle, src.ptr, dst.ptr, n))
+        eng.synchronize()
+        del src, dst
 
     dm, x, y = make_model(rs, eng, C4_SPEC, C4_BATCH, True)
     tensors, params = dm.parameter_count()
@@ -200,7 +222,9 @@ def main():
     flops_per_launch = sum(r["flops"] for r in launches) / len(launches)
     roofline = {"kernel": "gemm_f64_mfma (" + dominant + ")", "bound": "mfma",
                 "achieved": d["achieved_tflops"], "peak": PEAK_FP64_MFMA_TFLOPS, "unit": "TFLOP/s",
-                "frac": d["frac"], "traffic": None,
+                "frac": d["frac"], "traffic": C4_TRAFFIC_BYTES_PER_LAUNCH.get(dominant),
+                "traffic_unit": "bytes per launch (L2 misses + write-backs, rocprofv3 FETCH_SIZE/WRITE_SIZE)",
+                "algorithmic_bytes_per_launch": sum(r["bytes"] for r in launches) / len(launches),
                 "avg_launch_ms": d["avg_launch_ms"], "flops_per_launch": flops_per_launch}
     gemm_ms = sum(kernels[k]["ms_per_step"] for k in gemm_kinds)
     gemm_flops = sum(r["flops"] for r in recs if r["kernel"] in gemm_kinds) / args.steps
