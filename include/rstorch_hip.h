@@ -144,6 +144,28 @@ int rst_fill_normal(rst_engine* engine, double* dst, size_t count, uint64_t seed
 int rst_fill_one_hot(rst_engine* engine, double* dst, size_t rows, size_t cols, uint64_t seed,
                      uint64_t stream);
 
+/* ---- input staging (the step before the path: src/data/data_loader.rs:192-207 builds a batch
+ *      on the host, src/utils.rs:38-42 expands labels to one-hot rows) ------------------------ */
+typedef struct rst_stager rst_stager;
+/* `depth` slots of pinned host memory + device memory and a copy stream of its own: the transfer
+ * of batch k+1 overlaps the training step on batch k.  x is [rows <= max_rows, x_cols] f64. */
+int rst_stager_create(rst_engine* engine, size_t max_rows, size_t x_cols, size_t classes,
+                      int depth, rst_stager** out);
+int rst_stager_destroy(rst_stager* stager);
+/* Copies the host batch into the next free slot and starts its transfer; does not wait for the
+ * GPU.  Labels are class indices; the dense one-hot truth [rows, classes] is built on the device.
+ * RST_ERR_STATE when all slots are submitted and none has been taken with rst_stager_next. */
+int rst_stager_submit_labels(rst_stager* stager, const double* host_x, const uint32_t* host_labels,
+                             size_t rows);
+/* Same with a dense (possibly soft-label) truth matrix [rows, classes]. */
+int rst_stager_submit_dense(rst_stager* stager, const double* host_x, const double* host_truth,
+                            size_t rows);
+/* Hands out the oldest submitted batch: the engine's stream waits for its transfer (the host does
+ * not).  The device arrays stay valid until `depth` further submits; work that reads them must
+ * be enqueued on the engine before the submit that reuses their slot. */
+int rst_stager_next(rst_stager* stager, const double** x_dev, const double** truth_dev,
+                    size_t* rows);
+
 /* ---- device-resident Sequential (src/module/sequential.rs:78-109) ------------------------ */
 enum { RST_LAYER_IDENTITY = 0, RST_LAYER_LINEAR = 1, RST_LAYER_RELU = 2 };
 
@@ -159,6 +181,11 @@ int rst_model_parameter_count(rst_model* model, size_t* tensor_count, size_t* el
  * bias (1,out); src/module/linear.rs:71-78): device pointers of the parameter and its gradient. */
 int rst_model_parameter(rst_model* model, size_t index, double** parm, double** grad,
                         size_t* rows, size_t* cols);
+/* Every parameter packed without padding into / out of one host array of `count` =
+ * element_count doubles, tensors in the order of rst_model_parameter (a checkpoint; the reference
+ * has no serialisation, its weights are reachable only through parameters(), mod.rs:16-40). */
+int rst_model_export_parameters(rst_model* model, double* host_dst, size_t count);
+int rst_model_import_parameters(rst_model* model, const double* host_src, size_t count);
 /* KaimingNormal weights (std = 1/sqrt(in)), zero biases (src/module/init/mod.rs:15-17,
  * he.rs:11-14); tensor i uses generator stream `first_stream + i`. */
 int rst_model_init_kaiming(rst_model* model, uint64_t seed, uint64_t first_stream);

@@ -10,7 +10,7 @@ from ._ffi import NanError, RstorchError, ShapeError, StateError
 from .engine import Array2, Engine, as_array2, default_engine
 from .init import FromArrays, InitParameters, KaimingNormal, Normal, XavierNormal
 from .loss import CrossEntropyLoss, Loss
-from .model import BasicModel, DeviceModel
+from .model import BasicModel, BatchStager, DeviceModel
 from .module import (Identity, Linear, Module, Parameter, Parameters, ReLU, Sequential,
                      sequential)
 from .optim import SGD, Optimizer
@@ -21,6 +21,6 @@ __all__ = [
     "Module", "Parameter", "Parameters", "Identity", "Linear", "ReLU", "Sequential", "sequential",
     "Loss", "CrossEntropyLoss", "Optimizer", "SGD",
     "InitParameters", "KaimingNormal", "XavierNormal", "Normal", "FromArrays",
-    "BasicModel", "DeviceModel", "accuracy",
+    "BasicModel", "DeviceModel", "BatchStager", "accuracy",
     "RstorchError", "ShapeError", "StateError", "NanError",
 ]

@@ -93,6 +93,13 @@ SIGNATURES = {
     "rst_model_parameter_count": [_vp, c_size_p, c_size_p],
     "rst_model_parameter": [_vp, _sz, c_void_pp, c_void_pp, c_size_p, c_size_p],
     "rst_model_init_kaiming": [_vp, _u64, _u64],
+    "rst_model_export_parameters": [_vp, c_double_p, _sz],
+    "rst_model_import_parameters": [_vp, c_double_p, _sz],
+    "rst_stager_create": [_vp, _sz, _sz, _sz, _i32, c_void_pp],
+    "rst_stager_destroy": [_vp],
+    "rst_stager_submit_labels": [_vp, c_double_p, ctypes.POINTER(ctypes.c_uint32), _sz],
+    "rst_stager_submit_dense": [_vp, c_double_p, c_double_p, _sz],
+    "rst_stager_next": [_vp, c_void_pp, c_void_pp, c_size_p],
     "rst_model_forward": [_vp, _dp, _sz, c_void_pp],
     "rst_model_loss": [_vp, _dp, c_double_p],
     "rst_model_backward": [_vp, _dp, _i32, c_void_pp],

@@ -67,12 +67,18 @@ struct rst_model {
   bool loss_grad_valid = false;
   bool grads_valid = false;
   // the captured training step (one graph launch instead of ~10 kernel launches)
+  // (a few graphs are kept: a staged input pipeline alternates between its slots' buffers)
   bool graph_enabled = true;
-  hipGraphExec_t graph_exec = nullptr;
-  const double* graph_x = nullptr;
-  const double* graph_truth = nullptr;
-  size_t graph_batch = 0;
-  double graph_lr = 0.0;
+  struct StepGraph {
+    hipGraphExec_t exec;
+    const double* x;
+    const double* truth;
+    size_t batch;
+    double lr;
+    unsigned long long last_use;
+  };
+  std::vector<StepGraph> graphs;
+  unsigned long long graph_clock = 0;
   // profiling
   bool profiling = false;
   bool slot_open = false;
@@ -83,9 +89,11 @@ struct rst_model {
 
 namespace {
 
+constexpr size_t kMaxStepGraphs = 8;
+
 void drop_graph(rst_model* m) {
-  if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
-  m->graph_exec = nullptr;
+  for (auto& g : m->graphs) (void)hipGraphExecDestroy(g.exec);
+  m->graphs.clear();
 }
 
 int free_activations(rst_model* m) {
@@ -439,6 +447,35 @@ int rst_model_parameter(rst_model* m, size_t index, double** parm, double** grad
   return fail(RST_ERR_INVALID_ARGUMENT, "parameter index %zu out of range (%zu tensors)", index, k);
 }
 
+static int transfer_parameters(rst_model* m, double* host_dst, const double* host_src, size_t count) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  RST_TRY(engine_activate(m->engine));
+  if (count != m->element_count)
+    return fail(RST_ERR_SHAPE, "the model has %zu parameters, the buffer holds %zu", m->element_count, count);
+  if (!host_dst && !host_src) return fail(RST_ERR_INVALID_ARGUMENT, "host buffer is null");
+  size_t off = 0;
+  for (auto& l : m->layers) {
+    if (l.kind != RST_LAYER_LINEAR) continue;
+    double* tensors[2] = {l.w, l.b};
+    size_t counts[2] = {l.in * l.out, l.out};
+    for (int t = 0; t < 2; ++t) {
+      if (host_dst) RST_TRY(rst_download(m->engine, host_dst + off, tensors[t], counts[t]));
+      else RST_TRY(rst_upload(m->engine, tensors[t], host_src + off, counts[t]));
+      off += counts[t];
+    }
+  }
+  return RST_OK;
+}
+
+int rst_model_export_parameters(rst_model* m, double* host_dst, size_t count) {
+  return transfer_parameters(m, host_dst, nullptr, count);
+}
+
+int rst_model_import_parameters(rst_model* m, const double* host_src, size_t count) {
+  if (!host_src) return fail(RST_ERR_INVALID_ARGUMENT, "host buffer is null");
+  return transfer_parameters(m, nullptr, host_src, count);
+}
+
 int rst_model_init_kaiming(rst_model* m, uint64_t seed, uint64_t first_stream) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
   RST_TRY(engine_activate(m->engine));
@@ -496,10 +533,10 @@ int run_step(rst_model* m, const double* x, const double* truth, size_t batch, d
 // Records the launches of one step into a graph.  Everything the step allocates lazily is
 // reserved first, because allocation is not allowed while the stream is capturing.  The graph
 // holds kernel nodes only (no memset nodes).
-int capture_step(rst_model* m, const double* x, const double* truth, size_t batch, double lr) {
+int capture_step(rst_model* m, const double* x, const double* truth, size_t batch, double lr,
+                 hipGraphExec_t* out) {
   rst_engine* e = m->engine;
-  drop_graph(m);
-  RST_TRY(reserve_activations(m, batch));
+  RST_TRY(reserve_activations(m, batch));  // drops every graph if the buffers move
   RST_TRY(engine_reserve_row_loss(e, batch));
   RST_HIP(hipStreamBeginCapture(e->stream, hipStreamCaptureModeThreadLocal));
   const int status = run_step(m, x, truth, batch, lr);
@@ -510,13 +547,19 @@ int capture_step(rst_model* m, const double* x, const double* truth, size_t batc
     return status;
   }
   if (end != hipSuccess) return fail_hip(end, "hipStreamEndCapture", __FILE__, __LINE__);
-  const hipError_t inst = hipGraphInstantiate(&m->graph_exec, graph, nullptr, nullptr, 0);
+  hipGraphExec_t exec = nullptr;
+  const hipError_t inst = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
   (void)hipGraphDestroy(graph);
-  if (inst != hipSuccess) {
-    m->graph_exec = nullptr;
-    return fail_hip(inst, "hipGraphInstantiate", __FILE__, __LINE__);
+  if (inst != hipSuccess) return fail_hip(inst, "hipGraphInstantiate", __FILE__, __LINE__);
+  if (m->graphs.size() >= kMaxStepGraphs) {  // evict the least recently used
+    size_t victim = 0;
+    for (size_t i = 1; i < m->graphs.size(); ++i)
+      if (m->graphs[i].last_use < m->graphs[victim].last_use) victim = i;
+    (void)hipGraphExecDestroy(m->graphs[victim].exec);
+    m->graphs.erase(m->graphs.begin() + victim);
   }
-  m->graph_x = x; m->graph_truth = truth; m->graph_batch = batch; m->graph_lr = lr;
+  m->graphs.push_back(rst_model::StepGraph{exec, x, truth, batch, lr, 0});
+  *out = exec;
   return RST_OK;
 }
 
@@ -532,10 +575,17 @@ int rst_model_train_step(rst_model* m, const double* x, const double* truth, siz
   if (!x || !truth) return fail(RST_ERR_INVALID_ARGUMENT, "x or truth is null");
   if (batch == 0) return fail(RST_ERR_SHAPE, "training step on an empty batch");
   if (m->graph_enabled && !m->profiling) {
-    const bool hit = m->graph_exec && m->graph_x == x && m->graph_truth == truth &&
-                     m->graph_batch == batch && m->graph_lr == lr;
-    if (!hit) RST_TRY(capture_step(m, x, truth, batch, lr));
-    RST_HIP(hipGraphLaunch(m->graph_exec, e->stream));
+    hipGraphExec_t exec = nullptr;
+    for (auto& g : m->graphs)
+      if (g.x == x && g.truth == truth && g.batch == batch && g.lr == lr) {
+        exec = g.exec;
+        g.last_use = ++m->graph_clock;
+      }
+    if (!exec) {
+      RST_TRY(capture_step(m, x, truth, batch, lr, &exec));
+      m->graphs.back().last_use = ++m->graph_clock;
+    }
+    RST_HIP(hipGraphLaunch(exec, e->stream));
     // the state the eager calls leave behind
     m->batch = batch;
     m->forward_valid = false;

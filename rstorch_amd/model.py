@@ -99,6 +99,35 @@ class DeviceModel:
         for (p, _), h in zip(params, host_arrays):
             p.assign(np.asarray(h, dtype=np.float64).reshape(p.shape))
 
+    def state(self):
+        """All parameters as one flat host array (reference order, no padding): a checkpoint."""
+        n = self.parameter_count()[1]
+        out = np.empty(n, dtype=np.float64)
+        _ffi.check(self.engine.lib.rst_model_export_parameters(
+            self.handle, out.ctypes.data_as(_ffi.c_double_p), n))
+        return out
+
+    def load_state(self, flat):
+        flat = np.ascontiguousarray(flat, dtype=np.float64).ravel()
+        _ffi.check(self.engine.lib.rst_model_import_parameters(
+            self.handle, flat.ctypes.data_as(_ffi.c_double_p), flat.size))
+
+    def save(self, path):
+        """Writes the layer list and the parameters to an .npz file (no pickled objects)."""
+        spec = np.array([[_KINDS[l[0]], l[1] if len(l) > 1 else 0, l[2] if len(l) > 2 else 0]
+                         for l in self.spec], dtype=np.int64)
+        np.savez(path, spec=spec, parameters=self.state())
+
+    @classmethod
+    def load(cls, path, engine=None):
+        names = {v: k for k, v in _KINDS.items()}
+        with np.load(path, allow_pickle=False) as f:
+            spec = [(names[int(k)],) if int(k) != _ffi.LAYER_LINEAR else ("linear", int(i), int(o))
+                    for k, i, o in f["spec"]]
+            dm = cls(spec, engine)
+            dm.load_state(f["parameters"])
+        return dm
+
     def init_kaiming(self, seed, first_stream=0):
         _ffi.check(self.engine.lib.rst_model_init_kaiming(self.handle, seed, first_stream))
 
@@ -191,3 +220,54 @@ class BasicModel:
 
     def predict(self, input):
         return self.device.forward(input)
+
+
+class BatchStager:
+    """Pipelines host batches into HBM (pinned double buffering on a copy stream); labels travel
+    as class indices and become dense one-hot rows on the device."""
+
+    def __init__(self, max_rows, x_cols, classes, depth=2, engine=None):
+        self.engine = engine or default_engine()
+        self.x_cols, self.classes = int(x_cols), int(classes)
+        h = ctypes.c_void_p()
+        _ffi.check(self.engine.lib.rst_stager_create(self.engine.handle, int(max_rows), self.x_cols,
+                                                     self.classes, int(depth), ctypes.byref(h)))
+        self.handle = h
+
+    def close(self):
+        if getattr(self, "handle", None) and self.engine.handle:
+            self.engine.lib.rst_stager_destroy(self.handle)
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def submit(self, x, labels=None, truth=None):
+        x = np.ascontiguousarray(x, dtype=np.float64)
+        if x.ndim != 2 or x.shape[1] != self.x_cols:
+            raise _ffi.ShapeError(_ffi.RST_ERR_SHAPE, "x %r does not have %d columns" % (x.shape, self.x_cols))
+        if labels is not None:
+            lab = np.ascontiguousarray(labels, dtype=np.uint32).ravel()
+            if lab.size != x.shape[0]:
+                raise _ffi.ShapeError(_ffi.RST_ERR_SHAPE, "%d labels for %d rows" % (lab.size, x.shape[0]))
+            _ffi.check(self.engine.lib.rst_stager_submit_labels(
+                self.handle, x.ctypes.data_as(_ffi.c_double_p),
+                lab.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32)), x.shape[0]))
+        else:
+            t = np.ascontiguousarray(truth, dtype=np.float64)
+            if t.shape != (x.shape[0], self.classes):
+                raise _ffi.ShapeError(_ffi.RST_ERR_SHAPE, "truth %r" % (t.shape,))
+            _ffi.check(self.engine.lib.rst_stager_submit_dense(
+                self.handle, x.ctypes.data_as(_ffi.c_double_p), t.ctypes.data_as(_ffi.c_double_p),
+                x.shape[0]))
+
+    def next(self):
+        """(x, truth) device arrays of the oldest submitted batch (borrowed from the stager)."""
+        xp, tp, rows = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_size_t()
+        _ffi.check(self.engine.lib.rst_stager_next(self.handle, ctypes.byref(xp), ctypes.byref(tp),
+                                                   ctypes.byref(rows)))
+        return (Array2(self.engine, rows.value, self.x_cols, ptr=xp.value, owner=self),
+                Array2(self.engine, rows.value, self.classes, ptr=tp.value, owner=self))
