@@ -146,6 +146,53 @@ def bench_small(rs, eng, spec, batch, normal, steps, warmup):
             "steps_per_s": steps / wall, "samples_per_s": steps / wall * batch, "final_loss": loss}
 
 
+def bench_staged(rs, eng, spec, batch, normal, steps, warmup, in_place=False):
+    """Same step, but every batch comes from host memory through the pinned double-buffered
+    stager (x as f64, labels as u32 expanded to one-hot rows on the device): the PCIe-inclusive
+    rate.  The host arrays are prepared once; the per-step host work is the copy into pinned
+    memory that rst_stager_submit_labels does."""
+    import numpy as np
+    dm = rs.DeviceModel(spec, eng)
+    dm.init_kaiming(SEED, 0)
+    n_in, n_out = dm.in_width, dm.out_width
+    rng = np.random.default_rng(SEED)
+    pool = [((rng.standard_normal((batch, n_in)) if normal else rng.random((batch, n_in))),
+             rng.integers(0, n_out, batch).astype(np.uint32)) for _ in range(2)]
+    st = rs.BatchStager(batch, n_in, n_out, depth=2, engine=eng)
+
+    def send(k):
+        if in_place:   # the loader writes straight into pinned memory (already there: no copy)
+            st.host_slot(batch)
+            st.commit(batch)
+        else:
+            st.submit(pool[k % 2][0], labels=pool[k % 2][1])
+
+    if in_place:       # fill both pinned slots once
+        for k in range(2):
+            hx, hl = st.host_slot(batch)
+            hx[...] = pool[k][0]; hl[...] = pool[k][1]
+            st.commit(batch); st.next()
+
+    def run(n):
+        send(0)
+        for k in range(n):
+            if k + 1 < n:
+                send(k + 1)
+            x, y = st.next()
+            dm.train_step(x, y, LR, want_loss=False)
+        eng.synchronize()
+
+    run(warmup)
+    t0 = time.perf_counter()
+    run(steps)
+    wall = time.perf_counter() - t0
+    loss = dm.last_loss()
+    st.close(); dm.close()
+    return {"batch": batch, "steps": steps, "ms_per_step": wall * 1e3 / steps,
+            "steps_per_s": steps / wall, "samples_per_s": steps / wall * batch,
+            "host_bytes_per_step": batch * (8 * n_in + 4), "final_loss": loss}
+
+
 def cpu_baseline(sample_batch=64):
     """The oracle (CPU restatement of the reference) on the C4 network at batch `sample_batch`.
     Contraction and loss time scale linearly with the batch, SGD does not, so
@@ -256,6 +303,12 @@ def main():
             "C0_readme_b32": bench_small(rs, eng, C01_SPEC, 32, False, 2000, 100),
             "C1_readme_b8192": bench_small(rs, eng, C01_SPEC, 8192, False, 200, 20),
             "C2_wide_b2048": bench_small(rs, eng, C2_SPEC, 2048, True, 20, 3),
+        }
+        log("host-fed (PCIe-inclusive) runs ...")
+        result["host_fed"] = {
+            "C1_readme_b8192": bench_staged(rs, eng, C01_SPEC, 8192, False, 100, 10),
+            "C1_readme_b8192_pinned_in_place": bench_staged(rs, eng, C01_SPEC, 8192, False, 100, 10, True),
+            "C4_deep_b1024": bench_staged(rs, eng, C4_SPEC, C4_BATCH, True, 10, 3),
         }
 
     if not args.no_cpu:

@@ -157,6 +157,12 @@ int rst_stager_destroy(rst_stager* stager);
  * RST_ERR_STATE when all slots are submitted and none has been taken with rst_stager_next. */
 int rst_stager_submit_labels(rst_stager* stager, const double* host_x, const uint32_t* host_labels,
                              size_t rows);
+/* The same in two halves, without the intermediate copy: rst_stager_acquire_host returns the
+ * pinned buffers of the next free slot (x: max_rows * x_cols doubles, labels: max_rows u32; it
+ * waits until the slot's previous transfer has left them) for the caller's loader to fill in
+ * place, rst_stager_commit_labels(rows) starts the transfer of what was written. */
+int rst_stager_acquire_host(rst_stager* stager, double** host_x, uint32_t** host_labels);
+int rst_stager_commit_labels(rst_stager* stager, size_t rows);
 /* Same with a dense (possibly soft-label) truth matrix [rows, classes]. */
 int rst_stager_submit_dense(rst_stager* stager, const double* host_x, const double* host_truth,
                             size_t rows);

@@ -100,6 +100,8 @@ SIGNATURES = {
     "rst_stager_submit_labels": [_vp, c_double_p, ctypes.POINTER(ctypes.c_uint32), _sz],
     "rst_stager_submit_dense": [_vp, c_double_p, c_double_p, _sz],
     "rst_stager_next": [_vp, c_void_pp, c_void_pp, c_size_p],
+    "rst_stager_acquire_host": [_vp, ctypes.POINTER(c_double_p), ctypes.POINTER(ctypes.POINTER(ctypes.c_uint32))],
+    "rst_stager_commit_labels": [_vp, _sz],
     "rst_model_forward": [_vp, _dp, _sz, c_void_pp],
     "rst_model_loss": [_vp, _dp, c_double_p],
     "rst_model_backward": [_vp, _dp, _i32, c_void_pp],

@@ -138,19 +138,42 @@ int rst_stager_destroy(rst_stager* s) {
   return RST_OK;
 }
 
+int rst_stager_acquire_host(rst_stager* s, double** host_x, uint32_t** host_labels);
+int rst_stager_commit_labels(rst_stager* s, size_t rows);
+
 int rst_stager_submit_labels(rst_stager* s, const double* host_x, const uint32_t* host_labels,
                              size_t rows) {
   if (!host_x || !host_labels) return fail(RST_ERR_INVALID_ARGUMENT, "null host batch");
-  if (s) {
-    for (size_t r = 0; r < rows && r < s->max_rows; ++r)
-      if (host_labels[r] >= s->classes)
-        return fail(RST_ERR_INVALID_ARGUMENT, "label %u of row %zu is not below %zu classes",
-                    host_labels[r], r, s->classes);
-  }
+  if (!s) return fail(RST_ERR_INVALID_ARGUMENT, "stager is null");
+  if (rows == 0 || rows > s->max_rows)
+    return fail(RST_ERR_SHAPE, "batch of %zu rows does not fit the stager (max %zu)", rows, s->max_rows);
+  double* px = nullptr;
+  uint32_t* pl = nullptr;
+  RST_TRY(rst_stager_acquire_host(s, &px, &pl));
+  std::memcpy(px, host_x, rows * s->x_cols * sizeof(double));
+  std::memcpy(pl, host_labels, rows * sizeof(uint32_t));
+  return rst_stager_commit_labels(s, rows);
+}
+
+int rst_stager_acquire_host(rst_stager* s, double** host_x, uint32_t** host_labels) {
+  if (!s) return fail(RST_ERR_INVALID_ARGUMENT, "stager is null");
+  RST_TRY(engine_activate(s->engine));
+  if (s->pending == s->slots.size())
+    return fail(RST_ERR_STATE, "all %zu slots are submitted and none has been taken", s->slots.size());
+  Slot& slot = s->slots[s->head];
+  if (slot.ever_used) RST_HIP(hipEventSynchronize(slot.copied));  // its last transfer has left
+  if (host_x) *host_x = slot.h_x;
+  if (host_labels) *host_labels = slot.h_labels;
+  return RST_OK;
+}
+
+int rst_stager_commit_labels(rst_stager* s, size_t rows) {
   Slot* slot = nullptr;
   RST_TRY(begin_submit(s, rows, &slot));
-  std::memcpy(slot->h_x, host_x, rows * s->x_cols * sizeof(double));
-  std::memcpy(slot->h_labels, host_labels, rows * sizeof(uint32_t));
+  for (size_t r = 0; r < rows; ++r)
+    if (slot->h_labels[r] >= s->classes)
+      return fail(RST_ERR_INVALID_ARGUMENT, "label %u of row %zu is not below %zu classes",
+                  slot->h_labels[r], r, s->classes);
   RST_HIP(hipMemcpyAsync(slot->d_x, slot->h_x, rows * s->x_cols * sizeof(double), hipMemcpyHostToDevice,
                          s->copy_stream));
   RST_HIP(hipMemcpyAsync(slot->d_labels, slot->h_labels, rows * sizeof(uint32_t), hipMemcpyHostToDevice,

@@ -264,6 +264,18 @@ class BatchStager:
                 self.handle, x.ctypes.data_as(_ffi.c_double_p), t.ctypes.data_as(_ffi.c_double_p),
                 x.shape[0]))
 
+    def host_slot(self, rows):
+        """numpy views (x [rows, x_cols], labels [rows]) onto the pinned memory of the next free
+        slot, to be filled in place and sent with ``commit(rows)``: no intermediate copy."""
+        px = _ffi.c_double_p()
+        pl = ctypes.POINTER(ctypes.c_uint32)()
+        _ffi.check(self.engine.lib.rst_stager_acquire_host(self.handle, ctypes.byref(px), ctypes.byref(pl)))
+        return (np.ctypeslib.as_array(px, shape=(rows, self.x_cols)),
+                np.ctypeslib.as_array(pl, shape=(rows,)))
+
+    def commit(self, rows):
+        _ffi.check(self.engine.lib.rst_stager_commit_labels(self.handle, int(rows)))
+
     def next(self):
         """(x, truth) device arrays of the oldest submitted batch (borrowed from the stager)."""
         xp, tp, rows = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_size_t()

@@ -73,6 +73,19 @@ def test_training_from_staged_inputs_equals_resident_inputs(engine, oracle):
         np.testing.assert_array_equal(p.to_numpy(), q.to_numpy())
 
 
+def test_fill_pinned_slot_in_place(engine):
+    import rstorch_amd as rs
+    st = rs.BatchStager(16, 5, 4, depth=2)
+    for k in range(5):
+        hx, hl = st.host_slot(12)
+        hx[...] = np.arange(60.0).reshape(12, 5) + k
+        hl[...] = np.arange(12) % 4
+        st.commit(12)
+        x, t = st.next()
+        np.testing.assert_array_equal(x.to_numpy(), np.arange(60.0).reshape(12, 5) + k)
+        np.testing.assert_array_equal(t.to_numpy(), np.eye(4)[np.arange(12) % 4])
+
+
 def test_checkpoint_round_trip(engine, oracle, tmp_path):
     import rstorch_amd as rs
     spec = [("identity",), ("linear", 13, 7), ("relu",), ("linear", 7, 5)]
