@@ -193,10 +193,10 @@ def bench_staged(rs, eng, spec, batch, normal, steps, warmup, in_place=False):
             "host_bytes_per_step": batch * (8 * n_in + 4), "final_loss": loss}
 
 
-def cpu_baseline(sample_batch=64):
-    """The oracle (CPU restatement of the reference) on the C4 network at batch `sample_batch`.
-    Contraction and loss time scale linearly with the batch, SGD does not, so
-    t(1024) = t_sgd + (1024 / sample_batch) * (t_step(sample_batch) - t_sgd)."""
+def cpu_baseline(sample_batches=(32, 96)):
+    """The oracle (CPU restatement of the reference) on the C4 network at two reduced batches.
+    A step costs t(B) = a + b*B (a: SGD and operand packing, independent of the batch; b: the
+    per-row contraction and loss work), so two timed steps give t(1024) = a + 1024*b."""
     import numpy as np
     import oracle
     oracle.build()
@@ -207,22 +207,25 @@ def cpu_baseline(sample_batch=64):
         if p.shape[0] > 1:
             a = np.sqrt(3.0 / p.shape[1])  # uniform with the variance of N(0, 1/fan_in)
             p[...] = oracle.fill_uniform(p.shape, SEED, i, -a, a)
-    x = oracle.fill_normal((sample_batch, 4096), SEED, 1000)
-    y = oracle.fill_one_hot(sample_batch, 32768, SEED, 1001)
+    b_lo, b_hi = sample_batches
+    data = {B: (oracle.fill_normal((B, 4096), SEED, 1000), oracle.fill_one_hot(B, 32768, SEED, 1001))
+            for B in sample_batches}
     out = {}
     for label, threads in (("single", 1), ("all", cores)):
         oracle.set_threads(threads)
-        if label == "all":
-            ref.train_step(x, y, LR)  # warm the thread pool
-        t0 = time.perf_counter(); ref.train_step(x, y, LR); t_step = time.perf_counter() - t0
-        t0 = time.perf_counter(); ref.sgd_step(LR); t_sgd = time.perf_counter() - t0
-        scale = C4_BATCH / float(sample_batch)
-        t_full = t_sgd + scale * max(t_step - t_sgd, 0.0)
-        out[label] = {"threads": threads, "t_step_sample_s": t_step, "t_sgd_s": t_sgd,
-                      "t_full_step_s": t_full, "steps_per_s": 1.0 / t_full}
+        ref.train_step(*data[b_lo], LR)  # allocates the activation buffers, warms the thread pool
+        times = {}
+        for B in (b_hi, b_lo):
+            t0 = time.perf_counter(); ref.train_step(*data[B], LR); times[B] = time.perf_counter() - t0
+        slope = (times[b_hi] - times[b_lo]) / float(b_hi - b_lo)
+        fixed = max(times[b_lo] - slope * b_lo, 0.0)
+        t_full = fixed + slope * C4_BATCH
+        out[label] = {"threads": threads, "t_step_s": {str(B): times[B] for B in sample_batches},
+                      "per_row_s": slope, "batch_independent_s": fixed, "t_full_step_s": t_full,
+                      "steps_per_s": 1.0 / t_full}
     oracle.set_threads(1)
     del ref
-    return out, sample_batch, cores
+    return out, sample_batches, cores
 
 
 def main():
@@ -313,12 +316,12 @@ def main():
 
     if not args.no_cpu:
         log("CPU baseline (oracle) ...")
-        cpu, sample_batch, cores = cpu_baseline()
+        cpu, sample_batches, cores = cpu_baseline()
         result["cpu_baseline"] = {
             "value": cpu["single"]["steps_per_s"], "unit": "steps/s", "cores": 1, "kind": "port",
             "sample": "oracle (C restatement of the reference, single thread like the reference) on "
-                      "the same C4 network at batch %d: one full step timed, contraction+loss time "
-                      "scaled x%d to batch 1024, SGD time added unscaled" % (sample_batch, C4_BATCH // sample_batch),
+                      "the same C4 network: one full step timed at batch %d and at batch %d, "
+                      "t(B) = a + b*B fitted and evaluated at batch 1024" % tuple(sample_batches),
             "detail": cpu["single"],
         }
         result["cpu_baseline_all_cores"] = {

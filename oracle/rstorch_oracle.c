@@ -115,30 +115,28 @@ static void pack_a(const double* a, size_t lda, int a_kc, size_t i0, size_t mc, 
   }
 }
 
+/* pack one NR-column panel of B */
 __attribute__((target_clones("fma", "default")))
-static void pack_b(const double* b, size_t ldb, int b_kc, size_t j0, size_t nc, size_t p0,
-                   size_t kc, double* dst) {
-  /* panels of NR columns: dst[panel][p][NR] */
-  for (size_t jp = 0; jp < nc; jp += NR) {
-    size_t nr = nc - jp < NR ? nc - jp : NR;
-    if (!b_kc) {
-      for (size_t p = 0; p < kc; ++p) {
-        const double* src = b + (p0 + p) * ldb + j0 + jp;
-        for (size_t j = 0; j < NR; ++j) dst[p * NR + j] = j < nr ? src[j] : 0.0;
-      }
-    } else {
-      for (size_t j = 0; j < NR; ++j) {
-        if (j < nr) {
-          const double* src = b + (j0 + jp + j) * ldb + p0;
-          for (size_t p = 0; p < kc; ++p) dst[p * NR + j] = src[p];
-        } else {
-          for (size_t p = 0; p < kc; ++p) dst[p * NR + j] = 0.0;
-        }
+static void pack_b_panel(const double* b, size_t ldb, int b_kc, size_t jcol, size_t nr, size_t p0,
+                         size_t kc, double* dst) {
+  if (!b_kc) {
+    for (size_t p = 0; p < kc; ++p) {
+      const double* src = b + (p0 + p) * ldb + jcol;
+      for (size_t j = 0; j < NR; ++j) dst[p * NR + j] = j < nr ? src[j] : 0.0;
+    }
+  } else {
+    for (size_t j = 0; j < NR; ++j) {
+      if (j < nr) {
+        const double* src = b + (jcol + j) * ldb + p0;
+        for (size_t p = 0; p < kc; ++p) dst[p * NR + j] = src[p];
+      } else {
+        for (size_t p = 0; p < kc; ++p) dst[p * NR + j] = 0.0;
       }
     }
-    dst += kc * NR;
   }
 }
+
+#define JCHUNK 16 /* NR-panels per task: 128 columns */
 
 static void gemm(const double* a, size_t lda, int a_kc, const double* b, size_t ldb, int b_kc,
                  double* c, size_t ldc, size_t m, size_t n, size_t k) {
@@ -150,30 +148,48 @@ static void gemm(const double* a, size_t lda, int a_kc, const double* b, size_t 
   double* bpack = (double*)xmalloc(sizeof(double) * KC * (NC + NR));
   for (size_t j0 = 0; j0 < n; j0 += NC) {
     size_t nc = n - j0 < NC ? n - j0 : NC;
+    long n_panels = (long)((nc + NR - 1) / NR);
     for (size_t p0 = 0; p0 < k; p0 += KC) {
       size_t kc = k - p0 < KC ? k - p0 : KC;
       int first = (p0 == 0);
-      pack_b(b, ldb, b_kc, j0, nc, p0, kc, bpack);
       long n_iblocks = (long)((m + MC - 1) / MC);
+      long n_jchunks = (n_panels + JCHUNK - 1) / JCHUNK;
+      /* The k order inside every output element is the same for any thread count: threads only
+       * split the (row block, column chunk) grid. */
 #ifdef _OPENMP
 #pragma omp parallel num_threads(g_threads) if (g_threads > 1)
 #endif
       {
         double* apack = (double*)xmalloc(sizeof(double) * KC * (MC + MR));
 #ifdef _OPENMP
+#pragma omp for schedule(static)
+#endif
+        for (long jp = 0; jp < n_panels; ++jp) {
+          size_t jcol = (size_t)jp * NR;
+          size_t nr = nc - jcol < NR ? nc - jcol : NR;
+          pack_b_panel(b, ldb, b_kc, j0 + jcol, nr, p0, kc, bpack + (size_t)jp * kc * NR);
+        }
+        long packed_ib = -1;
+#ifdef _OPENMP
 #pragma omp for schedule(dynamic, 1)
 #endif
-        for (long ib = 0; ib < n_iblocks; ++ib) {
+        for (long task = 0; task < n_iblocks * n_jchunks; ++task) {
+          long ib = task / n_jchunks, jc = task % n_jchunks;
           size_t i0 = (size_t)ib * MC;
           size_t mc = m - i0 < MC ? m - i0 : MC;
-          pack_a(a, lda, a_kc, i0, mc, p0, kc, apack);
-          for (size_t jp = 0; jp < nc; jp += NR) {
-            size_t nr = nc - jp < NR ? nc - jp : NR;
-            const double* bp = bpack + (jp / NR) * kc * NR;
+          if (packed_ib != ib) {
+            pack_a(a, lda, a_kc, i0, mc, p0, kc, apack);
+            packed_ib = ib;
+          }
+          long jp_end = (jc + 1) * JCHUNK < n_panels ? (jc + 1) * JCHUNK : n_panels;
+          for (long jp = jc * JCHUNK; jp < jp_end; ++jp) {
+            size_t jcol = (size_t)jp * NR;
+            size_t nr = nc - jcol < NR ? nc - jcol : NR;
+            const double* bp = bpack + (size_t)jp * kc * NR;
             for (size_t ip = 0; ip < mc; ip += MR) {
               size_t mr = mc - ip < MR ? mc - ip : MR;
               const double* ap = apack + (ip / MR) * kc * MR;
-              micro_kernel(kc, ap, bp, c + (i0 + ip) * ldc + j0 + jp, ldc, mr, nr, first);
+              micro_kernel(kc, ap, bp, c + (i0 + ip) * ldc + j0 + jcol, ldc, mr, nr, first);
             }
           }
         }

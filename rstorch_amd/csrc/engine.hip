@@ -97,7 +97,7 @@ int rst_engine_create(int device, rst_engine** out) {
   if (err == hipSuccess) err = hipMalloc(&e->d_loss, sizeof(double));
   if (err == hipSuccess) err = hipMalloc(&e->d_flags, 4 * sizeof(int));
   if (err == hipSuccess) err = hipMalloc(&e->d_hits, sizeof(unsigned long long));
-  e->gemm_ws_count = (size_t)4 << 20;  // 4 Mi doubles = 32 MiB
+  e->gemm_ws_count = (size_t)16 << 20;  // 16 Mi doubles = 128 MiB
   if (err == hipSuccess) err = hipMalloc(&e->d_gemm_ws, e->gemm_ws_count * sizeof(double));
   if (err == hipSuccess) err = hipHostMalloc(&e->h_loss, sizeof(double), hipHostMallocDefault);
   if (err == hipSuccess) err = hipHostMalloc(&e->h_flags, 4 * sizeof(int), hipHostMallocDefault);

@@ -390,10 +390,11 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
   __shared__ __attribute__((aligned(1024))) double lds_a[STAGES][A_SIZE];
   __shared__ __attribute__((aligned(1024))) double lds_b[STAGES][B_SIZE];
 
-  const int n_blocks = gridDim.x;
+  const int n_blocks = p.tiles_m * p.tiles_n;
+  const int split = blockIdx.x / n_blocks;  // K slice of this workgroup (0 without split-K)
   int logical;
   {
-    const int pid = blockIdx.x;
+    const int pid = blockIdx.x - split * n_blocks;
     const int xcd = pid & 7, local = pid >> 3;
     const int base = n_blocks >> 3, rem = n_blocks & 7;
     logical = xcd * base + (xcd < rem ? xcd : rem) + local;
@@ -451,7 +452,16 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
 
-  const int nk = p.K / BK;
+  // K steps of this workgroup: all of them, or slice `split` of a split contraction
+  const int nk_all = p.K / BK;
+  const int kt0 = split * p.steps_per_split;
+  const int nk = (p.split_k > 1) ? ((nk_all - kt0 < p.steps_per_split) ? nk_all - kt0 : p.steps_per_split)
+                                 : nk_all;
+#pragma unroll
+  for (int h = 0; h < CH; ++h) {
+    ga[h] += (long)kt0 * a_step;
+    gb[h] += (long)kt0 * b_step;
+  }
   auto issue = [&](int stage) {
 #pragma unroll
     for (int h = 0; h < CH; ++h) {
@@ -506,9 +516,24 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
     nxt = nxt + 1 == STAGES ? 0 : nxt + 1;
   }
   if (!A_KC) {
-    if (do_colsum) colsum_finish<BM, NW * 64>(colsum_partial, lds_b[0], tid, m0, 0, p);
+    if (do_colsum) colsum_finish<BM, NW * 64>(colsum_partial, lds_b[0], tid, m0, split, p);
   }
 
+  if (p.split_k > 1) {  // raw partial products of this K slice; the reduction applies the epilogue
+    double* __restrict__ out = p.ws + (size_t)split * p.M * p.N;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = n0 + wn * WN + j * 16 + lr;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = m0 + wm * WM + i * 16 + 4 * r + lk;
+          if (row < p.M && col < p.N) out[(size_t)row * p.N + col] = acc[i][j][r];
+        }
+      }
+    return;
+  }
 #pragma unroll
   for (int i = 0; i < TM; ++i) {
 #pragma unroll
@@ -536,19 +561,6 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
   }
 }
 
-template <bool A_KC, bool B_KC>
-int launch_dma(hipStream_t stream, GemmParams p) {
-  p.tiles_m = (p.M + 127) / 128;
-  p.tiles_n = (p.N + 127) / 128;
-  p.split_k = 1;
-  const long long blocks = (long long)p.tiles_m * p.tiles_n;
-  if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
-  hipLaunchKernelGGL((gemm_f64_mfma_dma<A_KC, B_KC, 2, 4, 2, 1>), dim3((unsigned)blocks),
-                     dim3(512), 0, stream, p);
-  RST_HIP(hipGetLastError());
-  return RST_OK;
-}
-
 // Adds the K slices of a split contraction in slice order and applies the epilogue.
 __global__ __launch_bounds__(256) void split_reduce_kernel(const GemmParams p) {
   const size_t mn = (size_t)p.M * p.N;
@@ -573,6 +585,41 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const GemmParams p) {
     for (int s = 0; s < p.split_k; ++s) t += p.ws_colsum[(size_t)s * p.M + i];
     p.colsum[i] = t / p.colsum_div;
   }
+}
+
+int launch_split_reduce(hipStream_t stream, const GemmParams& p) {
+  const size_t mn = (size_t)p.M * p.N;
+  hipLaunchKernelGGL(split_reduce_kernel, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, stream, p);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+template <bool A_KC, bool B_KC>
+int launch_dma(hipStream_t stream, GemmParams p) {
+  p.tiles_m = (p.M + 127) / 128;
+  p.tiles_n = (p.N + 127) / 128;
+  p.split_k = 1;
+  p.steps_per_split = p.K / BK;
+  long long blocks = (long long)p.tiles_m * p.tiles_n;
+  // One workgroup per compute unit runs at about 78 % of the MFMA peak whatever the prefetch
+  // depth, two independent ones at about 85 %: their barriers and LDS waits interleave.  With
+  // fewer than 512 tiles, cut K in two halves so that every CU gets two workgroups; the two
+  // partial products are added (in slice order) by split_reduce_kernel, which costs less than
+  // the gain once the contraction is long enough.
+  const int nk = p.K / BK;
+  const size_t need = 2 * ((size_t)p.M * p.N + (size_t)p.M);
+  if (blocks < 512 && nk >= 128 && p.ws != nullptr && p.ws_capacity >= need) {
+    p.split_k = 2;
+    p.steps_per_split = (nk + 1) / 2;
+    p.ws_colsum = p.ws + (size_t)2 * p.M * p.N;
+    blocks *= 2;
+  }
+  if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
+  hipLaunchKernelGGL((gemm_f64_mfma_dma<A_KC, B_KC, 2, 4, 2, 1>), dim3((unsigned)blocks),
+                     dim3(512), 0, stream, p);
+  RST_HIP(hipGetLastError());
+  if (p.split_k > 1) RST_TRY(launch_split_reduce(stream, p));
+  return RST_OK;
 }
 
 template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
@@ -602,11 +649,7 @@ int launch_one(hipStream_t stream, GemmParams p) {
   hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, WGM, WGN, A_KC, B_KC, VEC>), dim3((unsigned)blocks),
                      dim3(WGM * WGN * 64), 0, stream, p);
   RST_HIP(hipGetLastError());
-  if (p.split_k > 1) {
-    const size_t mn = (size_t)p.M * p.N;
-    hipLaunchKernelGGL(split_reduce_kernel, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, stream, p);
-    RST_HIP(hipGetLastError());
-  }
+  if (p.split_k > 1) RST_TRY(launch_split_reduce(stream, p));
   return RST_OK;
 }
 
