@@ -58,6 +58,11 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
   constexpr int BLOCK = TPR > 256 ? TPR : 256;
   constexpr int RPB = BLOCK / TPR;
   __shared__ double red[3][TPR > 64 ? TPR / 64 : 1];
+  // Widest rows only (one 1024-thread workgroup per row, so one workgroup per compute unit and
+  // nothing else to overlap with): the first PF truth vectors of every thread are fetched
+  // straight into LDS (16 bytes per lane, no registers) while the exponentials are computed.
+  constexpr int PF = (CE && VEC == 2 && TPR == 1024 && IPT == 16) ? 8 : 0;
+  __shared__ __attribute__((aligned(1024))) double tstage[PF ? PF * TPR * 2 : 2];
 
   const int sub = threadIdx.x % TPR;
   const size_t row = (size_t)blockIdx.x * RPB + threadIdx.x / TPR;
@@ -87,6 +92,18 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
       }
     }
   }
+  if (PF) {
+    // wavefront w, vector i -> 1 KiB at tstage[(w*PF + i)*128]; lane l lands 16*l bytes in
+    double* wave_base = tstage + (size_t)(threadIdx.x >> 6) * PF * 128;
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const size_t c = (size_t)(sub + i * TPR) * VEC;
+      if (row_ok && c < cols)
+        __builtin_amdgcn_global_load_lds(
+            (const __attribute__((address_space(1))) void*)(truth + base + c),
+            (__attribute__((address_space(3))) void*)(uintptr_t)(wave_base + i * 128), 16, 0, 0);
+    }
+  }
   mx = group_reduce<TPR, MaxOp>(mx, red[0]);
 
   double s = 0.0;
@@ -102,6 +119,11 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
     }
   }
   s = group_reduce<TPR, SumOp>(s, red[1]);
+  if (PF) {
+    // every direct-to-LDS load of this wavefront has landed before its slots are read
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    asm volatile("" ::: "memory");
+  }
 
   double lsum = 0.0;
 #pragma unroll
@@ -114,7 +136,12 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
     for (int e = 0; e < VEC; ++e) p[e] = x[i][e] / s;
     if (CE) {
       double t[VEC];
-      if (VEC == 2) {
+      if (PF && i < PF) {
+        const v2d tv = *reinterpret_cast<const v2d*>(
+            tstage + ((size_t)(threadIdx.x >> 6) * PF + i) * 128 + 2 * (threadIdx.x & 63));
+        t[0] = tv.x;
+        t[VEC - 1] = tv.y;
+      } else if (VEC == 2) {
         v2d tv = __builtin_nontemporal_load(reinterpret_cast<const v2d*>(truth + base + c));
         t[0] = tv.x;
         t[VEC - 1] = tv.y;
