@@ -105,6 +105,16 @@ int rst_relu_backward(rst_engine* engine, const double* grad, const double* x, d
 /* Returns RST_ERR_NAN when a logit is NaN (checked when the call returns: this call waits). */
 int rst_softmax_rows(rst_engine* engine, const double* x, double* out, size_t rows, size_t cols);
 
+/* The Softmax MODULE (src/module/activation/softmax.rs:55-78; not on the training path, which
+ * uses the free function through CrossEntropyLoss).  forward: softmax along `axis` (1: rows,
+ * 0: columns; Softmax::with_axis).  backward: ONE cols x cols matrix for the whole batch,
+ * jacobian = -(output^T . output) with each diagonal entry d replaced by d*(1-d), and
+ * grad_input = grad . jacobian - literally what the reference computes. */
+int rst_softmax_forward(rst_engine* engine, const double* x, double* out, size_t rows, size_t cols,
+                        int axis);
+int rst_softmax_backward(rst_engine* engine, const double* grad, const double* output,
+                         double* grad_input, size_t rows, size_t cols);
+
 /* ---- CrossEntropyLoss (src/loss/cross_entropy.rs:34-47) ---------------------------------- */
 /* One pass: prob = softmax(pred); loss = -(sum truth*ln(prob)) / rows; grad_out = prob - truth
  * (what `backward()` returns; NOT divided by rows).  prob_out may be NULL.  host_loss may be

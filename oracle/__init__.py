@@ -60,6 +60,7 @@ def lib():
         "rsto_relu_forward": (None, [dp, dp, sz]),
         "rsto_relu_backward": (None, [dp, dp, dp, sz]),
         "rsto_softmax": (i32, [dp, dp, sz, sz, i32]),
+        "rsto_softmax_module_backward": (None, [dp, dp, dp, dp, sz, sz]),
         "rsto_cross_entropy_forward": (i32, [dp, dp, dp, sz, sz, dp]),
         "rsto_cross_entropy_backward": (None, [dp, dp, dp, sz]),
         "rsto_sgd_step": (None, [dp, dp, sz, dbl]),
@@ -143,6 +144,16 @@ def softmax(x, axis=1):
     if lib().rsto_softmax(_ptr(x), _ptr(out), x.shape[0], x.shape[1], axis) != 0:
         raise NanLogits()
     return out
+
+
+def softmax_module_backward(grad, out):
+    grad, out = _as2d(grad), _as2d(out)
+    assert grad.shape == out.shape
+    gin = np.empty_like(out)
+    jac = np.empty((out.shape[1], out.shape[1]), dtype=np.float64)
+    lib().rsto_softmax_module_backward(_ptr(grad), _ptr(out), _ptr(gin), _ptr(jac), out.shape[0],
+                                       out.shape[1])
+    return gin
 
 
 def cross_entropy_forward(pred, truth):

@@ -316,6 +316,27 @@ int rsto_softmax(const double* x, double* out, size_t rows, size_t cols, int axi
   return 0;
 }
 
+/* src/module/activation/softmax.rs:62-73 (Softmax module backward).  One C x C matrix for the
+ * whole batch: jacobian = -(out^T . out); its diagonal entries d = (out^T . out)_ii become
+ * d * (1 - d); the result is gradient . jacobian.  `jac` is C*C scratch. */
+void rsto_softmax_module_backward(const double* grad, const double* out, double* grad_in,
+                                  double* jac, size_t rows, size_t cols) {
+  gemm(out, cols, 0, out, cols, 0, jac, cols, cols, cols, rows); /* out^T . out */
+  for (size_t i = 0; i < cols; ++i)
+    for (size_t j = 0; j < cols; ++j) {
+      double v = jac[i * cols + j];
+      if (i == j) {
+        double el = -v;       /* jacobian = -(...) */
+        el = -el;             /* softmax.rs:67  *el = -*el          */
+        el = el * (1.0 - el); /* softmax.rs:68  *el = *el * (1 - *el) */
+        jac[i * cols + j] = el;
+      } else {
+        jac[i * cols + j] = -v;
+      }
+    }
+  gemm(grad, cols, 1, jac, cols, 0, grad_in, cols, rows, cols, cols); /* gradient . jacobian */
+}
+
 /* src/loss/cross_entropy.rs:34-42.  ln of the probability (not a log-sum-exp form): a
  * probability that underflowed to 0 gives 0 * -inf = NaN when truth is 0 there, as in the
  * reference.  EPSILON (cross_entropy.rs:6) is unused by the reference and here. */

@@ -63,6 +63,12 @@ void rsto_relu_backward(const double* g, const double* x, double* out, size_t n)
  * Returns 0, or -1 if a NaN is met while taking the maximum (the reference panics there). */
 int rsto_softmax(const double* x, double* out, size_t rows, size_t cols, int axis);
 
+/* src/module/activation/softmax.rs:62-73 : the Softmax MODULE's backward (a "next" row, not on
+ * the training path): jacobian = -(out^T . out) with diagonal d -> d*(1-d), result = grad . jacobian.
+ * Pinned by the reference KAT (softmax.rs:105-113, tolerance 0.01) and an independent einsum. */
+void rsto_softmax_module_backward(const double* grad, const double* out, double* grad_in,
+                                  double* jac, size_t rows, size_t cols);
+
 /* src/loss/cross_entropy.rs:34-42 : prob = softmax(pred, axis 1);
  * loss = -(sum(truth * ln(prob))) / rows.  prob[rows,cols] is written (the reference caches it).
  * Returns 0, or -1 on NaN logits (reference panic). */

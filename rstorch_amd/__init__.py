@@ -12,13 +12,13 @@ from .init import FromArrays, InitParameters, KaimingNormal, Normal, XavierNorma
 from .loss import CrossEntropyLoss, Loss
 from .model import BasicModel, BatchStager, DeviceModel
 from .module import (Identity, Linear, Module, Parameter, Parameters, ReLU, Sequential,
-                     sequential)
+                     Softmax, sequential)
 from .optim import SGD, Optimizer
 from .utils import accuracy
 
 __all__ = [
     "Array2", "Engine", "as_array2", "default_engine",
-    "Module", "Parameter", "Parameters", "Identity", "Linear", "ReLU", "Sequential", "sequential",
+    "Module", "Parameter", "Parameters", "Identity", "Linear", "ReLU", "Softmax", "Sequential", "sequential",
     "Loss", "CrossEntropyLoss", "Optimizer", "SGD",
     "InitParameters", "KaimingNormal", "XavierNormal", "Normal", "FromArrays",
     "BasicModel", "DeviceModel", "BatchStager", "accuracy",

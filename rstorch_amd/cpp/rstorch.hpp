@@ -263,6 +263,36 @@ class ReLU : public Module {
   bool has_ = false;
 };
 
+// ---- Softmax: src/module/activation/softmax.rs:5-78 ---------------------------------------------
+class Softmax : public Module {
+ public:
+  Softmax() : axis_(1) {}
+  static Softmax with_axis(int axis) { Softmax s; s.axis_ = axis; return s; }
+  Array2 forward(Array2 input) override {
+    Array2 out(input.nrows(), input.ncols());
+    check(rst_softmax_forward(input.engine(), input.data(), out.data(), input.nrows(), input.ncols(), axis_));
+    output_ = out;
+    has_ = true;
+    return out.clone();  // softmax.rs:58-59 keeps the output and returns a clone
+  }
+  Array2 backward(Array2 gradient) override {
+    if (!has_) throw Panic(RST_ERR_STATE, "Softmax::backward without a forward");
+    has_ = false;
+    Array2 out = std::move(output_);
+    if (!out.same_shape(gradient)) throw Panic(RST_ERR_SHAPE, "Softmax: gradient shape");
+    Array2 gin(out.nrows(), out.ncols());
+    check(rst_softmax_backward(out.engine(), gradient.data(), out.data(), gin.data(), out.nrows(), out.ncols()));
+    return gin;
+  }
+  Parameters parameters() override { return Parameters(); }
+  std::string debug() const override { return "Softmax { axis: " + std::to_string(axis_) + " }"; }
+
+ private:
+  int axis_;
+  Array2 output_;
+  bool has_ = false;
+};
+
 // ---- Linear: src/module/linear.rs ---------------------------------------------------------------
 class Linear : public Module {
  public:

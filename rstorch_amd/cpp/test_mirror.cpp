@@ -57,6 +57,16 @@ int main() {
       EXPECT(array_eq(m.backward(Array2::ones(3, 2)), Array2{{1.0, 1.0}, {1.0, 0.0}, {0.0, 0.0}}));
       EXPECT(panics([&] { m.backward(Array2::ones(3, 2)); }));
     }
+    {  // softmax.rs:85-113
+      Softmax m;
+      auto out = m.forward(Array2{{1.0, 10.0}, {-3.0, 4.0}, {5.0, 6.0}}).to_host();
+      EXPECT(std::fabs(out[0] + out[1] - 1.0) < 1e-6 && out[0] + out[1] + out[2] + out[3] + out[4] + out[5] == 3.0);
+      Softmax b;
+      b.forward(Array2{{1.0, 2.0}, {3.0, 4.0}, {5.0, 6.0}});
+      EXPECT(array_eq(b.backward(Array2::ones(3, 2)), Array2{{-0.41, -1.55}, {-0.41, -1.55}, {-0.41, -1.55}}, 0.01));
+      auto col = Softmax::with_axis(0).forward(Array2{{1.0, 2.0}, {3.0, 4.0}, {5.0, 6.0}}).to_host();
+      EXPECT(col[0] + col[1] + col[2] + col[3] + col[4] + col[5] == 2.0);
+    }
     {  // identity.rs:35-51
       Identity m;
       Array2 d{{1.0, 2.0}, {3.0, 4.0}, {5.0, 6.0}};
@@ -73,8 +83,8 @@ int main() {
       EXPECT(linear.weight().to_host() == w0);
     }
     {  // sequential.rs:119-172 plus the container operations
-      Sequential module = sequential(Linear(3, 10), ReLU(), Linear(10, 100), ReLU(), Linear(100, 2));
-      EXPECT(module.len() == 5 && !module.is_empty());
+      Sequential module = sequential(Linear(3, 10), ReLU(), Linear(10, 100), ReLU(), Linear(100, 2), Softmax());
+      EXPECT(module.len() == 6 && !module.is_empty());
       Array2 out = module.forward(Array2{{1.0, 2.0, 3.0}, {-4.0, -5.0, -6.0}});
       EXPECT(out.nrows() == 2 && out.ncols() == 2);
       Array2 gin = module.backward(Array2{{1.0, 2.0}, {3.0, -4.0}});
@@ -83,7 +93,7 @@ int main() {
       EXPECT(module.remove(9) == nullptr);
       module.insert(0, Identity());
       module.push(ReLU());
-      EXPECT(module.len() == 7);
+      EXPECT(module.len() == 8);
       EXPECT(module.forward(Array2{{1.0, 2.0, 3.0}}).ncols() == 2);
     }
     {  // fused Sequential == layer-by-layer calls, bit for bit, and the loss/accuracy path

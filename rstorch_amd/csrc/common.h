@@ -98,6 +98,9 @@ int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* g
 int launch_softmax_rows(hipStream_t s, const double* z, const double* t, double* grad_out,
                         double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
                         size_t cols);
+int launch_softmax_columns(hipStream_t s, const double* z, double* out, int* flags, size_t rows,
+                           size_t cols);
+int launch_softmax_jacobian(hipStream_t s, double* jac, size_t cols);
 // hits[0] = number of rows whose first arg-max agrees
 int launch_accuracy(hipStream_t s, const double* pred, const double* truth, size_t rows,
                     size_t cols, unsigned long long* hits);

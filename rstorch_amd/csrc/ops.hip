@@ -125,6 +125,59 @@ int rst_softmax_rows(rst_engine* e, const double* x, double* out, size_t rows, s
   return RST_OK;
 }
 
+int rst_softmax_forward(rst_engine* e, const double* x, double* out, size_t rows, size_t cols,
+                        int axis) {
+  if (axis == 1) return rst_softmax_rows(e, x, out, rows, cols);
+  RST_TRY(engine_activate(e));
+  if (axis != 0) return fail(RST_ERR_INVALID_ARGUMENT, "softmax axis %d of a 2-D array", axis);
+  if (rows == 0 || cols == 0) return RST_OK;
+  if (!x || !out) return fail(RST_ERR_INVALID_ARGUMENT, "softmax_forward: null operand");
+  hipLaunchKernelGGL(reset_softmax_flag_kernel, dim3(1), dim3(1), 0, e->stream, e->d_flags);
+  RST_HIP(hipGetLastError());
+  RST_TRY(launch_softmax_columns(e->stream, x, out, e->d_flags, rows, cols));
+  RST_HIP(hipMemcpyAsync(e->h_flags, e->d_flags, 4 * sizeof(int), hipMemcpyDeviceToHost, e->stream));
+  RST_HIP(hipStreamSynchronize(e->stream));
+  if (e->h_flags[2] & 1)
+    return fail(RST_ERR_NAN, "softmax: NaN in the input (the reference panics in softmax.rs:38)");
+  return RST_OK;
+}
+
+int rst_softmax_backward(rst_engine* e, const double* grad, const double* output, double* grad_input,
+                         size_t rows, size_t cols) {
+  RST_TRY(engine_activate(e));
+  if (rows == 0 || cols == 0) return RST_OK;
+  if (!grad || !output || !grad_input)
+    return fail(RST_ERR_INVALID_ARGUMENT, "softmax_backward: null operand");
+  RST_TRY(check_dim(rows, "rows"));
+  RST_TRY(check_dim(cols, "cols"));
+  double* jac = nullptr;
+  RST_TRY(rst_malloc(e, cols * cols, &jac));
+  int status = RST_OK;
+  {  // jac[C,C] = output^T . output
+    GemmDesc d{};
+    d.A = output; d.B = output; d.C = jac;
+    d.M = (int)cols; d.N = (int)cols; d.K = (int)rows;
+    d.lda = (long)cols; d.ldb = (long)cols; d.ldc = (long)cols;
+    d.a_kc = false; d.b_kc = false;
+    d.epilogue = EPI_NONE;
+    d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
+    status = launch_gemm(e->stream, d);
+  }
+  if (status == RST_OK) status = launch_softmax_jacobian(e->stream, jac, cols);
+  if (status == RST_OK) {  // grad_input[B,C] = grad . jac
+    GemmDesc d{};
+    d.A = grad; d.B = jac; d.C = grad_input;
+    d.M = (int)rows; d.N = (int)cols; d.K = (int)cols;
+    d.lda = (long)cols; d.ldb = (long)cols; d.ldc = (long)cols;
+    d.a_kc = true; d.b_kc = false;
+    d.epilogue = EPI_NONE;
+    d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
+    status = launch_gemm(e->stream, d);
+  }
+  (void)rst_free(e, jac);  // stream-ordered reuse: the launches above are already enqueued
+  return status;
+}
+
 int rst_cross_entropy(rst_engine* e, const double* pred, const double* truth, double* grad_out,
                       double* prob_out, size_t rows, size_t cols, double* host_loss) {
   RST_TRY(engine_activate(e));

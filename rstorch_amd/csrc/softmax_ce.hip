@@ -237,6 +237,41 @@ __global__ __launch_bounds__(1024) void loss_reduce_kernel(const double* __restr
   }
 }
 
+// softmax down the columns (Softmax::with_axis(0), src/module/activation/softmax.rs:23-28):
+// one thread per column walks the rows three times; a rarely used orientation, kept simple.
+__global__ __launch_bounds__(256) void softmax_columns_kernel(const double* __restrict__ z,
+                                                             double* __restrict__ out,
+                                                             int* __restrict__ flags, size_t rows,
+                                                             size_t cols) {
+  const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= cols) return;
+  double mx = -DBL_MAX;
+  bool saw_nan = false;
+  for (size_t r = 0; r < rows; ++r) {
+    const double v = z[r * cols + c];
+    saw_nan |= (v != v);
+    mx = MaxOp::apply(mx, v);
+  }
+  double s = 0.0;
+  for (size_t r = 0; r < rows; ++r) {
+    const double e = exp(z[r * cols + c] - mx);
+    out[r * cols + c] = e;
+    s += e;
+  }
+  for (size_t r = 0; r < rows; ++r) out[r * cols + c] = out[r * cols + c] / s;
+  if (saw_nan) atomicOr(&flags[2], 1);
+}
+
+// jacobian fix-up of the Softmax module's backward (softmax.rs:64-69): off-diagonal entries of
+// out^T.out are negated, a diagonal entry d becomes d * (1 - d).
+__global__ __launch_bounds__(256) void softmax_jacobian_kernel(double* __restrict__ jac, size_t cols) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= cols * cols) return;
+  const size_t r = i / cols, c = i - r * cols;
+  const double v = jac[i];
+  jac[i] = (r == c) ? v * (1.0 - v) : -v;
+}
+
 template <int TPR, int IPT, int VEC>
 int launch_rows(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
                 double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce) {
@@ -288,6 +323,23 @@ int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* g
     hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(1024), 0, s, row_loss, loss, flags, rows);
     RST_HIP(hipGetLastError());
   }
+  return RST_OK;
+}
+
+int launch_softmax_columns(hipStream_t s, const double* z, double* out, int* flags, size_t rows,
+                           size_t cols) {
+  if (rows == 0 || cols == 0) return RST_OK;
+  hipLaunchKernelGGL(softmax_columns_kernel, dim3((unsigned)((cols + 255) / 256)), dim3(256), 0, s, z,
+                     out, flags, rows, cols);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
+int launch_softmax_jacobian(hipStream_t s, double* jac, size_t cols) {
+  if (cols == 0) return RST_OK;
+  hipLaunchKernelGGL(softmax_jacobian_kernel, dim3((unsigned)((cols * cols + 255) / 256)), dim3(256),
+                     0, s, jac, cols);
+  RST_HIP(hipGetLastError());
   return RST_OK;
 }
 

@@ -118,6 +118,46 @@ class ReLU(Module):
         return "ReLU"
 
 
+class Softmax(Module):
+    """src/module/activation/softmax.rs:5-78: softmax along an axis; the backward pass builds the
+    reference's single batch-summed Jacobian."""
+
+    def __init__(self, axis=1):
+        self.axis = int(axis)
+        self.output = None
+
+    @classmethod
+    def new(cls):
+        return cls(1)
+
+    @classmethod
+    def with_axis(cls, axis):
+        return cls(axis)
+
+    def forward(self, input):
+        x = as_array2(input)
+        out = x.engine.empty(x.rows, x.cols)
+        _ffi.check(x.engine.lib.rst_softmax_forward(x.engine.handle, x.ptr, out.ptr, x.rows, x.cols,
+                                                    self.axis))
+        self.output = out
+        return out.clone()  # the reference returns a clone and keeps the output (softmax.rs:58-59)
+
+    def backward(self, gradient):
+        if self.output is None:
+            raise _ffi.StateError(_ffi.RST_ERR_STATE, "Softmax.backward without a forward")
+        out, self.output = self.output, None  # take()
+        g = as_array2(gradient, out.engine)
+        if g.shape != out.shape:
+            raise _ffi.ShapeError(_ffi.RST_ERR_SHAPE, "gradient %r vs output %r" % (g.shape, out.shape))
+        gin = out.engine.empty(out.rows, out.cols)
+        _ffi.check(out.engine.lib.rst_softmax_backward(out.engine.handle, g.ptr, out.ptr, gin.ptr,
+                                                       out.rows, out.cols))
+        return gin
+
+    def __repr__(self):
+        return "Softmax(axis=%d)" % self.axis
+
+
 class Linear(Module):
     """src/module/linear.rs:8-79.  weight (out, in), bias (1, out)."""
 

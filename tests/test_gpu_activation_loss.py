@@ -118,6 +118,38 @@ def test_softmax_nan_is_an_error(engine):
     assert p[0, 1] == 0.0 and abs(p[0].sum() - 1.0) < 1e-15
 
 
+# ---- the Softmax module (forward on both axes, batch-summed Jacobian backward) -----------------
+def test_softmax_module_reference_known_answers(engine):
+    import rstorch_amd as rs
+    k1, k0 = KATS["softmax_axis1"], KATS["softmax_axis0"]
+    out = rs.Softmax.new().forward(np.array(k1["input"])).to_numpy()
+    assert np.all(np.abs(out.sum(axis=1) - 1.0) <= k1["row_sum_tolerance"]) and out.sum() == k1["total_exact"]
+    out = rs.Softmax.with_axis(0).forward(np.array(k0["input"])).to_numpy()
+    assert np.all(np.abs(out.sum(axis=0) - 1.0) <= k0["col_sum_tolerance"]) and out.sum() == k0["total_exact"]
+    kb = KATS["softmax_module_backward"]
+    m = rs.Softmax.new()
+    m.forward(np.array(kb["input"]))
+    got = m.backward(np.array(kb["gradient"])).to_numpy()
+    assert np.all(np.abs(got - np.array(kb["expected"])) <= kb["tolerance"])
+    with pytest.raises(rs.StateError):
+        m.backward(np.array(kb["gradient"]))
+
+
+@pytest.mark.parametrize("rows,cols,axis", [(3, 2, 1), (33, 11, 1), (64, 300, 1), (300, 64, 0), (7, 5, 0),
+                                            (512, 1000, 1)])
+def test_softmax_module_matches_oracle(engine, oracle, rows, cols, axis):
+    import rstorch_amd as rs
+    rng = np.random.default_rng(rows * 31 + cols + axis)
+    x = rng.standard_normal((rows, cols)) * 2
+    g = rng.standard_normal((rows, cols))
+    m = rs.Softmax.with_axis(axis)
+    out = m.forward(x).to_numpy()
+    want = oracle.softmax(x, axis=axis)
+    assert rel_err(out, want) <= TOL
+    gin = m.backward(g).to_numpy()
+    assert rel_err(gin, oracle.softmax_module_backward(g, want)) <= TOL
+
+
 # ---- CrossEntropyLoss ---------------------------------------------------------------------------
 @pytest.mark.parametrize("rows,cols", [(1, 2), (32, 10), (33, 11), (64, 100), (128, 1000),
                                        (16, 4096), (4, 32768), (3, 33000)])

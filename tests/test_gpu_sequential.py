@@ -132,14 +132,16 @@ def test_lr_one_instability_run_stays_matched(engine, oracle):
 def test_reference_sequential_cases(engine):
     """src/module/sequential.rs:119-172: both builder spellings; forward/backward run."""
     import rstorch_amd as rs
-    a = rs.sequential((rs.Linear, 3, 10), (rs.ReLU,), (rs.Linear, 10, 100), (rs.ReLU,), (rs.Linear, 100, 2))
+    a = rs.sequential((rs.Linear, 3, 10), (rs.ReLU,), (rs.Linear, 10, 100), (rs.ReLU,), (rs.Linear, 100, 2),
+                      (rs.Softmax,))
     b = rs.sequential(rs.Linear.new(3, 10), rs.ReLU.new(), rs.Linear.new(10, 100), rs.ReLU.new(),
-                      rs.Linear.new(100, 2))
+                      rs.Linear.new(100, 2), rs.Softmax.new())
     k = KATS["sequential"]
     for m in (a, b):
-        assert m.len() == 5 and not m.is_empty()
+        assert m.len() == 6 and not m.is_empty()
         out = m.forward(np.array(k["input"]))
         assert out.shape == (2, 2)
+        assert np.all(np.abs(out.to_numpy().sum(axis=1) - 1.0) <= 1e-15)
         gin = m.backward(np.array(k["backward_gradient"]))
         assert gin.shape == (2, 3)
         assert len(m.parameters()) == 6

@@ -58,13 +58,13 @@ def test_sgd_zero_gradient_kat():
 
 def test_sequential_kat_shapes():
     k = KATS["sequential"]
-    m = oracle.Model([tuple(l) for l in k["layers"]])
+    m = oracle.Model([tuple(l) for l in k["layers"] if l[0] != "softmax"])
     rng = np.random.default_rng(1)
     for p, _ in m.parameters():
         p[...] = rng.standard_normal(p.shape)
-    out = m.forward(np.array(k["input"]))
-    assert out.shape == (2, 2)
-    gin = m.backward(np.array(k["backward_gradient"]))
+    out = oracle.softmax(m.forward(np.array(k["input"])))  # the reference's net ends in Softmax
+    assert out.shape == (2, 2) and np.all(np.abs(out.sum(axis=1) - 1) < 1e-15)
+    gin = m.backward(oracle.softmax_module_backward(np.array(k["backward_gradient"]), out))
     assert gin.shape == (2, 3)
     shapes = [p.shape for p, _ in m.parameters()]
     assert shapes == [(10, 3), (1, 10), (100, 10), (1, 100), (2, 100), (1, 2)]  # weight, bias per layer
@@ -171,6 +171,21 @@ def test_softmax_invariants():
         oracle.softmax(np.array([[0.0, np.nan]]))
     y = np.array([[-np.inf, 0.0, 0.0]])
     np.testing.assert_array_equal(oracle.softmax(y), np.array([[0.0, 0.5, 0.5]]))
+
+
+def test_softmax_module_backward_kat_and_independent_form():
+    k = KATS["softmax_module_backward"]
+    out = oracle.softmax(k["input"])
+    got = oracle.softmax_module_backward(k["gradient"], out)
+    assert np.all(np.abs(got - np.array(k["expected"])) <= k["tolerance"])
+    # independent statement of softmax.rs:62-73: J = -(P^T P), J_ii = d (1 - d), result = G J
+    rng = np.random.default_rng(12)
+    p = oracle.softmax(rng.standard_normal((9, 5))); g = rng.standard_normal((9, 5))
+    ptp = np.einsum("bi,bj->ij", p, p)
+    jac = -ptp
+    d = np.diag(ptp)
+    jac[np.arange(5), np.arange(5)] = d * (1 - d)
+    np.testing.assert_allclose(oracle.softmax_module_backward(g, p), g @ jac, rtol=0, atol=1e-14)
 
 
 # ---- cross entropy (the reference has no test for it: closed forms only) ------------------------
