@@ -223,6 +223,12 @@ int rst_model_sgd_step(rst_model* model, double lr);
  * host_loss may be NULL: then the call returns without waiting for the GPU. */
 int rst_model_train_step(rst_model* model, const double* x, const double* truth, size_t batch,
                          double lr, double* host_loss);
+/* By default rst_model_train_step applies SGD::step inside the weight-gradient launches (each
+ * stores its gradient, then updates the parameter at the same index: parm - (lr * grad), two
+ * roundings, the same bits as the separate pass; the layer's input gradient, which needs the
+ * old weights, is launched first).  enabled == 0 runs the optimiser as its own pass over the
+ * parameter arena, as rst_model_sgd_step does. */
+int rst_model_fuse_sgd(rst_model* model, int enabled);
 /* rst_model_train_step records its launches into a HIP graph the first time it sees a given
  * (x, truth, batch, lr) and replays the graph afterwards; a different argument re-records.
  * enabled == 0 switches to plain launches (profiling does so by itself).  Default: enabled. */

@@ -111,6 +111,7 @@ SIGNATURES = {
     "rst_model_train_step": [_vp, _dp, _dp, _sz, _dbl, c_double_p],
     "rst_model_profile_enable": [_vp, _i32],
     "rst_model_graph_enable": [_vp, _i32],
+    "rst_model_fuse_sgd": [_vp, _i32],
     "rst_model_profile_read": [_vp, ctypes.POINTER(KernelRecord), _sz, c_size_p],
 }
 _SPECIAL = {

@@ -61,6 +61,11 @@ struct GemmDesc {
   // the bias gradient, computed by the workgroups of the first tile column.  NULL: not wanted.
   double* colsum;
   double colsum_div;
+  // only with EPI_DIVIDE (the fused training step): after the gradient is stored, the parameter
+  // at the same index gets parm -= lr * grad (two roundings); sgd_bias likewise next to colsum
+  double* sgd_parm;
+  double* sgd_bias;
+  double sgd_lr;
   // scratch for split-K partial products (small outputs with a long contraction); NULL: never split
   double* workspace;
   size_t workspace_count;

@@ -36,6 +36,11 @@ struct GemmParams {
   long ldmask;
   double* colsum;        // weight-gradient launches only: colsum[i] = (sum_k A(i,k)) / colsum_div
   double colsum_div;
+  // weight-gradient launches of the fused training step: once C = acc / divisor (and colsum) are
+  // stored, the SGD update parm -= lr * grad is applied to the parameter of the same index
+  double* sgd_parm;      // same shape and leading dimension as C, or NULL
+  double* sgd_bias;      // same shape as colsum, or NULL
+  double sgd_lr;
   int tiles_m, tiles_n;
   // split-K (small outputs with a long contraction): slice s of the K steps is multiplied by
   // workgroups [s*tiles, (s+1)*tiles) and lands, without epilogue, in ws[s][M][N] (and its
@@ -156,6 +161,13 @@ __device__ __forceinline__ double read_frag(const double* __restrict__ lds, int 
   return KC ? lds[e * S + (k ^ (e & 15))] : lds[k * S + e];
 }
 
+// parm - (lr * grad) with the product rounded before the subtraction (src/optim/sgd.rs:23)
+__device__ __forceinline__ double sgd_apply(double w, double g, double lr) {
+#pragma clang fp contract(off)
+  const double step = lr * g;
+  return w - step;
+}
+
 // Bias gradient inside the weight-gradient contraction (output-contiguous A = grad^T): the
 // workgroups of tile column 0 also add up their A tile over the contraction index.  Thread t
 // owns output row t % BM and every (THREADS/BM)-th contraction row; partial sums are combined
@@ -181,8 +193,13 @@ __device__ __forceinline__ void colsum_finish(double partial, double* __restrict
     double t = 0.0;
 #pragma unroll
     for (int g = 0; g < G; ++g) t += scratch[g * BM + e];
-    if (p.split_k > 1) p.ws_colsum[(size_t)split * p.M + m0 + e] = t;  // slice sum, reduced later
-    else p.colsum[m0 + e] = t / p.colsum_div;
+    if (p.split_k > 1) {
+      p.ws_colsum[(size_t)split * p.M + m0 + e] = t;  // slice sum, reduced later
+    } else {
+      const double g = t / p.colsum_div;
+      p.colsum[m0 + e] = g;
+      if (p.sgd_bias) p.sgd_bias[m0 + e] = sgd_apply(p.sgd_bias[m0 + e], g, p.sgd_lr);
+    }
   }
 }
 
@@ -333,6 +350,10 @@ __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm
           default: break;
         }
         p.C[(size_t)row * p.ldc + col] = v;
+        if (p.sgd_parm) {
+          double* w = p.sgd_parm + (size_t)row * p.ldc + col;
+          *w = sgd_apply(*w, v, p.sgd_lr);
+        }
       }
     }
   }
@@ -556,6 +577,10 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
           default: break;
         }
         p.C[(size_t)row * p.ldc + col] = v;
+        if (p.sgd_parm) {
+          double* w = p.sgd_parm + (size_t)row * p.ldc + col;
+          *w = sgd_apply(*w, v, p.sgd_lr);
+        }
       }
     }
   }
@@ -579,11 +604,17 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const GemmParams p) {
       default: break;
     }
     p.C[(size_t)row * p.ldc + col] = v;
+    if (p.sgd_parm) {
+      double* w = p.sgd_parm + (size_t)row * p.ldc + col;
+      *w = sgd_apply(*w, v, p.sgd_lr);
+    }
   }
   if (p.colsum != nullptr && i < (size_t)p.M) {
     double t = 0.0;
     for (int s = 0; s < p.split_k; ++s) t += p.ws_colsum[(size_t)s * p.M + i];
-    p.colsum[i] = t / p.colsum_div;
+    const double g = t / p.colsum_div;
+    p.colsum[i] = g;
+    if (p.sgd_bias) p.sgd_bias[i] = sgd_apply(p.sgd_bias[i], g, p.sgd_lr);
   }
 }
 
@@ -681,6 +712,9 @@ int launch_gemm(hipStream_t stream, const GemmDesc& d) {
   p.bias = d.bias; p.divisor = d.divisor; p.mask = d.mask; p.ldmask = d.ldmask;
   p.colsum = (!d.a_kc) ? d.colsum : nullptr;
   p.colsum_div = d.colsum_div;
+  p.sgd_parm = (d.epilogue == EPI_DIVIDE) ? d.sgd_parm : nullptr;
+  p.sgd_bias = p.colsum ? d.sgd_bias : nullptr;
+  p.sgd_lr = d.sgd_lr;
   p.split_k = 1; p.steps_per_split = 0;
   p.ws = d.workspace; p.ws_colsum = nullptr; p.ws_capacity = d.workspace ? d.workspace_count : 0;
   auto vec_ok = [](const double* ptr, long ld, int contiguous_extent) {

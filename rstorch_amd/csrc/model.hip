@@ -79,6 +79,8 @@ struct rst_model {
   };
   std::vector<StepGraph> graphs;
   unsigned long long graph_clock = 0;
+  // train_step applies the optimiser update inside the weight-gradient launches
+  bool fuse_sgd = true;
   // profiling
   bool profiling = false;
   bool slot_open = false;
@@ -235,7 +237,10 @@ int do_loss(rst_model* m, const double* truth, double* host_loss) {
   return RST_OK;
 }
 
-int do_backward(rst_model* m, const double* grad, int need_input_grad, const double** input_grad) {
+// fused_lr != NULL: every weight-gradient launch also applies the SGD update to its layer
+// (the input gradient, which needs the old weights, is launched first).
+int do_backward(rst_model* m, const double* grad, int need_input_grad, const double** input_grad,
+                const double* fused_lr) {
   rst_engine* e = m->engine;
   if (!m->forward_valid)
     return fail(RST_ERR_STATE, "backward without a forward (the reference panics on a consumed cache)");
@@ -263,8 +268,29 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
       cur = l.grad_in_buf;
       continue;
     }
-    // Linear: linear.rs:60-69
+    // Linear: linear.rs:60-69.  The input gradient goes first: it reads the weights, which the
+    // weight-gradient launch may update in place when the optimiser step is fused in.
     const double mnk = (double)batch * (double)l.in * (double)l.out;
+    const bool wanted = need_input_grad || i != first_linear;
+    const int pv = prev_non_identity(m, i);
+    const bool mask = pv >= 0 && m->layers[pv].kind == RST_LAYER_RELU;
+    if (wanted) {
+      GemmDesc d{};
+      d.A = cur; d.B = l.w; d.C = l.grad_in_buf;
+      d.M = (int)batch; d.N = (int)l.in; d.K = (int)l.out;
+      d.lda = (long)l.out; d.ldb = (long)l.in; d.ldc = (long)l.in;
+      d.a_kc = true; d.b_kc = false;
+      d.epilogue = mask ? EPI_MASK : EPI_NONE;
+      d.mask = mask ? l.input : nullptr;  // the ReLU's output is this layer's input
+      d.ldmask = (long)l.in;
+      const double bytes = 8.0 * ((double)batch * l.out + (double)l.in * l.out +
+                                  (double)batch * l.in * (mask ? 2.0 : 1.0));
+      RST_TRY(prof_begin(m, RST_KERNEL_GRAD_INPUT, i, 2.0 * mnk, bytes));
+      d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
+      RST_TRY(launch_gemm(e->stream, d));
+      RST_TRY(prof_end(m));
+      if (mask) m->layers[pv].backward_absorbed = true;
+    }
     {
       GemmDesc d{};
       d.A = cur; d.B = l.input; d.C = l.gw;
@@ -276,7 +302,13 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
       const bool fused_bias = l.in > 0 && batch > 0;
       d.colsum = fused_bias ? l.gb : nullptr;
       d.colsum_div = n_rows;
-      const double bytes = 8.0 * ((double)batch * l.out + (double)batch * l.in + (double)l.in * l.out);
+      if (fused_lr) {
+        d.sgd_parm = l.w;
+        d.sgd_bias = fused_bias ? l.b : nullptr;
+        d.sgd_lr = *fused_lr;
+      }
+      double bytes = 8.0 * ((double)batch * l.out + (double)batch * l.in + (double)l.in * l.out);
+      if (fused_lr) bytes += 16.0 * ((double)l.in * l.out + l.out);  // read and write the parameters
       RST_TRY(prof_begin(m, RST_KERNEL_GRAD_WEIGHT, i, 2.0 * mnk, bytes));
       d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
       RST_TRY(launch_gemm(e->stream, d));
@@ -285,28 +317,10 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
         RST_TRY(prof_begin(m, RST_KERNEL_GRAD_BIAS, i, 0.0, 8.0 * ((double)batch * l.out + l.out)));
         RST_TRY(launch_column_mean(e->stream, cur, l.gb, batch, l.out, n_rows));
         RST_TRY(prof_end(m));
+        if (fused_lr) RST_TRY(launch_sgd_flat(e->stream, l.b, l.gb, l.out, *fused_lr));
       }
     }
-
-    const bool wanted = need_input_grad || i != first_linear;
     if (!wanted) { cur = nullptr; break; }
-    const int pv = prev_non_identity(m, i);
-    const bool mask = pv >= 0 && m->layers[pv].kind == RST_LAYER_RELU;
-    GemmDesc d{};
-    d.A = cur; d.B = l.w; d.C = l.grad_in_buf;
-    d.M = (int)batch; d.N = (int)l.in; d.K = (int)l.out;
-    d.lda = (long)l.out; d.ldb = (long)l.in; d.ldc = (long)l.in;
-    d.a_kc = true; d.b_kc = false;
-    d.epilogue = mask ? EPI_MASK : EPI_NONE;
-    d.mask = mask ? l.input : nullptr;  // the ReLU's output is this layer's input
-    d.ldmask = (long)l.in;
-    const double bytes = 8.0 * ((double)batch * l.out + (double)l.in * l.out +
-                                (double)batch * l.in * (mask ? 2.0 : 1.0));
-    RST_TRY(prof_begin(m, RST_KERNEL_GRAD_INPUT, i, 2.0 * mnk, bytes));
-    d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
-      RST_TRY(launch_gemm(e->stream, d));
-    RST_TRY(prof_end(m));
-    if (mask) m->layers[pv].backward_absorbed = true;
     cur = l.grad_in_buf;
   }
   if (input_grad) *input_grad = cur;
@@ -509,7 +523,7 @@ int rst_model_backward(rst_model* m, const double* grad, int need_input_grad,
                        const double** input_grad) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
   RST_TRY(engine_activate(m->engine));
-  return do_backward(m, grad, need_input_grad, input_grad);
+  return do_backward(m, grad, need_input_grad, input_grad, nullptr);
 }
 
 int rst_model_sgd_step(rst_model* m, double lr) {
@@ -525,8 +539,12 @@ namespace {
 int run_step(rst_model* m, const double* x, const double* truth, size_t batch, double lr) {
   RST_TRY(do_forward(m, x, batch));
   RST_TRY(do_loss(m, truth, nullptr));
-  RST_TRY(do_backward(m, nullptr, 0, nullptr));
-  RST_TRY(do_sgd(m, lr));
+  if (m->fuse_sgd) {  // SGD::step rides in the epilogues of the weight-gradient launches
+    RST_TRY(do_backward(m, nullptr, 0, nullptr, &lr));
+  } else {
+    RST_TRY(do_backward(m, nullptr, 0, nullptr, nullptr));
+    RST_TRY(do_sgd(m, lr));
+  }
   return RST_OK;
 }
 
@@ -596,6 +614,13 @@ int rst_model_train_step(rst_model* m, const double* x, const double* truth, siz
     RST_TRY(run_step(m, x, truth, batch, lr));
   }
   if (host_loss) return rst_loss_value(e, host_loss);
+  return RST_OK;
+}
+
+int rst_model_fuse_sgd(rst_model* m, int enabled) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->fuse_sgd = enabled != 0;
+  drop_graph(m);
   return RST_OK;
 }
 

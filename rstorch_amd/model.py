@@ -186,6 +186,10 @@ class DeviceModel:
         _ffi.check(self.engine.lib.rst_loss_value(self.engine.handle, ctypes.byref(v)))
         return v.value
 
+    def fuse_sgd(self, on=True):
+        """Apply SGD inside the weight-gradient launches of train_step (default) or as a pass."""
+        _ffi.check(self.engine.lib.rst_model_fuse_sgd(self.handle, 1 if on else 0))
+
     def graph_enable(self, on=True):
         """Replay the step as a HIP graph (default) or launch its kernels one by one."""
         _ffi.check(self.engine.lib.rst_model_graph_enable(self.handle, 1 if on else 0))

@@ -135,9 +135,13 @@ def test_profile_records_cover_every_launch(engine, oracle):
     kinds = [r["kernel"] for r in recs]
     assert kinds.count("linear_forward") == 3 and kinds.count("grad_weight") == 3
     assert kinds.count("grad_input") == 2      # the first layer's input gradient is skipped
-    assert kinds.count("cross_entropy") == 1 and kinds.count("sgd") == 1
+    # the optimiser rides in the weight-gradient launches unless asked to be a pass of its own
+    assert kinds.count("cross_entropy") == 1 and kinds.count("sgd") == 0
     assert "relu_forward" not in kinds and "relu_backward" not in kinds  # fused away
     assert all(r["ms"] > 0 for r in recs)
+    dm.fuse_sgd(False)
+    dm.train_step(x, y, 0.01)
+    assert [r["kernel"] for r in dm.profile_read()].count("sgd") == 1
     dm.profile_enable(False)
 
 
@@ -167,3 +171,40 @@ def test_graph_replay_equals_eager_launches(engine, oracle):
     with pytest.raises(rs.StateError):
         g.backward(None)
     g.sgd_step(0.0)  # gradients exist
+
+
+FUSE_CASES = [
+    # tiny outputs (split-K with the ordered reduction), ragged tiles, a 128x128-tile problem that
+    # takes the two-way split, and one that fills the chip without a split
+    ("readme_b32", README_MLP, 32),
+    ("readme_b4096", README_MLP, 4096),
+    ("ragged", [("identity",), ("linear", 33, 65), ("relu",), ("identity",), ("linear", 65, 129),
+                ("relu",), ("linear", 129, 7)], 67),
+    ("two_way_split", [("linear", 2048, 2048), ("relu",), ("linear", 2048, 2560)], 2048),
+    ("full_grid", [("linear", 1024, 4096), ("relu",), ("linear", 4096, 4096), ("relu",),
+                   ("linear", 4096, 1000)], 512),
+]
+
+
+@pytest.mark.parametrize("name,spec,batch", FUSE_CASES, ids=[c[0] for c in FUSE_CASES])
+@pytest.mark.parametrize("graph", [False, True], ids=["eager", "graph"])
+def test_sgd_in_weight_gradient_epilogue_is_bit_identical(engine, oracle, name, spec, batch, graph):
+    """train_step with the optimiser inside the weight-gradient launches against the same step
+    with SGD as its own pass: losses, parameters and gradients must agree to the bit."""
+    import rstorch_amd as rs
+    weights = make_weights(oracle, spec, 77)
+    models = []
+    for fused in (True, False):
+        dm = rs.DeviceModel(spec)
+        dm.load_parameters(weights)
+        dm.fuse_sgd(fused)
+        dm.graph_enable(graph)
+        models.append(dm)
+    x, y = batch_data(oracle, batch, models[0].in_width, models[0].out_width, 3, 0, True)
+    xd, yd = engine.from_numpy(x), engine.from_numpy(y)
+    for step in range(3):
+        losses = [dm.train_step(xd, yd, 0.05) for dm in models]
+        assert losses[0] == losses[1], "step %d" % step
+        for (p, g), (q, h) in zip(models[0].parameters(), models[1].parameters()):
+            assert np.array_equal(p.to_numpy(), q.to_numpy()), "step %d" % step
+            assert np.array_equal(g.to_numpy(), h.to_numpy()), "step %d" % step
