@@ -503,38 +503,79 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
   double colsum_partial = 0.0;
 
   int cur = 0, nxt = DIST % STAGES;
+  // Fragment registers are double-buffered by hand: the LDS reads of step ks+1 are issued
+  // before the matrix cores start on step ks, and the reads of the next tile's first step are
+  // issued right after the barrier, under the last MFMAs of the current tile.  The reads are
+  // inline assembly so that their place in the instruction stream is fixed; the waits carry
+  // the fragment registers as operands, which keeps every MFMA behind the wait that covers it.
+  static_assert(TM == 4 && TN == 2, "fragment reads below are written for 64x32 wave tiles");
+  uint32_t a_off[BK / 4], b_off[BK / 4];  // byte offsets inside a stage
+#pragma unroll
+  for (int ks = 0; ks < BK / 4; ++ks) {
+    const int k = ks * 4 + lk;
+    a_off[ks] = 8u * (A_KC ? (uint32_t)((wm * WM + lr) * BK + 2 * ((k >> 1) ^ ((lr >> 1) & 7)) + (k & 1))
+                           : (uint32_t)(k * (BM + 16) + wm * WM + lr));
+    b_off[ks] = 8u * (B_KC ? (uint32_t)((wn * WN + lr) * BK + 2 * ((k >> 1) ^ ((lr >> 1) & 7)) + (k & 1))
+                           : (uint32_t)(k * (BN + 16) + wn * WN + lr));
+  }
+  const uint32_t a_base = (uint32_t)(uintptr_t)&lds_a[0][0], b_base = (uint32_t)(uintptr_t)&lds_b[0][0];
+  v2d fa0[2], fa1[2], fb0[2];  // [buffer]: A fragments 0-1, 2-3, B fragments 0-1
+  auto read_frags = [&](int buf, int stage, int ks) {
+    const uint32_t aa = a_base + (uint32_t)stage * (A_SIZE * 8) + a_off[ks];
+    const uint32_t bb = b_base + (uint32_t)stage * (B_SIZE * 8) + b_off[ks];
+    if constexpr (A_KC) {
+      asm volatile("ds_read2st64_b64 %0, %2 offset1:4\n\tds_read2st64_b64 %1, %2 offset0:8 offset1:12"
+                   : "=&v"(fa0[buf]), "=&v"(fa1[buf]) : "v"(aa) : "memory");
+    } else {
+      asm volatile("ds_read2_b64 %0, %2 offset1:16\n\tds_read2_b64 %1, %2 offset0:32 offset1:48"
+                   : "=&v"(fa0[buf]), "=&v"(fa1[buf]) : "v"(aa) : "memory");
+    }
+    if constexpr (B_KC) {
+      asm volatile("ds_read2st64_b64 %0, %1 offset1:4" : "=&v"(fb0[buf]) : "v"(bb) : "memory");
+    } else {
+      asm volatile("ds_read2_b64 %0, %1 offset1:16" : "=&v"(fb0[buf]) : "v"(bb) : "memory");
+    }
+  };
+  // wait until only the `pending` youngest LDS reads are outstanding
+  auto wait_frags3 = [&](int buf) {
+    asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(fa0[buf]), "+v"(fa1[buf]), "+v"(fb0[buf]));
+  };
+  auto wait_frags0 = [&](int buf) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa0[buf]), "+v"(fa1[buf]), "+v"(fb0[buf]));
+  };
+  auto mfmas = [&](int buf) {
+    const double a[4] = {fa0[buf].x, fa0[buf].y, fa1[buf].x, fa1[buf].y};
+    const double b[2] = {fb0[buf].x, fb0[buf].y};
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
+  };
+  if (nk > 0) read_frags(0, 0, 0);
   for (int kt = 0; kt < nk; ++kt) {
     if (kt + DIST < nk) issue(nxt);
-    const double* __restrict__ sa = lds_a[cur];
-    const double* __restrict__ sb = lds_b[cur];
     if (!A_KC) {
-      if (do_colsum) colsum_accumulate<BM, NW * 64>(colsum_partial, sa, tid);
+      if (do_colsum) colsum_accumulate<BM, NW * 64>(colsum_partial, lds_a[cur], tid);
     }
-#pragma unroll
-    for (int ks = 0; ks < BK / 4; ++ks) {
-      double fa[TM], fb[TN];
-#pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const int e = wm * WM + i * 16 + lr, k = ks * 4 + lk;
-        fa[i] = A_KC ? read_frag_kc16(sa, e, k) : sa[k * (BM + 16) + e];
-      }
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int e = wn * WN + j * 16 + lr, k = ks * 4 + lk;
-        fb[j] = B_KC ? read_frag_kc16(sb, e, k) : sb[k * (BN + 16) + e];
-      }
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[i], fb[j], acc[i][j], 0, 0, 0);
-    }
+    read_frags(1, cur, 1);
+    wait_frags3(0);
+    mfmas(0);
+    read_frags(0, cur, 2);
+    wait_frags3(1);
+    mfmas(1);
+    read_frags(1, cur, 3);
+    wait_frags3(0);
+    mfmas(0);
+    __builtin_amdgcn_sched_barrier(0);
     // tile kt+1 must have landed: at most DIST-1 younger tiles may still be in flight
     if (kt + DIST < nk) wait_vmcnt((DIST - 1) * 2 * CH); else wait_vmcnt(0);
-    __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wave's LDS reads of `cur` are done
+    wait_frags0(1);  // this wave's LDS reads of `cur` are done
     __builtin_amdgcn_s_barrier();
     cur = cur + 1 == STAGES ? 0 : cur + 1;
     nxt = nxt + 1 == STAGES ? 0 : nxt + 1;
+    if (kt + 1 < nk) read_frags(0, cur, 0);
+    mfmas(1);
   }
   if (!A_KC) {
     if (do_colsum) colsum_finish<BM, NW * 64>(colsum_partial, lds_b[0], tid, m0, split, p);
