@@ -67,15 +67,21 @@ def time_steps(eng, dm, x, y, steps, warmup, profile):
     eng.synchronize()
     if profile:
         dm.profile_enable(True)
-    ev0, ev1 = eng.event(), eng.event()
+    # the profiled (headline) run also marks every step, for the median and minimum step time
+    marks = [eng.event() for _ in range(steps + 1 if profile else 2)]
     t0 = time.perf_counter()
-    ev0.record()
-    for _ in range(steps):
+    marks[0].record()
+    for i in range(steps):
         dm.train_step(x, y, LR, want_loss=False)
-    ev1.record()
+        if profile:
+            marks[i + 1].record()
+    if not profile:
+        marks[1].record()
     eng.synchronize()
     wall = time.perf_counter() - t0
-    dev_ms = ev0.elapsed_ms(ev1)
+    dev_ms = marks[0].elapsed_ms(marks[-1])
+    if profile:
+        time_steps.per_step_ms = sorted(marks[i].elapsed_ms(marks[i + 1]) for i in range(steps))
     loss = dm.last_loss()
     recs = dm.profile_read() if profile else []
     if profile:
@@ -233,10 +239,12 @@ def cpu_baseline(sample_batches=(32, 96)):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
+    ap.add_argument("--sgd-only", action="store_true",
+                    help="time only SGD::step over the configs[3] parameter set (for profiler runs)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one streaming ReLU over 1 GiB (reads 1 GiB, writes 1 GiB): the "
                          "known-size kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE are scaled by")
@@ -249,6 +257,10 @@ def main():
     eng = rs.default_engine()
     info = eng.device_info()
     log("device: %s, %d CUs" % (info["name"], info["compute_units"]))
+
+    if args.sgd_only:
+        print(json.dumps({"sgd_c3": bench_sgd_c3(rs, eng)}), flush=True)
+        return
 
     if args.calibration_copy:
         from rstorch_amd import _ffi
@@ -263,6 +275,7 @@ def main():
     tensors, params = dm.parameter_count()
     wall, dev_ms, loss, recs = time_steps(eng, dm, x, y, args.steps, args.warmup, True)
     ms_per_step = wall * 1e3 / args.steps
+    per_step = time_steps.per_step_ms
     kernels = summarise(recs, args.steps)
     dm.close()
     log("C4: %.3f ms/step, loss %.6f" % (ms_per_step, loss))
@@ -294,6 +307,8 @@ def main():
                                "batch 1024, CrossEntropyLoss, SGD lr=0.01 (BASELINE.json configs[4])",
                    "batch": C4_BATCH, "parameters": params, "samples_per_s": args.steps / wall * C4_BATCH,
                    "device": info["name"], "device_ms_per_step": dev_ms / args.steps,
+                   "device_ms_per_step_median": per_step[len(per_step) // 2],
+                   "device_ms_per_step_min": per_step[0],
                    "final_loss": loss, "per_launch_events": True},
         "roofline": roofline,
         "contractions": all_gemm,
