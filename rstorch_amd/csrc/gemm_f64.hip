@@ -365,8 +365,10 @@ __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm
 // base + 16*l), so no staging registers and no ds_write instructions are spent on the operand
 // tiles; a wavefront moves one 1 KiB chunk of a tile per instruction:
 //   contraction-contiguous operand: a chunk is 8 rows x 16 doubles; lane l fetches, for row
-//       l/8, the pair k = 2*((l%8) ^ ((row>>1)&7)), i.e. the XOR swizzle is applied by choosing
-//       the global address, and fragment reads undo it (read_frag_kc16);
+//       l/8, the pair k = 2*((l%8) ^ (row&7)), i.e. the XOR swizzle is applied by choosing the
+//       global address; a fragment read takes the whole 16-byte slot (ds_read_b128), and with
+//       this swizzle any eight consecutive lanes (eight rows, one pair) hit eight different
+//       slots: SQ_LDS_BANK_CONFLICT reads 0;
 //   output-contiguous operand: a chunk is one k row of 128 doubles; rows sit 144 doubles apart.
 // STAGES LDS stages form a ring, tile kt+DIST is requested while tile kt is multiplied; the
 // wait before the barrier only covers the tile needed next.
@@ -377,13 +379,6 @@ __device__ __forceinline__ void dma16(const double* g, double* lds_wave_base) {
   // every lane moves 16 bytes; lane l lands at lds_wave_base + 16*l
   __builtin_amdgcn_global_load_lds((gbl_ptr_t)g, (lds_ptr_t)(uintptr_t)lds_wave_base, 16, 0, 0);
 }
-
-// contraction-contiguous tile for DMA: [EXT][16], 16-byte slot j of row e holds the pair
-// k = 2*(j ^ ((e >> 1) & 7)), unswapped.
-__device__ __forceinline__ double read_frag_kc16(const double* __restrict__ lds, int e, int k) {
-  return lds[e * BK + 2 * ((k >> 1) ^ ((e >> 1) & 7)) + (k & 1)];
-}
-
 
 __device__ __forceinline__ void wait_vmcnt(int n) {
   // s_waitcnt with only the vector-memory counter constrained (gfx9 encoding)
@@ -397,6 +392,25 @@ __device__ __forceinline__ void wait_vmcnt(int n) {
     case 8: __builtin_amdgcn_s_waitcnt(0x0F70 | 8); break;
     case 12: __builtin_amdgcn_s_waitcnt(0x0F70 | 12); break;
     default: __builtin_amdgcn_s_waitcnt(0x0F70 | 0); break;
+  }
+}
+
+// One fragment of one pair of K steps: 16 bytes per lane, .x feeds the first step, .y the second.
+//   contraction-contiguous tile: the 16-byte slot (k, k+1) of row I*16 + lr -> one ds_read_b128;
+//   output-contiguous tile: column I*16 + lr of k rows k and k+1 (144 doubles apart) -> ds_read2_b64.
+template <bool KC, int I>
+__device__ __forceinline__ void read_quad(v2d& q, uint32_t addr) {
+  static_assert(I >= 0 && I < 4, "four fragments at most");
+  if constexpr (KC) {
+    if constexpr (I == 0) asm volatile("ds_read_b128 %0, %1" : "=v"(q) : "v"(addr) : "memory");
+    if constexpr (I == 1) asm volatile("ds_read_b128 %0, %1 offset:2048" : "=v"(q) : "v"(addr) : "memory");
+    if constexpr (I == 2) asm volatile("ds_read_b128 %0, %1 offset:4096" : "=v"(q) : "v"(addr) : "memory");
+    if constexpr (I == 3) asm volatile("ds_read_b128 %0, %1 offset:6144" : "=v"(q) : "v"(addr) : "memory");
+  } else {
+    if constexpr (I == 0) asm volatile("ds_read2_b64 %0, %1 offset1:144" : "=v"(q) : "v"(addr) : "memory");
+    if constexpr (I == 1) asm volatile("ds_read2_b64 %0, %1 offset0:16 offset1:160" : "=v"(q) : "v"(addr) : "memory");
+    if constexpr (I == 2) asm volatile("ds_read2_b64 %0, %1 offset0:32 offset1:176" : "=v"(q) : "v"(addr) : "memory");
+    if constexpr (I == 3) asm volatile("ds_read2_b64 %0, %1 offset0:48 offset1:192" : "=v"(q) : "v"(addr) : "memory");
   }
 }
 
@@ -446,7 +460,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
     if (A_KC) {
       const int row = 8 * c + (lane >> 3);
       int gr = m0 + row; gr = gr < p.M ? gr : p.M - 1;
-      ga[h] = p.A + (size_t)gr * p.lda + 2 * ((lane & 7) ^ ((row >> 1) & 7));
+      ga[h] = p.A + (size_t)gr * p.lda + 2 * ((lane & 7) ^ (row & 7));
       la[h] = c * 128;
     } else {
       int ge = m0 + 2 * lane; ge = ge + 1 < p.M ? ge : p.M - 2;
@@ -456,7 +470,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
     if (B_KC) {
       const int row = 8 * c + (lane >> 3);
       int gr = n0 + row; gr = gr < p.N ? gr : p.N - 1;
-      gb[h] = p.B + (size_t)gr * p.ldb + 2 * ((lane & 7) ^ ((row >> 1) & 7));
+      gb[h] = p.B + (size_t)gr * p.ldb + 2 * ((lane & 7) ^ (row & 7));
       lb[h] = c * 128;
     } else {
       int ge = n0 + 2 * lane; ge = ge + 1 < p.N ? ge : p.N - 2;
@@ -502,81 +516,95 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
   const bool do_colsum = !A_KC && p.colsum != nullptr && tile_n == 0;
   double colsum_partial = 0.0;
 
-  int cur = 0, nxt = DIST % STAGES;
-  // Fragment registers are double-buffered by hand: the LDS reads of step ks+1 are issued
-  // before the matrix cores start on step ks, and the reads of the next tile's first step are
-  // issued right after the barrier, under the last MFMAs of the current tile.  The reads are
-  // inline assembly so that their place in the instruction stream is fixed; the waits carry
-  // the fragment registers as operands, which keeps every MFMA behind the wait that covers it.
-  static_assert(TM == 4 && TN == 2, "fragment reads below are written for 64x32 wave tiles");
-  uint32_t a_off[BK / 4], b_off[BK / 4];  // byte offsets inside a stage
+  // The 16 contraction indices of a tile are consumed as two pairs of MFMA steps; in pair s the
+  // lane group lk multiplies k = 8s + 2lk in the first step and k = 8s + 2lk + 1 in the second (both
+  // operands use the same assignment, so only the order of the summation changes).  That makes a
+  // fragment of both steps one 16-byte LDS read per lane.  The reads are inline assembly so that
+  // their place in the instruction stream is fixed: each A fragment of the next pair is requested
+  // as soon as the MFMAs that consume the current one have been issued, the two B fragments are
+  // double-buffered and requested a whole step ahead, and across a tile boundary the requests go
+  // out right after the barrier, under the second step of the last pair.  Every wait carries the
+  // registers it covers as operands, which keeps the MFMAs that read them behind it.
+  static_assert(TM == 4 && TN == 2 && BK == 16, "the schedule below is written for 64x32 wave tiles");
+  uint32_t a_off[2], b_off[2];  // byte offset of this lane's fragment 0 inside a stage, per pair
 #pragma unroll
-  for (int ks = 0; ks < BK / 4; ++ks) {
-    const int k = ks * 4 + lk;
-    a_off[ks] = 8u * (A_KC ? (uint32_t)((wm * WM + lr) * BK + 2 * ((k >> 1) ^ ((lr >> 1) & 7)) + (k & 1))
-                           : (uint32_t)(k * (BM + 16) + wm * WM + lr));
-    b_off[ks] = 8u * (B_KC ? (uint32_t)((wn * WN + lr) * BK + 2 * ((k >> 1) ^ ((lr >> 1) & 7)) + (k & 1))
-                           : (uint32_t)(k * (BN + 16) + wn * WN + lr));
+  for (int s2 = 0; s2 < 2; ++s2) {
+    const int pr = 4 * s2 + lk;  // pair index = k / 2
+    a_off[s2] = 8u * (A_KC ? (uint32_t)((wm * WM + lr) * BK + 2 * (pr ^ (lr & 7)))
+                           : (uint32_t)(2 * pr * (BM + 16) + wm * WM + lr));
+    b_off[s2] = 8u * (B_KC ? (uint32_t)((wn * WN + lr) * BK + 2 * (pr ^ (lr & 7)))
+                           : (uint32_t)(2 * pr * (BN + 16) + wn * WN + lr));
   }
   const uint32_t a_base = (uint32_t)(uintptr_t)&lds_a[0][0], b_base = (uint32_t)(uintptr_t)&lds_b[0][0];
-  v2d fa0[2], fa1[2], fb0[2];  // [buffer]: A fragments 0-1, 2-3, B fragments 0-1
-  auto read_frags = [&](int buf, int stage, int ks) {
-    const uint32_t aa = a_base + (uint32_t)stage * (A_SIZE * 8) + a_off[ks];
-    const uint32_t bb = b_base + (uint32_t)stage * (B_SIZE * 8) + b_off[ks];
-    if constexpr (A_KC) {
-      asm volatile("ds_read2st64_b64 %0, %2 offset1:4\n\tds_read2st64_b64 %1, %2 offset0:8 offset1:12"
-                   : "=&v"(fa0[buf]), "=&v"(fa1[buf]) : "v"(aa) : "memory");
-    } else {
-      asm volatile("ds_read2_b64 %0, %2 offset1:16\n\tds_read2_b64 %1, %2 offset0:32 offset1:48"
-                   : "=&v"(fa0[buf]), "=&v"(fa1[buf]) : "v"(aa) : "memory");
-    }
-    if constexpr (B_KC) {
-      asm volatile("ds_read2st64_b64 %0, %1 offset1:4" : "=&v"(fb0[buf]) : "v"(bb) : "memory");
-    } else {
-      asm volatile("ds_read2_b64 %0, %1 offset1:16" : "=&v"(fb0[buf]) : "v"(bb) : "memory");
-    }
+  v2d fa[4], fb[2][2];  // A fragments (single set), B fragments [buffer][j]
+  auto a_addr = [&](int stage, int s2) { return a_base + (uint32_t)stage * (A_SIZE * 8) + a_off[s2]; };
+  auto b_addr = [&](int stage, int s2) { return b_base + (uint32_t)stage * (B_SIZE * 8) + b_off[s2]; };
+  auto mfma_row = [&](int i, double a, double b0, double b1) {
+    acc[i][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b0, acc[i][0], 0, 0, 0);
+    acc[i][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b1, acc[i][1], 0, 0, 0);
   };
-  // wait until only the `pending` youngest LDS reads are outstanding
-  auto wait_frags3 = [&](int buf) {
-    asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(fa0[buf]), "+v"(fa1[buf]), "+v"(fb0[buf]));
+  // first step of a pair: the six reads B0 B1 A0 A1 A2 A3 are outstanding in that order
+  auto first_step = [&](int bb) {
+    asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(fa[0]), "+v"(fb[bb][0]), "+v"(fb[bb][1]));
+    mfma_row(0, fa[0].x, fb[bb][0].x, fb[bb][1].x);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(fa[1]));
+    mfma_row(1, fa[1].x, fb[bb][0].x, fb[bb][1].x);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(fa[2]));
+    mfma_row(2, fa[2].x, fb[bb][0].x, fb[bb][1].x);
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[3]));
+    mfma_row(3, fa[3].x, fb[bb][0].x, fb[bb][1].x);
+    __builtin_amdgcn_sched_barrier(0);
   };
-  auto wait_frags0 = [&](int buf) {
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa0[buf]), "+v"(fa1[buf]), "+v"(fb0[buf]));
+  // second step of a pair, requesting the fragments of pair (stage, s2) meanwhile.  After the
+  // last tile the requests fetch stale LDS contents that nobody uses; they are drained below.
+  auto second_step = [&](int bb, int stage, int s2) {
+    const uint32_t aa = a_addr(stage, s2), ba = b_addr(stage, s2);
+    read_quad<B_KC, 0>(fb[bb ^ 1][0], ba);
+    read_quad<B_KC, 1>(fb[bb ^ 1][1], ba);
+    mfma_row(0, fa[0].y, fb[bb][0].y, fb[bb][1].y);
+    __builtin_amdgcn_sched_barrier(0);
+    read_quad<A_KC, 0>(fa[0], aa);
+    mfma_row(1, fa[1].y, fb[bb][0].y, fb[bb][1].y);
+    __builtin_amdgcn_sched_barrier(0);
+    read_quad<A_KC, 1>(fa[1], aa);
+    mfma_row(2, fa[2].y, fb[bb][0].y, fb[bb][1].y);
+    __builtin_amdgcn_sched_barrier(0);
+    read_quad<A_KC, 2>(fa[2], aa);
+    mfma_row(3, fa[3].y, fb[bb][0].y, fb[bb][1].y);
+    __builtin_amdgcn_sched_barrier(0);
+    read_quad<A_KC, 3>(fa[3], aa);
   };
-  auto mfmas = [&](int buf) {
-    const double a[4] = {fa0[buf].x, fa0[buf].y, fa1[buf].x, fa1[buf].y};
-    const double b[2] = {fb0[buf].x, fb0[buf].y};
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(a[i], b[j], acc[i][j], 0, 0, 0);
-  };
-  if (nk > 0) read_frags(0, 0, 0);
+  {
+    const uint32_t aa = a_addr(0, 0), ba = b_addr(0, 0);
+    read_quad<B_KC, 0>(fb[0][0], ba);
+    read_quad<B_KC, 1>(fb[0][1], ba);
+    read_quad<A_KC, 0>(fa[0], aa);
+    read_quad<A_KC, 1>(fa[1], aa);
+    read_quad<A_KC, 2>(fa[2], aa);
+    read_quad<A_KC, 3>(fa[3], aa);
+  }
+  int cur = 0, nxt = DIST % STAGES;
   for (int kt = 0; kt < nk; ++kt) {
     if (kt + DIST < nk) issue(nxt);
     if (!A_KC) {
       if (do_colsum) colsum_accumulate<BM, NW * 64>(colsum_partial, lds_a[cur], tid);
     }
-    read_frags(1, cur, 1);
-    wait_frags3(0);
-    mfmas(0);
-    read_frags(0, cur, 2);
-    wait_frags3(1);
-    mfmas(1);
-    read_frags(1, cur, 3);
-    wait_frags3(0);
-    mfmas(0);
-    __builtin_amdgcn_sched_barrier(0);
+    first_step(0);
+    second_step(0, cur, 1);
+    first_step(1);  // ends with lgkmcnt(0): this wave's LDS reads of `cur` are done
     // tile kt+1 must have landed: at most DIST-1 younger tiles may still be in flight
     if (kt + DIST < nk) wait_vmcnt((DIST - 1) * 2 * CH); else wait_vmcnt(0);
-    wait_frags0(1);  // this wave's LDS reads of `cur` are done
     __builtin_amdgcn_s_barrier();
     cur = cur + 1 == STAGES ? 0 : cur + 1;
     nxt = nxt + 1 == STAGES ? 0 : nxt + 1;
-    if (kt + 1 < nk) read_frags(0, cur, 0);
-    mfmas(1);
+    second_step(1, cur, 0);
   }
+  // the fragment registers stay reserved until the last (unused) requests have returned
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]),
+               "+v"(fb[0][0]), "+v"(fb[0][1]), "+v"(fb[1][0]), "+v"(fb[1][1]));
   if (!A_KC) {
     if (do_colsum) colsum_finish<BM, NW * 64>(colsum_partial, lds_b[0], tid, m0, split, p);
   }
