@@ -168,6 +168,92 @@ __device__ __forceinline__ double sgd_apply(double w, double g, double lr) {
   return w - step;
 }
 
+// Epilogue of one wavefront's block of 16x16 tiles: accumulator register r of fragment (i, j) is
+// row row0 + 16*i + 4*r + lk, column col0 + 16*j + lr.  What an element needs from memory (the ReLU
+// mask, or the parameter that the fused SGD update rewrites) is requested for one fragment row at
+// a time from clamped, always valid addresses before any of it is used, so that the loads of a
+// batch are in flight together; only the stores are predicated on the bounds.
+template <int TM, int TN, int EPI, bool SGD>
+__device__ __forceinline__ void store_block(const GemmParams& p, const v4d* acc, int row0, int col0,
+                                            int lr, int lk) {
+  constexpr int IB = 1;  // two rows at a time would spill in the 128x128 kernels
+#pragma unroll
+  for (int i0 = 0; i0 < TM; i0 += IB) {
+    double extra[IB][TN][4];
+    double bias[TN];
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int col = col0 + j * 16 + lr;
+      const int cc = col < p.N ? col : p.N - 1;
+      if (EPI == EPI_BIAS || EPI == EPI_BIAS_RELU) bias[j] = p.bias[cc];
+      if (EPI == EPI_MASK || SGD) {
+#pragma unroll
+        for (int ii = 0; ii < IB; ++ii)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int row = row0 + (i0 + ii) * 16 + 4 * r + lk;
+            const int rc = row < p.M ? row : p.M - 1;
+            extra[ii][j][r] = (EPI == EPI_MASK) ? p.mask[(size_t)rc * p.ldmask + cc]
+                                                : p.sgd_parm[(size_t)rc * p.ldc + cc];
+          }
+      }
+    }
+#pragma unroll
+    for (int ii = 0; ii < IB; ++ii)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = col0 + j * 16 + lr;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = row0 + (i0 + ii) * 16 + 4 * r + lk;
+          double v = acc[(i0 + ii) * TN + j][r];
+          if (EPI == EPI_BIAS) v = v + bias[j];
+          if (EPI == EPI_BIAS_RELU) v = fmax(v + bias[j], 0.0);
+          if (EPI == EPI_RELU) v = fmax(v, 0.0);
+          if (EPI == EPI_DIVIDE) v = v / p.divisor;
+          if (EPI == EPI_MASK) v = v * (extra[ii][j][r] > 0.0 ? 1.0 : 0.0);
+          if (row < p.M && col < p.N) {
+            p.C[(size_t)row * p.ldc + col] = v;
+            if (SGD) p.sgd_parm[(size_t)row * p.ldc + col] = sgd_apply(extra[ii][j][r], v, p.sgd_lr);
+          }
+        }
+      }
+  }
+}
+
+// Writes the block either as raw partial products of K slice `split` (the reduction applies the
+// epilogue later) or finished, with the epilogue the launch asks for.
+template <int TM, int TN>
+__device__ __forceinline__ void write_block(const GemmParams& p, const v4d* acc, int row0, int col0,
+                                            int lr, int lk, int split) {
+  if (p.split_k > 1) {
+    double* __restrict__ out = p.ws + (size_t)split * p.M * p.N;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int col = col0 + j * 16 + lr;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int row = row0 + i * 16 + 4 * r + lk;
+          if (row < p.M && col < p.N) out[(size_t)row * p.N + col] = acc[i * TN + j][r];
+        }
+      }
+    return;
+  }
+  switch (p.epilogue) {
+    case EPI_BIAS: store_block<TM, TN, EPI_BIAS, false>(p, acc, row0, col0, lr, lk); break;
+    case EPI_BIAS_RELU: store_block<TM, TN, EPI_BIAS_RELU, false>(p, acc, row0, col0, lr, lk); break;
+    case EPI_RELU: store_block<TM, TN, EPI_RELU, false>(p, acc, row0, col0, lr, lk); break;
+    case EPI_MASK: store_block<TM, TN, EPI_MASK, false>(p, acc, row0, col0, lr, lk); break;
+    case EPI_DIVIDE:
+      if (p.sgd_parm) store_block<TM, TN, EPI_DIVIDE, true>(p, acc, row0, col0, lr, lk);
+      else store_block<TM, TN, EPI_DIVIDE, false>(p, acc, row0, col0, lr, lk);
+      break;
+    default: store_block<TM, TN, EPI_NONE, false>(p, acc, row0, col0, lr, lk); break;
+  }
+}
+
 // Bias gradient inside the weight-gradient contraction (output-contiguous A = grad^T): the
 // workgroups of tile column 0 also add up their A tile over the contraction index.  Thread t
 // owns output row t % BM and every (THREADS/BM)-th contraction row; partial sums are combined
@@ -312,51 +398,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm
     if (do_colsum) colsum_finish<BM, kThreads>(colsum_partial, lds_b[0], tid, m0, split, p);
   }
 
-  // Epilogue: accumulator register r of this lane is row 4*r + lk, column lr of its tile.
-  if (p.split_k > 1) {  // raw partial products of this K slice; the reduction applies the epilogue
-    double* __restrict__ out = p.ws + (size_t)split * p.M * p.N;
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int col = n0 + wn * WN + j * 16 + lr;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int row = m0 + wm * WM + i * 16 + 4 * r + lk;
-          if (row < p.M && col < p.N) out[(size_t)row * p.N + col] = acc[i][j][r];
-        }
-      }
-    return;
-  }
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = n0 + wn * WN + j * 16 + lr;
-      if (col >= p.N) continue;
-      double bias = 0.0;
-      if (p.epilogue == EPI_BIAS || p.epilogue == EPI_BIAS_RELU) bias = p.bias[col];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int row = m0 + wm * WM + i * 16 + 4 * r + lk;
-        if (row >= p.M) continue;
-        double v = acc[i][j][r];
-        switch (p.epilogue) {
-          case EPI_BIAS: v = v + bias; break;
-          case EPI_BIAS_RELU: v = fmax(v + bias, 0.0); break;
-          case EPI_RELU: v = fmax(v, 0.0); break;
-          case EPI_DIVIDE: v = v / p.divisor; break;
-          case EPI_MASK: v = v * (p.mask[(size_t)row * p.ldmask + col] > 0.0 ? 1.0 : 0.0); break;
-          default: break;
-        }
-        p.C[(size_t)row * p.ldc + col] = v;
-        if (p.sgd_parm) {
-          double* w = p.sgd_parm + (size_t)row * p.ldc + col;
-          *w = sgd_apply(*w, v, p.sgd_lr);
-        }
-      }
-    }
-  }
+  write_block<TM, TN>(p, &acc[0][0], m0 + wm * WM, n0 + wn * WN, lr, lk, split);
 }
 
 // ---- 128x128 tiles fed by direct global -> LDS loads ------------------------------------------
@@ -609,50 +651,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
     if (do_colsum) colsum_finish<BM, NW * 64>(colsum_partial, lds_b[0], tid, m0, split, p);
   }
 
-  if (p.split_k > 1) {  // raw partial products of this K slice; the reduction applies the epilogue
-    double* __restrict__ out = p.ws + (size_t)split * p.M * p.N;
-#pragma unroll
-    for (int i = 0; i < TM; ++i)
-#pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const int col = n0 + wn * WN + j * 16 + lr;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int row = m0 + wm * WM + i * 16 + 4 * r + lk;
-          if (row < p.M && col < p.N) out[(size_t)row * p.N + col] = acc[i][j][r];
-        }
-      }
-    return;
-  }
-#pragma unroll
-  for (int i = 0; i < TM; ++i) {
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int col = n0 + wn * WN + j * 16 + lr;
-      if (col >= p.N) continue;
-      double bias = 0.0;
-      if (p.epilogue == EPI_BIAS || p.epilogue == EPI_BIAS_RELU) bias = p.bias[col];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int row = m0 + wm * WM + i * 16 + 4 * r + lk;
-        if (row >= p.M) continue;
-        double v = acc[i][j][r];
-        switch (p.epilogue) {
-          case EPI_BIAS: v = v + bias; break;
-          case EPI_BIAS_RELU: v = fmax(v + bias, 0.0); break;
-          case EPI_RELU: v = fmax(v, 0.0); break;
-          case EPI_DIVIDE: v = v / p.divisor; break;
-          case EPI_MASK: v = v * (p.mask[(size_t)row * p.ldmask + col] > 0.0 ? 1.0 : 0.0); break;
-          default: break;
-        }
-        p.C[(size_t)row * p.ldc + col] = v;
-        if (p.sgd_parm) {
-          double* w = p.sgd_parm + (size_t)row * p.ldc + col;
-          *w = sgd_apply(*w, v, p.sgd_lr);
-        }
-      }
-    }
-  }
+  write_block<TM, TN>(p, &acc[0][0], m0 + wm * WM, n0 + wn * WN, lr, lk, split);
 }
 
 // Adds the K slices of a split contraction in slice order and applies the epilogue.
