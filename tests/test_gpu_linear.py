@@ -27,8 +27,10 @@ SHAPES = [
     # >= 256 tiles of 128x128 with ragged edges: the direct-to-LDS kernels (K % 16 == 0) and the
     # register-staged kernel with a K tail, for each of the three operand layouts
     (2050, 64, 2046), (2064, 2046, 2046), (2050, 2046, 2048),
-    # 256..511 tiles with a long contraction: the direct-to-LDS kernels cut K in two halves
-    (2064, 2048, 2046),
+    # 256..511 tiles with a long contraction (K >= 6144): the direct-to-LDS kernels cut K in two
+    # halves - forward, input gradient and weight gradient (+ bias gradient over slices) in turn;
+    # (2064, 2048, 2046) is the same tile count below the threshold
+    (2064, 2048, 2046), (2064, 6144, 2046), (2064, 2048, 6144), (6144, 2048, 2046),
     # small outputs with a long contraction: the split-K path (with and without a K tail)
     (8192, 784, 100), (8192, 100, 10), (32, 4099, 24), (4100, 7, 9), (16384, 33, 65),
 ]
