@@ -30,12 +30,13 @@ PEAK_HBM_GBPS = 8000.0
 # (8 hidden layers + the head).  Measured with two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE)
 # of this script, scaled by the same counters on a streaming kernel of known size
 # (--calibration-copy: FETCH x 2.0, WRITE x 1.0); the summary is kept under profiles/.
-# A launch = the contraction plus, where its 256 tiles are contracted as two K slices, the reduction
-# of the two partial results (117.5 MB); the weight gradient carries the SGD update of its layer.
+# A launch = the contraction plus, for the one that is contracted as two K slices (the head's input
+# gradient), the reduction of the two partial results (134.3 MB); the weight gradient carries the SGD
+# update of its layer.
 C4_TRAFFIC_BYTES_PER_LAUNCH = {
-    "linear_forward": (8 * (487.5e6 + 117.5e6) + 4034.5e6) / 9,
-    "grad_weight": (8 * 789.0e6 + 6449.5e6) / 9,
-    "grad_input": 892.4e6 + 117.5e6,
+    "linear_forward": (8 * 439.8e6 + 4846.9e6) / 9,
+    "grad_weight": (8 * 797.0e6 + 6526.8e6) / 9,
+    "grad_input": (7 * 470.1e6 + 4788.5e6 + 134.3e6) / 8,
 }
 
 C4_SPEC = [("linear", 4096, 4096), ("relu",)] * 8 + [("linear", 4096, 32768)]
