@@ -7,9 +7,15 @@
 // without materialising a transpose: the operand layout only changes how a tile is copied
 // into LDS and which LDS stride the MFMA fragments are read with.
 //
-// Tiling: 256 threads = 4 wavefronts in a 2x2 grid, each owning a (BM/2)x(BN/2) block of
-// 16x16 MFMA tiles held in registers; K advances in steps of 16 through two LDS stages, the
-// global loads of step k+1 are in flight while step k is multiplied.
+// Two kernels share the template parameters and the epilogues:
+//   gemm_f64_mfma      register-staged tiles of 32x32, 64x64 or 128x128 (WGM x WGN wavefronts, each
+//                      owning a (BM/WGM)x(BN/WGN) block of 16x16 MFMA tiles in registers), any
+//                      shape and alignment, optional split-K for small outputs;
+//   gemm_f64_mfma_dma  128x128 tiles, eight wavefronts of 64x32, operand tiles moved global -> LDS
+//                      by global_load_lds_dwordx4 and a hand-scheduled inner loop: the path of
+//                      the large aligned products (K a multiple of 16, at least 256 tiles).
+// K advances in steps of 16 through two LDS stages; the loads of step k+1 are in flight while
+// step k is multiplied.
 //
 // MFMA register layout (64 lanes): A fragment lane l holds A[l%16][l/16], B fragment lane l
 // holds B[l/16][l%16], and accumulator register r of lane l holds D[4*r + l/16][l%16].
