@@ -281,7 +281,7 @@ def main():
     dm.close()
     log("C4: %.3f ms/step, loss %.6f" % (ms_per_step, loss))
 
-    gemm_kinds = [k for k in ("linear_forward", "grad_weight", "grad_input") if k in kernels]
+    gemm_kinds = [k for k in ("linear_forward", "grad_weight", "grad_input", "grad_pair") if k in kernels]
     dominant = max(gemm_kinds, key=lambda k: kernels[k]["ms_per_step"])
     d = kernels[dominant]
     launches = [r for r in recs if r["kernel"] == dominant]

@@ -229,6 +229,13 @@ int rst_model_train_step(rst_model* model, const double* x, const double* truth,
  * old weights, is launched first).  enabled == 0 runs the optimiser as its own pass over the
  * parameter arena, as rst_model_sgd_step does. */
 int rst_model_fuse_sgd(rst_model* model, int enabled);
+/* enabled != 0: the backward pass holds each layer's weight gradient back until the next layer's
+ * input gradient is due and launches the two, which do not depend on each other, as one grid when
+ * both are large aligned products (a 256-tile input gradient alone leaves one workgroup per CU).
+ * Results are identical either way.  Off by default: on MI355X the gain depends on where the
+ * dispatcher places the long tiles (measured 0.99 or 1.10 ms per pair at C4's hidden width, at
+ * random, against 1.02 ms for the two launches one after the other). */
+int rst_model_pair_gradients(rst_model* model, int enabled);
 /* rst_model_train_step records its launches into a HIP graph the first time it sees a given
  * (x, truth, batch, lr) and replays the graph afterwards; a different argument re-records.
  * enabled == 0 switches to plain launches (profiling does so by itself).  Default: enabled. */
@@ -253,7 +260,8 @@ enum {
   RST_KERNEL_RELU_BACKWARD = 5,
   RST_KERNEL_CROSS_ENTROPY = 6,
   RST_KERNEL_LOSS_REDUCE = 7,
-  RST_KERNEL_SGD = 8
+  RST_KERNEL_SGD = 8,
+  RST_KERNEL_GRAD_PAIR = 9   /* one layer's input gradient and the weight gradient of the layer above, one grid */
 };
 int rst_model_profile_enable(rst_model* model, int enabled);
 int rst_model_profile_read(rst_model* model, rst_kernel_record* host_records, size_t capacity,

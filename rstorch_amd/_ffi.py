@@ -24,7 +24,7 @@ LAYER_IDENTITY, LAYER_LINEAR, LAYER_RELU = 0, 1, 2
 
 KERNEL_NAMES = {
     0: "linear_forward", 1: "grad_weight", 2: "grad_bias", 3: "grad_input", 4: "relu_forward",
-    5: "relu_backward", 6: "cross_entropy", 7: "loss_reduce", 8: "sgd",
+    5: "relu_backward", 6: "cross_entropy", 7: "loss_reduce", 8: "sgd", 9: "grad_pair",
 }
 
 
@@ -112,6 +112,7 @@ SIGNATURES = {
     "rst_model_profile_enable": [_vp, _i32],
     "rst_model_graph_enable": [_vp, _i32],
     "rst_model_fuse_sgd": [_vp, _i32],
+    "rst_model_pair_gradients": [_vp, _i32],
     "rst_model_profile_read": [_vp, ctypes.POINTER(KernelRecord), _sz, c_size_p],
 }
 _SPECIAL = {

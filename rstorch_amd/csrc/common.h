@@ -72,6 +72,12 @@ struct GemmDesc {
 };
 
 int launch_gemm(hipStream_t stream, const GemmDesc& d);
+// Two independent contractions, the input gradient of one layer (A contraction-contiguous, B
+// output-contiguous) and the weight gradient of another (both output-contiguous), in one grid.
+// Possible when both run as unsplit 128x128 direct-to-LDS tiles and the first alone would
+// under-fill the chip (fewer than 512 tiles).
+bool can_pair_gemm(const GemmDesc& input_grad, const GemmDesc& weight_grad);
+int launch_gemm_pair(hipStream_t stream, const GemmDesc& input_grad, const GemmDesc& weight_grad);
 
 // ---- streaming kernels -----------------------------------------------------------------------
 int launch_relu_forward(hipStream_t s, const double* x, double* out, size_t n);

@@ -199,8 +199,10 @@ __device__ __forceinline__ void store_block(const GemmParams& p, const v4d* acc,
           for (int r = 0; r < 4; ++r) {
             const int row = row0 + (i0 + ii) * 16 + 4 * r + lk;
             const int rc = row < p.M ? row : p.M - 1;
-            extra[ii][j][r] = (EPI == EPI_MASK) ? p.mask[(size_t)rc * p.ldmask + cc]
-                                                : p.sgd_parm[(size_t)rc * p.ldc + cc];
+            // a parameter is read once and rewritten once per step: keep it out of the caches
+            extra[ii][j][r] = (EPI == EPI_MASK)
+                                  ? p.mask[(size_t)rc * p.ldmask + cc]
+                                  : __builtin_nontemporal_load(p.sgd_parm + (size_t)rc * p.ldc + cc);
           }
       }
     }
@@ -219,8 +221,13 @@ __device__ __forceinline__ void store_block(const GemmParams& p, const v4d* acc,
           if (EPI == EPI_DIVIDE) v = v / p.divisor;
           if (EPI == EPI_MASK) v = v * (extra[ii][j][r] > 0.0 ? 1.0 : 0.0);
           if (row < p.M && col < p.N) {
-            p.C[(size_t)row * p.ldc + col] = v;
-            if (SGD) p.sgd_parm[(size_t)row * p.ldc + col] = sgd_apply(extra[ii][j][r], v, p.sgd_lr);
+            if (EPI == EPI_DIVIDE)  // a weight gradient: nothing reads it again soon
+              __builtin_nontemporal_store(v, p.C + (size_t)row * p.ldc + col);
+            else
+              p.C[(size_t)row * p.ldc + col] = v;
+            if (SGD)
+              __builtin_nontemporal_store(sgd_apply(extra[ii][j][r], v, p.sgd_lr),
+                                          p.sgd_parm + (size_t)row * p.ldc + col);
           }
         }
       }
@@ -462,22 +469,26 @@ __device__ __forceinline__ void read_quad(v2d& q, uint32_t addr) {
   }
 }
 
+// Work of one workgroup: output tile number `block` (and its K slice) of problem p.  lds_a / lds_b
+// are the workgroup's STAGES operand stages (kDmaStage doubles each).
+constexpr int kDmaStage = BK * (128 + 16);  // the larger of the two tile layouts
+
 template <bool A_KC, bool B_KC, int WGM, int WGN, int STAGES, int DIST>
-__global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const GemmParams p) {
+__device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double* __restrict__ lds_a,
+                                         double* __restrict__ lds_b) {
   constexpr int BM = 128, BN = 128, NW = WGM * WGN;
   constexpr int WM = BM / WGM, WN = BN / WGN, TM = WM / 16, TN = WN / 16;
   constexpr int CH = 16 / NW;  // 1 KiB chunks of each operand tile moved by one wavefront
   static_assert(16 % NW == 0 && CH >= 1, "chunks must split over the wavefronts");
   constexpr int A_SIZE = A_KC ? BM * BK : BK * (BM + 16);
   constexpr int B_SIZE = B_KC ? BN * BK : BK * (BN + 16);
-  __shared__ __attribute__((aligned(1024))) double lds_a[STAGES][A_SIZE];
-  __shared__ __attribute__((aligned(1024))) double lds_b[STAGES][B_SIZE];
+  static_assert(A_SIZE <= kDmaStage && B_SIZE <= kDmaStage, "stage size");
 
   const int n_blocks = p.tiles_m * p.tiles_n;
-  const int split = blockIdx.x / n_blocks;  // K slice of this workgroup (0 without split-K)
+  const int split = block / n_blocks;  // K slice of this workgroup (0 without split-K)
   int logical;
   {
-    const int pid = blockIdx.x - split * n_blocks;
+    const int pid = block - split * n_blocks;
     const int xcd = pid & 7, local = pid >> 3;
     const int base = n_blocks >> 3, rem = n_blocks & 7;
     logical = xcd * base + (xcd < rem ? xcd : rem) + local;
@@ -548,8 +559,8 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
   auto issue = [&](int stage) {
 #pragma unroll
     for (int h = 0; h < CH; ++h) {
-      dma16(ga[h], &lds_a[stage][la[h]]);
-      dma16(gb[h], &lds_b[stage][lb[h]]);
+      dma16(ga[h], lds_a + stage * A_SIZE + la[h]);
+      dma16(gb[h], lds_b + stage * B_SIZE + lb[h]);
       ga[h] += a_step;
       gb[h] += b_step;
     }
@@ -583,7 +594,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
     b_off[s2] = 8u * (B_KC ? (uint32_t)((wn * WN + lr) * BK + 2 * (pr ^ (lr & 7)))
                            : (uint32_t)(2 * pr * (BN + 16) + wn * WN + lr));
   }
-  const uint32_t a_base = (uint32_t)(uintptr_t)&lds_a[0][0], b_base = (uint32_t)(uintptr_t)&lds_b[0][0];
+  const uint32_t a_base = (uint32_t)(uintptr_t)lds_a, b_base = (uint32_t)(uintptr_t)lds_b;
   v2d fa[4], fb[2][2];  // A fragments (single set), B fragments [buffer][j]
   auto a_addr = [&](int stage, int s2) { return a_base + (uint32_t)stage * (A_SIZE * 8) + a_off[s2]; };
   auto b_addr = [&](int stage, int s2) { return b_base + (uint32_t)stage * (B_SIZE * 8) + b_off[s2]; };
@@ -638,7 +649,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
   for (int kt = 0; kt < nk; ++kt) {
     if (kt + DIST < nk) issue(nxt);
     if (!A_KC) {
-      if (do_colsum) colsum_accumulate<BM, NW * 64>(colsum_partial, lds_a[cur], tid);
+      if (do_colsum) colsum_accumulate<BM, NW * 64>(colsum_partial, lds_a + cur * A_SIZE, tid);
     }
     first_step(0);
     second_step(0, cur, 1);
@@ -654,10 +665,47 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
   asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[0]), "+v"(fa[1]), "+v"(fa[2]), "+v"(fa[3]),
                "+v"(fb[0][0]), "+v"(fb[0][1]), "+v"(fb[1][0]), "+v"(fb[1][1]));
   if (!A_KC) {
-    if (do_colsum) colsum_finish<BM, NW * 64>(colsum_partial, lds_b[0], tid, m0, split, p);
+    if (do_colsum) colsum_finish<BM, NW * 64>(colsum_partial, lds_b, tid, m0, split, p);
   }
 
   write_block<TM, TN>(p, &acc[0][0], m0 + wm * WM, n0 + wn * WN, lr, lk, split);
+}
+
+template <bool A_KC, bool B_KC, int WGM, int WGN, int STAGES, int DIST>
+__global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const GemmParams p) {
+  constexpr int A_SIZE = A_KC ? 128 * BK : kDmaStage, B_SIZE = B_KC ? 128 * BK : kDmaStage;
+  __shared__ __attribute__((aligned(1024))) double lds_a[STAGES * A_SIZE];
+  __shared__ __attribute__((aligned(1024))) double lds_b[STAGES * B_SIZE];
+  dma_tile<A_KC, B_KC, WGM, WGN, STAGES, DIST>(p, (int)blockIdx.x, lds_a, lds_b);
+}
+
+// Two independent products in one grid: workgroups [0, first_blocks) work on `first`, the others on
+// `second`.  Used for the input gradient of one layer (256 long tiles at C4's hidden width: on its
+// own one workgroup per CU) together with the weight gradient of the layer above it (many short
+// tiles): the long tiles are dispatched first, the short ones fill the second workgroup slot of
+// every CU, so both run at the two-workgroups-per-CU rate.
+template <bool A_KC1, bool B_KC1, bool A_KC2, bool B_KC2>
+__global__ __launch_bounds__(512, 4) void gemm_f64_mfma_dma_pair(const GemmParams first, const GemmParams second,
+                                                                  int first_blocks) {
+  __shared__ __attribute__((aligned(1024))) double lds_a[2 * kDmaStage];
+  __shared__ __attribute__((aligned(1024))) double lds_b[2 * kDmaStage];
+  // Workgroup b goes to XCD b % 8.  The first 2*first_blocks workgroups alternate between the two
+  // problems in groups of eight (one per XCD), with the phase flipped every 32 groups, so that the
+  // long tiles of `first` spread over the CUs under the usual hand-out orders; tile numbers keep
+  // their value mod 8, which the XCD-aware tile walk relies on.  The placement is still the
+  // dispatcher's: a CU that ends up with two runs of short tiles (each ending in an SGD epilogue)
+  // finishes about 10 % late.
+  const int b = (int)blockIdx.x;
+  if (b < 2 * first_blocks) {
+    const int g = b >> 3;
+    const int local = (g >> 1) * 8 + (b & 7);
+    if (((g + (g >> 5)) & 1) == 0)
+      dma_tile<A_KC1, B_KC1, 2, 4, 2, 1>(first, local, lds_a, lds_b);
+    else
+      dma_tile<A_KC2, B_KC2, 2, 4, 2, 1>(second, local, lds_a, lds_b);
+  } else {
+    dma_tile<A_KC2, B_KC2, 2, 4, 2, 1>(second, b - first_blocks, lds_a, lds_b);
+  }
 }
 
 // Adds the K slices of a split contraction in slice order and applies the epilogue.
@@ -699,6 +747,8 @@ int launch_split_reduce(hipStream_t stream, const GemmParams& p) {
   return RST_OK;
 }
 
+constexpr int kSplitMinSteps = 384;  // K >= 6144
+
 template <bool A_KC, bool B_KC>
 int launch_dma(hipStream_t stream, GemmParams p) {
   p.tiles_m = (p.M + 127) / 128;
@@ -713,7 +763,7 @@ int launch_dma(hipStream_t stream, GemmParams p) {
   // of about 31 us per launch at 1024 x 4096 outputs, which pays off from K of about 5400 on.
   const int nk = p.K / BK;
   const size_t need = 2 * ((size_t)p.M * p.N + (size_t)p.M);
-  if (blocks < 512 && nk >= 384 && p.ws != nullptr && p.ws_capacity >= need) {
+  if (blocks < 512 && nk >= kSplitMinSteps && p.ws != nullptr && p.ws_capacity >= need) {
     p.split_k = 2;
     p.steps_per_split = (nk + 1) / 2;
     p.ws_colsum = p.ws + (size_t)2 * p.M * p.N;
@@ -776,8 +826,18 @@ int launch_layout(hipStream_t stream, const GemmParams& p) {
 
 }  // namespace
 
-int launch_gemm(hipStream_t stream, const GemmDesc& d) {
-  if (d.M <= 0 || d.N <= 0) return RST_OK;
+namespace {
+
+// 16-byte loads need both operands aligned with even leading dimensions and extents
+bool desc_vec_ok(const GemmDesc& d) {
+  auto ok = [](const double* ptr, long ld, int contiguous_extent) {
+    return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && (ld % 2 == 0) &&
+           (contiguous_extent % 2 == 0);
+  };
+  return ok(d.A, d.lda, d.a_kc ? d.K : d.M) && ok(d.B, d.ldb, d.b_kc ? d.K : d.N);
+}
+
+GemmParams make_params(const GemmDesc& d) {
   GemmParams p;
   p.A = d.A; p.B = d.B; p.C = d.C;
   p.M = d.M; p.N = d.N; p.K = d.K;
@@ -791,13 +851,24 @@ int launch_gemm(hipStream_t stream, const GemmDesc& d) {
   p.sgd_lr = d.sgd_lr;
   p.split_k = 1; p.steps_per_split = 0;
   p.ws = d.workspace; p.ws_colsum = nullptr; p.ws_capacity = d.workspace ? d.workspace_count : 0;
-  auto vec_ok = [](const double* ptr, long ld, int contiguous_extent) {
-    return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && (ld % 2 == 0) &&
-           (contiguous_extent % 2 == 0);
-  };
-  // 16-byte loads need both operands aligned with even leading dimensions and extents
-  const bool vec = vec_ok(d.A, d.lda, d.a_kc ? d.K : d.M) && vec_ok(d.B, d.ldb, d.b_kc ? d.K : d.N);
   p.tiles_m = p.tiles_n = 0;
+  return p;
+}
+
+// true when launch_gemm would run d as unsplit 128x128 direct-to-LDS tiles
+bool takes_plain_dma(const GemmDesc& d, long long* blocks) {
+  if (d.M < 2 || d.N < 2 || d.K <= 0 || d.K % BK != 0 || !desc_vec_ok(d)) return false;
+  *blocks = (long long)((d.M + 127) / 128) * ((d.N + 127) / 128);
+  if (*blocks < 256) return false;
+  return !(*blocks < 512 && d.K / BK >= kSplitMinSteps && d.workspace != nullptr);
+}
+
+}  // namespace
+
+int launch_gemm(hipStream_t stream, const GemmDesc& d) {
+  if (d.M <= 0 || d.N <= 0) return RST_OK;
+  const GemmParams p = make_params(d);
+  const bool vec = desc_vec_ok(d);
   if (d.a_kc && d.b_kc)
     return vec ? launch_layout<true, true, true>(stream, p) : launch_layout<true, true, false>(stream, p);
   if (!d.a_kc && !d.b_kc)
@@ -805,6 +876,27 @@ int launch_gemm(hipStream_t stream, const GemmDesc& d) {
   if (d.a_kc && !d.b_kc)
     return vec ? launch_layout<true, false, true>(stream, p) : launch_layout<true, false, false>(stream, p);
   return vec ? launch_layout<false, true, true>(stream, p) : launch_layout<false, true, false>(stream, p);
+}
+
+bool can_pair_gemm(const GemmDesc& input_grad, const GemmDesc& weight_grad) {
+  long long b1 = 0, b2 = 0;
+  const bool layouts = input_grad.a_kc && !input_grad.b_kc && !weight_grad.a_kc && !weight_grad.b_kc;
+  // worth it when the input gradient alone would leave one workgroup per CU
+  return layouts && takes_plain_dma(input_grad, &b1) && takes_plain_dma(weight_grad, &b2) && b1 < 512 &&
+         b1 % 8 == 0 && b2 >= b1 && b1 + b2 <= 0x7fffffffLL;
+}
+
+int launch_gemm_pair(hipStream_t stream, const GemmDesc& input_grad, const GemmDesc& weight_grad) {
+  if (!can_pair_gemm(input_grad, weight_grad))
+    return fail(RST_ERR_INVALID_ARGUMENT, "these two contractions cannot share a grid");
+  GemmParams p1 = make_params(input_grad), p2 = make_params(weight_grad);
+  p1.tiles_m = (p1.M + 127) / 128; p1.tiles_n = (p1.N + 127) / 128; p1.steps_per_split = p1.K / BK;
+  p2.tiles_m = (p2.M + 127) / 128; p2.tiles_n = (p2.N + 127) / 128; p2.steps_per_split = p2.K / BK;
+  const long long b1 = (long long)p1.tiles_m * p1.tiles_n, b2 = (long long)p2.tiles_m * p2.tiles_n;
+  hipLaunchKernelGGL((gemm_f64_mfma_dma_pair<true, false, false, false>), dim3((unsigned)(b1 + b2)), dim3(512),
+                     0, stream, p1, p2, (int)b1);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
 }
 
 }  // namespace rst

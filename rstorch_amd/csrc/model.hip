@@ -81,6 +81,10 @@ struct rst_model {
   unsigned long long graph_clock = 0;
   // train_step applies the optimiser update inside the weight-gradient launches
   bool fuse_sgd = true;
+  // backward launches a layer's weight gradient together with the next layer's input gradient.
+  // Off unless asked for: on C4 a pair takes 0.99 or 1.10 ms at random (which CUs end up with two
+  // long input-gradient tiles is the dispatcher's choice) against 1.02 ms for the two launches apart.
+  bool pair_gradients = false;
   // profiling
   bool profiling = false;
   bool slot_open = false;
@@ -256,6 +260,31 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
   for (int i = 0; i < n; ++i)
     if (m->layers[i].kind == RST_LAYER_LINEAR) { first_linear = i; break; }
 
+  // the weight gradient that has been described but not launched yet
+  struct {
+    bool active = false;
+    GemmDesc d{};
+    int layer = -1;
+    double flops = 0.0, bytes = 0.0;
+    bool fused_bias = false;
+    const double* grad = nullptr;  // gradient w.r.t. that layer's output
+  } pend;
+  auto flush_pending = [&]() -> int {
+    if (!pend.active) return RST_OK;
+    pend.active = false;
+    Layer& pl = m->layers[pend.layer];
+    RST_TRY(prof_begin(m, RST_KERNEL_GRAD_WEIGHT, pend.layer, pend.flops, pend.bytes));
+    RST_TRY(launch_gemm(e->stream, pend.d));
+    RST_TRY(prof_end(m));
+    if (!pend.fused_bias) {
+      RST_TRY(prof_begin(m, RST_KERNEL_GRAD_BIAS, pend.layer, 0.0, 8.0 * ((double)batch * pl.out + pl.out)));
+      RST_TRY(launch_column_mean(e->stream, pend.grad, pl.gb, batch, pl.out, n_rows));
+      RST_TRY(prof_end(m));
+      if (fused_lr) RST_TRY(launch_sgd_flat(e->stream, pl.b, pl.gb, pl.out, *fused_lr));
+    }
+    return RST_OK;
+  };
+
   for (int i = n - 1; i >= 0; --i) {
     Layer& l = m->layers[i];
     if (l.kind == RST_LAYER_IDENTITY) continue;  // identity.rs:22-24
@@ -269,60 +298,70 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
       continue;
     }
     // Linear: linear.rs:60-69.  The input gradient goes first: it reads the weights, which the
-    // weight-gradient launch may update in place when the optimiser step is fused in.
+    // weight-gradient launch may update in place when the optimiser step is fused in.  The weight
+    // gradient itself is held back one layer: it does not depend on anything the next layer down
+    // computes, so it can share a grid with that layer's input gradient (launch_gemm_pair).
     const double mnk = (double)batch * (double)l.in * (double)l.out;
     const bool wanted = need_input_grad || i != first_linear;
     const int pv = prev_non_identity(m, i);
     const bool mask = pv >= 0 && m->layers[pv].kind == RST_LAYER_RELU;
+    GemmDesc dx{};
+    double dx_bytes = 0.0;
     if (wanted) {
-      GemmDesc d{};
-      d.A = cur; d.B = l.w; d.C = l.grad_in_buf;
-      d.M = (int)batch; d.N = (int)l.in; d.K = (int)l.out;
-      d.lda = (long)l.out; d.ldb = (long)l.in; d.ldc = (long)l.in;
-      d.a_kc = true; d.b_kc = false;
-      d.epilogue = mask ? EPI_MASK : EPI_NONE;
-      d.mask = mask ? l.input : nullptr;  // the ReLU's output is this layer's input
-      d.ldmask = (long)l.in;
-      const double bytes = 8.0 * ((double)batch * l.out + (double)l.in * l.out +
-                                  (double)batch * l.in * (mask ? 2.0 : 1.0));
-      RST_TRY(prof_begin(m, RST_KERNEL_GRAD_INPUT, i, 2.0 * mnk, bytes));
-      d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
-      RST_TRY(launch_gemm(e->stream, d));
-      RST_TRY(prof_end(m));
-      if (mask) m->layers[pv].backward_absorbed = true;
+      dx.A = cur; dx.B = l.w; dx.C = l.grad_in_buf;
+      dx.M = (int)batch; dx.N = (int)l.in; dx.K = (int)l.out;
+      dx.lda = (long)l.out; dx.ldb = (long)l.in; dx.ldc = (long)l.in;
+      dx.a_kc = true; dx.b_kc = false;
+      dx.epilogue = mask ? EPI_MASK : EPI_NONE;
+      dx.mask = mask ? l.input : nullptr;  // the ReLU's output is this layer's input
+      dx.ldmask = (long)l.in;
+      dx.workspace = e->d_gemm_ws; dx.workspace_count = e->gemm_ws_count;
+      dx_bytes = 8.0 * ((double)batch * l.out + (double)l.in * l.out +
+                        (double)batch * l.in * (mask ? 2.0 : 1.0));
     }
+    if (pend.active && wanted && m->pair_gradients && can_pair_gemm(dx, pend.d)) {
+      RST_TRY(prof_begin(m, RST_KERNEL_GRAD_PAIR, i, 2.0 * mnk + pend.flops, dx_bytes + pend.bytes));
+      RST_TRY(launch_gemm_pair(e->stream, dx, pend.d));
+      RST_TRY(prof_end(m));
+      pend.active = false;
+    } else {
+      RST_TRY(flush_pending());
+      if (wanted) {
+        RST_TRY(prof_begin(m, RST_KERNEL_GRAD_INPUT, i, 2.0 * mnk, dx_bytes));
+        RST_TRY(launch_gemm(e->stream, dx));
+        RST_TRY(prof_end(m));
+      }
+    }
+    if (wanted && mask) m->layers[pv].backward_absorbed = true;
     {
-      GemmDesc d{};
+      GemmDesc& d = pend.d;
+      d = GemmDesc{};
       d.A = cur; d.B = l.input; d.C = l.gw;
       d.M = (int)l.out; d.N = (int)l.in; d.K = (int)batch;
       d.lda = (long)l.out; d.ldb = (long)l.in; d.ldc = (long)l.in;
       d.a_kc = false; d.b_kc = false;
       d.epilogue = EPI_DIVIDE; d.divisor = n_rows;
       // the bias gradient (linear.rs:65-67) is accumulated by the same launch
-      const bool fused_bias = l.in > 0 && batch > 0;
-      d.colsum = fused_bias ? l.gb : nullptr;
+      pend.fused_bias = l.in > 0 && batch > 0;
+      d.colsum = pend.fused_bias ? l.gb : nullptr;
       d.colsum_div = n_rows;
       if (fused_lr) {
         d.sgd_parm = l.w;
-        d.sgd_bias = fused_bias ? l.b : nullptr;
+        d.sgd_bias = pend.fused_bias ? l.b : nullptr;
         d.sgd_lr = *fused_lr;
       }
-      double bytes = 8.0 * ((double)batch * l.out + (double)batch * l.in + (double)l.in * l.out);
-      if (fused_lr) bytes += 16.0 * ((double)l.in * l.out + l.out);  // read and write the parameters
-      RST_TRY(prof_begin(m, RST_KERNEL_GRAD_WEIGHT, i, 2.0 * mnk, bytes));
       d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
-      RST_TRY(launch_gemm(e->stream, d));
-      RST_TRY(prof_end(m));
-      if (!fused_bias) {
-        RST_TRY(prof_begin(m, RST_KERNEL_GRAD_BIAS, i, 0.0, 8.0 * ((double)batch * l.out + l.out)));
-        RST_TRY(launch_column_mean(e->stream, cur, l.gb, batch, l.out, n_rows));
-        RST_TRY(prof_end(m));
-        if (fused_lr) RST_TRY(launch_sgd_flat(e->stream, l.b, l.gb, l.out, *fused_lr));
-      }
+      pend.bytes = 8.0 * ((double)batch * l.out + (double)batch * l.in + (double)l.in * l.out);
+      if (fused_lr) pend.bytes += 16.0 * ((double)l.in * l.out + l.out);  // read and write the parameters
+      pend.flops = 2.0 * mnk;
+      pend.layer = i;
+      pend.grad = cur;
+      pend.active = true;
     }
     if (!wanted) { cur = nullptr; break; }
     cur = l.grad_in_buf;
   }
+  RST_TRY(flush_pending());
   if (input_grad) *input_grad = cur;
   // the caches are consumed (Option::take in linear.rs:61, relu.rs:26, cross_entropy.rs:46)
   m->forward_valid = false;
@@ -620,6 +659,13 @@ int rst_model_train_step(rst_model* m, const double* x, const double* truth, siz
 int rst_model_fuse_sgd(rst_model* m, int enabled) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
   m->fuse_sgd = enabled != 0;
+  drop_graph(m);
+  return RST_OK;
+}
+
+int rst_model_pair_gradients(rst_model* m, int enabled) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->pair_gradients = enabled != 0;
   drop_graph(m);
   return RST_OK;
 }

@@ -190,6 +190,10 @@ class DeviceModel:
         """Apply SGD inside the weight-gradient launches of train_step (default) or as a pass."""
         _ffi.check(self.engine.lib.rst_model_fuse_sgd(self.handle, 1 if on else 0))
 
+    def pair_gradients(self, on=True):
+        """Launch a layer's weight gradient in one grid with the next layer's input gradient."""
+        _ffi.check(self.engine.lib.rst_model_pair_gradients(self.handle, 1 if on else 0))
+
     def graph_enable(self, on=True):
         """Replay the step as a HIP graph (default) or launch its kernels one by one."""
         _ffi.check(self.engine.lib.rst_model_graph_enable(self.handle, 1 if on else 0))

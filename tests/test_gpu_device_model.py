@@ -209,3 +209,55 @@ def test_sgd_in_weight_gradient_epilogue_is_bit_identical(engine, oracle, name, 
         for (p, g), (q, h) in zip(models[0].parameters(), models[1].parameters()):
             assert np.array_equal(p.to_numpy(), q.to_numpy()), "step %d" % step
             assert np.array_equal(g.to_numpy(), h.to_numpy()), "step %d" % step
+
+
+PAIR_CASES = [
+    # layer widths at which the hidden input gradients are 256..511 tiles of 128x128 and the weight
+    # gradients at least 256: the two share a grid; the ragged net never pairs (tiles too few)
+    ("paired", [("linear", 2048, 2048), ("relu",)] * 3 + [("linear", 2048, 4096)], 2048),
+    ("paired_ragged_edges", [("linear", 2050, 2046), ("relu",), ("linear", 2046, 2064), ("relu",),
+                             ("linear", 2064, 2304)], 2064),
+    ("never_paired", README_MLP, 64),
+]
+
+
+@pytest.mark.parametrize("name,spec,batch", PAIR_CASES, ids=[c[0] for c in PAIR_CASES])
+@pytest.mark.parametrize("fused", [True, False], ids=["sgd_fused", "sgd_separate"])
+def test_paired_gradient_launches_are_bit_identical(engine, oracle, name, spec, batch, fused):
+    """The weight gradient of a layer launched in one grid with the next layer's input gradient
+    against the same launches one after the other: loss, parameters and gradients to the bit."""
+    import rstorch_amd as rs
+    weights = make_weights(oracle, spec, 91)
+    models = []
+    for paired in (True, False):
+        dm = rs.DeviceModel(spec)
+        dm.load_parameters(weights)
+        dm.fuse_sgd(fused)
+        dm.pair_gradients(paired)
+        dm.graph_enable(False)
+        models.append(dm)
+    x, y = batch_data(oracle, batch, models[0].in_width, models[0].out_width, 5, 0, True)
+    xd, yd = engine.from_numpy(x), engine.from_numpy(y)
+    models[0].profile_enable(True)
+    for step in range(2):
+        losses = [dm.train_step(xd, yd, 0.05) for dm in models]
+        assert losses[0] == losses[1], "step %d" % step
+        for (p, g), (q, h) in zip(models[0].parameters(), models[1].parameters()):
+            assert np.array_equal(p.to_numpy(), q.to_numpy()), "step %d" % step
+            assert np.array_equal(g.to_numpy(), h.to_numpy()), "step %d" % step
+    kinds = [r["kernel"] for r in models[0].profile_read()]
+    n_linear = sum(1 for l in spec if l[0] == "linear")
+    if name == "never_paired":
+        assert "grad_pair" not in kinds
+    else:
+        # per step: the last layer's input gradient goes alone (nothing is pending yet), every other
+        # wanted one rides with the weight gradient of the layer above, and the two lowest weight
+        # gradients go alone (the first layer's input gradient is not computed)
+        assert kinds.count("grad_pair") == 2 * (n_linear - 2)
+        assert kinds.count("grad_input") == 2 and kinds.count("grad_weight") == 4
+    models[0].profile_enable(False)
+    # the piecewise backward (rst_model_backward) takes the same path
+    for dm in models:
+        dm.forward(xd); dm.loss(yd, want_value=False)
+    gins = [dm.backward(None, need_input_grad=True).to_numpy() for dm in models]
+    assert np.array_equal(gins[0], gins[1])
