@@ -510,35 +510,41 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
   const int wm = wave / WGN, wn = wave % WGN;
   const int lr = lane & 15, lk = lane >> 4;
 
-  const double* ga[CH];
-  const double* gb[CH];
+  // Tile DMA addressing: a uniform byte pointer per operand (tile origin, advanced along K by
+  // scalar adds) plus one constant 32-bit lane offset per chunk, so that issuing a tile costs no
+  // vector ALU work at all; the LDS destinations are uniform too (the wavefront number is read
+  // into a scalar register).
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const char* a_ptr = reinterpret_cast<const char*>(p.A + (A_KC ? (size_t)m0 * p.lda : (size_t)m0));
+  const char* b_ptr = reinterpret_cast<const char*>(p.B + (B_KC ? (size_t)n0 * p.ldb : (size_t)n0));
+  uint32_t ao[CH], bo[CH];
   int la[CH], lb[CH];
 #pragma unroll
   for (int h = 0; h < CH; ++h) {
-    const int c = wave + NW * h;
+    const int c = wave + NW * h, cs = wave_s + NW * h;
     if (A_KC) {
       const int row = 8 * c + (lane >> 3);
-      int gr = m0 + row; gr = gr < p.M ? gr : p.M - 1;
-      ga[h] = p.A + (size_t)gr * p.lda + 2 * ((lane & 7) ^ (row & 7));
-      la[h] = c * 128;
+      const int rr = m0 + row < p.M ? row : p.M - 1 - m0;
+      ao[h] = 8u * (uint32_t)((size_t)rr * p.lda + 2 * ((lane & 7) ^ (row & 7)));
+      la[h] = cs * 128;
     } else {
-      int ge = m0 + 2 * lane; ge = ge + 1 < p.M ? ge : p.M - 2;
-      ga[h] = p.A + (size_t)c * p.lda + ge;
-      la[h] = c * (BM + 16);
+      const int ge = m0 + 2 * lane + 1 < p.M ? 2 * lane : p.M - 2 - m0;
+      ao[h] = 8u * (uint32_t)((size_t)c * p.lda + ge);
+      la[h] = cs * (BM + 16);
     }
     if (B_KC) {
       const int row = 8 * c + (lane >> 3);
-      int gr = n0 + row; gr = gr < p.N ? gr : p.N - 1;
-      gb[h] = p.B + (size_t)gr * p.ldb + 2 * ((lane & 7) ^ (row & 7));
-      lb[h] = c * 128;
+      const int rr = n0 + row < p.N ? row : p.N - 1 - n0;
+      bo[h] = 8u * (uint32_t)((size_t)rr * p.ldb + 2 * ((lane & 7) ^ (row & 7)));
+      lb[h] = cs * 128;
     } else {
-      int ge = n0 + 2 * lane; ge = ge + 1 < p.N ? ge : p.N - 2;
-      gb[h] = p.B + (size_t)c * p.ldb + ge;
-      lb[h] = c * (BN + 16);
+      const int ge = n0 + 2 * lane + 1 < p.N ? 2 * lane : p.N - 2 - n0;
+      bo[h] = 8u * (uint32_t)((size_t)c * p.ldb + ge);
+      lb[h] = cs * (BN + 16);
     }
   }
-  const long a_step = A_KC ? BK : (long)BK * p.lda;
-  const long b_step = B_KC ? BK : (long)BK * p.ldb;
+  const long a_step = 8 * (A_KC ? BK : (long)BK * p.lda);  // bytes per K step
+  const long b_step = 8 * (B_KC ? BK : (long)BK * p.ldb);
 
   v4d acc[TM][TN];
 #pragma unroll
@@ -551,19 +557,19 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
   const int kt0 = split * p.steps_per_split;
   const int nk = (p.split_k > 1) ? ((nk_all - kt0 < p.steps_per_split) ? nk_all - kt0 : p.steps_per_split)
                                  : nk_all;
-#pragma unroll
-  for (int h = 0; h < CH; ++h) {
-    ga[h] += (long)kt0 * a_step;
-    gb[h] += (long)kt0 * b_step;
-  }
+  a_ptr += (long)kt0 * a_step;
+  b_ptr += (long)kt0 * b_step;
   auto issue = [&](int stage) {
 #pragma unroll
     for (int h = 0; h < CH; ++h) {
-      dma16(ga[h], lds_a + stage * A_SIZE + la[h]);
-      dma16(gb[h], lds_b + stage * B_SIZE + lb[h]);
-      ga[h] += a_step;
-      gb[h] += b_step;
+      // the empty asm keeps the zero-extension of the offset next to the load, where instruction
+      // selection can fold "scalar base + 32-bit lane offset" into the load's addressing mode
+      asm volatile("" : "+v"(ao[h]), "+v"(bo[h]));
+      dma16(reinterpret_cast<const double*>(a_ptr + ao[h]), lds_a + stage * A_SIZE + la[h]);
+      dma16(reinterpret_cast<const double*>(b_ptr + bo[h]), lds_b + stage * B_SIZE + lb[h]);
     }
+    a_ptr += a_step;
+    b_ptr += b_step;
   };
   // prologue: tiles 0 .. DIST-1 in flight, tile 0 landed
 #pragma unroll
@@ -817,7 +823,9 @@ int launch_layout(hipStream_t stream, const GemmParams& p) {
     return (long long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
   };
   if (tiles(128, 128) >= 256) {
-    if (VEC && p.K % BK == 0 && p.K > 0 && p.M >= 2 && p.N >= 2) return launch_dma<A_KC, B_KC>(stream, p);
+    // (leading dimensions below 2^22 doubles keep the 32-bit lane offsets of the tile DMA in range)
+    if (VEC && p.K % BK == 0 && p.K > 0 && p.M >= 2 && p.N >= 2 && p.lda < (1L << 22) && p.ldb < (1L << 22))
+      return launch_dma<A_KC, B_KC>(stream, p);
     return launch_one<128, 128, 2, 4, A_KC, B_KC, VEC>(stream, p);
   }
   if (tiles(64, 64) >= 1024) return launch_one<64, 64, 2, 2, A_KC, B_KC, VEC>(stream, p);
@@ -858,6 +866,7 @@ GemmParams make_params(const GemmDesc& d) {
 // true when launch_gemm would run d as unsplit 128x128 direct-to-LDS tiles
 bool takes_plain_dma(const GemmDesc& d, long long* blocks) {
   if (d.M < 2 || d.N < 2 || d.K <= 0 || d.K % BK != 0 || !desc_vec_ok(d)) return false;
+  if (d.lda >= (1L << 22) || d.ldb >= (1L << 22)) return false;
   *blocks = (long long)((d.M + 127) / 128) * ((d.N + 127) / 128);
   if (*blocks < 256) return false;
   return !(*blocks < 512 && d.K / BK >= kSplitMinSteps && d.workspace != nullptr);
