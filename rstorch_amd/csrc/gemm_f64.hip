@@ -753,7 +753,7 @@ int launch_split_reduce(hipStream_t stream, const GemmParams& p) {
   return RST_OK;
 }
 
-constexpr int kSplitMinSteps = 384;  // K >= 6144
+constexpr int kSplitMinSteps = 1536;  // K >= 24576
 
 template <bool A_KC, bool B_KC>
 int launch_dma(hipStream_t stream, GemmParams p) {
@@ -763,10 +763,11 @@ int launch_dma(hipStream_t stream, GemmParams p) {
   p.steps_per_split = p.K / BK;
   long long blocks = (long long)p.tiles_m * p.tiles_n;
   // Two independent workgroups per compute unit interleave their barriers and LDS waits: measured
-  // on 256 tiles, the K loop runs at 92.6 % of the MFMA peak with two against 88.2 % with one.
+  // on 256 tiles, the K loop runs about 1.5 points of the MFMA peak faster with two than with one.
   // With fewer than 512 tiles K can be cut in two halves so that every CU gets two workgroups;
   // the two partial products are then added (in slice order) by split_reduce_kernel, a fixed cost
-  // of about 31 us per launch at 1024 x 4096 outputs, which pays off from K of about 5400 on.
+  // of about 30 us per launch at 1024 x 4096 outputs: level at K = 16384 (1838 us unsplit, 1847
+  // split), 0.5 % ahead at K = 32768.
   const int nk = p.K / BK;
   const size_t need = 2 * ((size_t)p.M * p.N + (size_t)p.M);
   if (blocks < 512 && nk >= kSplitMinSteps && p.ws != nullptr && p.ws_capacity >= need) {

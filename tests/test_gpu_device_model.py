@@ -180,8 +180,8 @@ FUSE_CASES = [
     ("readme_b4096", README_MLP, 4096),
     ("ragged", [("identity",), ("linear", 33, 65), ("relu",), ("identity",), ("linear", 65, 129),
                 ("relu",), ("linear", 129, 7)], 67),
-    ("two_way_split", [("linear", 6144, 2048), ("relu",), ("linear", 2048, 6144)], 2048),
-    ("two_way_split_weight_gradient", [("linear", 2048, 2048), ("relu",), ("linear", 2048, 2560)], 6144),
+    ("two_way_split", [("linear", 24576, 2048), ("relu",), ("linear", 2048, 24576)], 2048),
+    ("two_way_split_weight_gradient", [("linear", 2048, 2048), ("relu",), ("linear", 2048, 2560)], 24576),
     ("full_grid", [("linear", 1024, 4096), ("relu",), ("linear", 4096, 4096), ("relu",),
                    ("linear", 4096, 1000)], 512),
 ]

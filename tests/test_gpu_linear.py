@@ -27,10 +27,8 @@ SHAPES = [
     # >= 256 tiles of 128x128 with ragged edges: the direct-to-LDS kernels (K % 16 == 0) and the
     # register-staged kernel with a K tail, for each of the three operand layouts
     (2050, 64, 2046), (2064, 2046, 2046), (2050, 2046, 2048),
-    # 256..511 tiles with a long contraction (K >= 6144): the direct-to-LDS kernels cut K in two
-    # halves - forward, input gradient and weight gradient (+ bias gradient over slices) in turn;
-    # (2064, 2048, 2046) is the same tile count below the threshold
-    (2064, 2048, 2046), (2064, 6144, 2046), (2064, 2048, 6144), (6144, 2048, 2046),
+    # 256..511 tiles: one workgroup per CU on the direct-to-LDS kernels
+    (2064, 2048, 2046),
     # small outputs with a long contraction: the split-K path (with and without a K tail)
     (8192, 784, 100), (8192, 100, 10), (32, 4099, 24), (4100, 7, 9), (16384, 33, 65),
 ]
@@ -66,6 +64,31 @@ def test_backward_matches_oracle(engine, oracle, batch, k, n):
     want_gw, want_gb, want_gx = oracle.linear_backward(g, x, w)
     params = list(lin.parameters())
     assert params[0].grad.shape == w.shape and params[1].grad.shape == b.shape
+    assert rel_err(params[0].grad.to_numpy(), want_gw) <= TOL
+    assert rel_err(params[1].grad.to_numpy(), want_gb) <= TOL
+    assert rel_err(gx, want_gx) <= TOL
+
+
+# 256..511 tiles with a very long contraction (K >= 24576): the direct-to-LDS kernels cut K in two
+# halves - forward, input gradient, and weight gradient (+ bias gradient over slices) in turn
+@pytest.mark.parametrize("batch,k,n", [(2048, 24576, 2046), (2064, 2048, 24576), (24576, 2048, 2046)])
+def test_two_way_k_split_matches_oracle(engine, oracle, batch, k, n):
+    import rstorch_amd as rs
+    rng = np.random.default_rng(batch + 3 * k + 7 * n)
+    x = rng.standard_normal((batch, k))
+    w = rng.standard_normal((n, k)) / np.sqrt(k)
+    b = rng.standard_normal((1, n))
+    g = rng.standard_normal((batch, n))
+    lin = _linear(rs, w, b)
+    out = lin._forward(x, True).to_numpy()
+    gx = lin.backward(g).to_numpy()
+    params = list(lin.parameters())
+    oracle.set_threads(8)
+    try:
+        assert rel_err(out, oracle.relu_forward(oracle.linear_forward(x, w, b))) <= TOL
+        want_gw, want_gb, want_gx = oracle.linear_backward(g, x, w)
+    finally:
+        oracle.set_threads(1)
     assert rel_err(params[0].grad.to_numpy(), want_gw) <= TOL
     assert rel_err(params[1].grad.to_numpy(), want_gb) <= TOL
     assert rel_err(gx, want_gx) <= TOL
