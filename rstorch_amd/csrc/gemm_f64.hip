@@ -56,6 +56,10 @@ struct GemmParams {
   double* ws;
   double* ws_colsum;
   size_t ws_capacity;    // doubles available at ws
+  // 128x128 direct-to-LDS kernel, launches of more than one round of workgroups: the workgroups of
+  // the first round that sit in the upper wave slots of their CU start this many 10 ns ticks late
+  int dephase_ticks;
+  int first_round;       // workgroups that fit on the chip at once
 };
 
 // LDS geometry of one operand tile of EXT rows/cols by BK contraction steps.
@@ -199,10 +203,8 @@ __device__ __forceinline__ void store_block(const GemmParams& p, const v4d* acc,
           for (int r = 0; r < 4; ++r) {
             const int row = row0 + (i0 + ii) * 16 + 4 * r + lk;
             const int rc = row < p.M ? row : p.M - 1;
-            // a parameter is read once and rewritten once per step: keep it out of the caches
-            extra[ii][j][r] = (EPI == EPI_MASK)
-                                  ? p.mask[(size_t)rc * p.ldmask + cc]
-                                  : __builtin_nontemporal_load(p.sgd_parm + (size_t)rc * p.ldc + cc);
+            extra[ii][j][r] = (EPI == EPI_MASK) ? p.mask[(size_t)rc * p.ldmask + cc]
+                                                : p.sgd_parm[(size_t)rc * p.ldc + cc];
           }
       }
     }
@@ -225,9 +227,9 @@ __device__ __forceinline__ void store_block(const GemmParams& p, const v4d* acc,
               __builtin_nontemporal_store(v, p.C + (size_t)row * p.ldc + col);
             else
               p.C[(size_t)row * p.ldc + col] = v;
-            if (SGD)
-              __builtin_nontemporal_store(sgd_apply(extra[ii][j][r], v, p.sgd_lr),
-                                          p.sgd_parm + (size_t)row * p.ldc + col);
+            // the parameter is read and rewritten through the L2 (measured faster than streaming
+            // either side of the read-modify-write past it)
+            if (SGD) p.sgd_parm[(size_t)row * p.ldc + col] = sgd_apply(extra[ii][j][r], v, p.sgd_lr);
           }
         }
       }
@@ -571,6 +573,21 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
     a_ptr += a_step;
     b_ptr += b_step;
   };
+  // The two workgroups that share a CU start together and, with equal tiles, would also reach
+  // their epilogues together, round after round, and with them every other CU's: a burst of stores
+  // (and, with the SGD update, of parameter loads) during which the matrix cores idle.  For some
+  // tile lengths this costs 15-20 % of the launch (the weight gradient with SGD at K = 1800..2600).
+  // So, in the first round, the workgroup in the upper wave slots of its CU starts about a quarter
+  // of a tile late - the other has the CU to itself meanwhile, nothing is lost - and from then on
+  // the two alternate.  Only the timing depends on what the hardware ID register says.
+  if (p.dephase_ticks > 0 && block < p.first_round) {
+    const unsigned wave_slot = __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 4);  // HW_ID.WAVE_ID
+    if (wave_slot & 2) {
+      const unsigned long long t0 = __builtin_amdgcn_s_memrealtime();  // 100 MHz
+      while (__builtin_amdgcn_s_memrealtime() - t0 < (unsigned long long)p.dephase_ticks)
+        __builtin_amdgcn_s_sleep(32);
+    }
+  }
   // prologue: tiles 0 .. DIST-1 in flight, tile 0 landed
 #pragma unroll
   for (int d = 0; d < DIST; ++d)
@@ -755,6 +772,17 @@ int launch_split_reduce(hipStream_t stream, const GemmParams& p) {
 
 constexpr int kSplitMinSteps = 1536;  // K >= 24576
 
+int compute_units() {
+  static const int cus = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+      n = 256;
+    return n;
+  }();
+  return cus;
+}
+
 template <bool A_KC, bool B_KC>
 int launch_dma(hipStream_t stream, GemmParams p) {
   p.tiles_m = (p.M + 127) / 128;
@@ -777,6 +805,9 @@ int launch_dma(hipStream_t stream, GemmParams p) {
     blocks *= 2;
   }
   if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
+  // more than one round of workgroups (two per CU fit): stagger the first round by 0.4 us per K step
+  p.first_round = 2 * compute_units();
+  p.dephase_ticks = blocks > p.first_round ? (p.steps_per_split < 250 ? 40 * p.steps_per_split : 10000) : 0;
   hipLaunchKernelGGL((gemm_f64_mfma_dma<A_KC, B_KC, 2, 4, 2, 1>), dim3((unsigned)blocks),
                      dim3(512), 0, stream, p);
   RST_HIP(hipGetLastError());
@@ -861,6 +892,7 @@ GemmParams make_params(const GemmDesc& d) {
   p.split_k = 1; p.steps_per_split = 0;
   p.ws = d.workspace; p.ws_colsum = nullptr; p.ws_capacity = d.workspace ? d.workspace_count : 0;
   p.tiles_m = p.tiles_n = 0;
+  p.dephase_ticks = 0; p.first_round = 0;
   return p;
 }
 
