@@ -783,8 +783,9 @@ int compute_units() {
   return cus;
 }
 
+// want_split > 1: cut K into that many slices (the caller has checked the workspace)
 template <bool A_KC, bool B_KC>
-int launch_dma(hipStream_t stream, GemmParams p) {
+int launch_dma(hipStream_t stream, GemmParams p, int want_split = 0) {
   p.tiles_m = (p.M + 127) / 128;
   p.tiles_n = (p.N + 127) / 128;
   p.split_k = 1;
@@ -798,7 +799,12 @@ int launch_dma(hipStream_t stream, GemmParams p) {
   // split), 0.5 % ahead at K = 32768.
   const int nk = p.K / BK;
   const size_t need = 2 * ((size_t)p.M * p.N + (size_t)p.M);
-  if (blocks < 512 && nk >= kSplitMinSteps && p.ws != nullptr && p.ws_capacity >= need) {
+  if (want_split > 1) {
+    p.steps_per_split = (nk + want_split - 1) / want_split;
+    p.split_k = (nk + p.steps_per_split - 1) / p.steps_per_split;
+    p.ws_colsum = p.ws + (size_t)p.split_k * p.M * p.N;
+    blocks *= p.split_k;
+  } else if (blocks < 512 && nk >= kSplitMinSteps && p.ws != nullptr && p.ws_capacity >= need) {
     p.split_k = 2;
     p.steps_per_split = (nk + 1) / 2;
     p.ws_colsum = p.ws + (size_t)2 * p.M * p.N;
@@ -854,11 +860,25 @@ int launch_layout(hipStream_t stream, const GemmParams& p) {
   auto tiles = [&](int bm, int bn) {
     return (long long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
   };
-  if (tiles(128, 128) >= 256) {
-    // (leading dimensions below 2^22 doubles keep the 32-bit lane offsets of the tile DMA in range)
-    if (VEC && p.K % BK == 0 && p.K > 0 && p.M >= 2 && p.N >= 2 && p.lda < (1L << 22) && p.ldb < (1L << 22))
-      return launch_dma<A_KC, B_KC>(stream, p);
+  // (leading dimensions below 2^22 doubles keep the 32-bit lane offsets of the tile DMA in range)
+  const bool dma_ok = VEC && p.K % BK == 0 && p.K > 0 && p.M >= 2 && p.N >= 2 && p.lda < (1L << 22) &&
+                      p.ldb < (1L << 22);
+  const long long t128 = tiles(128, 128);
+  if (t128 >= 256) {
+    if (dma_ok) return launch_dma<A_KC, B_KC>(stream, p);
     return launch_one<128, 128, 2, 4, A_KC, B_KC, VEC>(stream, p);
+  }
+  // 32..255 tiles of 128x128 with a long contraction: the direct-to-LDS kernel on up to eight K
+  // slices (about two workgroups per CU, at least 32 K steps each) plus the ordered reduction
+  // beats the smaller register-staged tiles by far (128 tiles, K = 4096: 87 % of the MFMA peak
+  // against 62 %), as long as the slices still fill the chip.
+  if (dma_ok && p.ws != nullptr) {
+    const int nk = p.K / BK;
+    int s = (int)((512 + t128 - 1) / t128);
+    if (s > 8) s = 8;
+    while (s > 1 && nk / s < 32) --s;
+    while (s > 1 && p.ws_capacity < (size_t)s * ((size_t)p.M * p.N + (size_t)p.M)) --s;
+    if (s > 1 && t128 * s >= 256) return launch_dma<A_KC, B_KC>(stream, p, s);
   }
   if (tiles(64, 64) >= 1024) return launch_one<64, 64, 2, 2, A_KC, B_KC, VEC>(stream, p);
   return launch_one<32, 32, 2, 2, A_KC, B_KC, VEC>(stream, p);

@@ -29,6 +29,10 @@ SHAPES = [
     (2050, 64, 2046), (2064, 2046, 2046), (2050, 2046, 2048),
     # 256..511 tiles: one workgroup per CU on the direct-to-LDS kernels
     (2064, 2048, 2046),
+    # 32..255 tiles with a long contraction: the direct-to-LDS kernels on up to eight K slices
+    # (forward 128 tiles x 4 slices, input gradient 64 tiles x 8; ragged: 128 tiles x 4; weight
+    # gradient with its bias gradient over 4 slices)
+    (512, 2048, 4096), (498, 2048, 4094), (2048, 1024, 1000),
     # small outputs with a long contraction: the split-K path (with and without a K tail)
     (8192, 784, 100), (8192, 100, 10), (32, 4099, 24), (4100, 7, 9), (16384, 33, 65),
 ]
