@@ -417,7 +417,8 @@ __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm
 }
 
 // ---- 128x128 tiles fed by direct global -> LDS loads ------------------------------------------
-// The main path for large, aligned problems (K a multiple of 16, 16-byte aligned operands).
+// The main path for large problems with 16-byte aligned operands (even leading dimensions and
+// extents; K need not be a multiple of 16: its remainder is a masked extra tile).
 // global_load_lds_dwordx4 moves 16 bytes per lane straight into LDS (lane l lands at
 // base + 16*l), so no staging registers and no ds_write instructions are spent on the operand
 // tiles; a wavefront moves one 1 KiB chunk of a tile per instruction:
@@ -435,6 +436,24 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 __device__ __forceinline__ void dma16(const double* g, double* lds_wave_base) {
   // every lane moves 16 bytes; lane l lands at lds_wave_base + 16*l
   __builtin_amdgcn_global_load_lds((gbl_ptr_t)g, (lds_ptr_t)(uintptr_t)lds_wave_base, 16, 0, 0);
+}
+
+// Registers -> LDS in the layouts of the DMA tiles (for the masked K tail): pair q of the tile as
+// load_tile numbers them.
+template <int EXT, bool KC, int THREADS>
+__device__ __forceinline__ void store_tile_dma(double* __restrict__ lds, const v2d* __restrict__ reg,
+                                               int tid) {
+  constexpr int L = EXT * BK / 2 / THREADS;
+#pragma unroll
+  for (int u = 0; u < L; ++u) {
+    const int q = tid + u * THREADS;
+    if (KC) {
+      const int e = q >> 3, pr = q & 7;  // row, pair k/2
+      *reinterpret_cast<v2d*>(lds + e * BK + 2 * (pr ^ (e & 7))) = reg[u];
+    } else {
+      *reinterpret_cast<v2d*>(lds + (q / (EXT / 2)) * (EXT + 16) + 2 * (q % (EXT / 2))) = reg[u];
+    }
+  }
 }
 
 __device__ __forceinline__ void wait_vmcnt(int n) {
@@ -472,7 +491,7 @@ __device__ __forceinline__ void read_quad(v2d& q, uint32_t addr) {
 }
 
 // Work of one workgroup: output tile number `block` (and its K slice) of problem p.  lds_a / lds_b
-// are the workgroup's STAGES operand stages (kDmaStage doubles each).
+// are the workgroup's STAGES operand stages (A_SIZE / B_SIZE doubles each, at most kDmaStage).
 constexpr int kDmaStage = BK * (128 + 16);  // the larger of the two tile layouts
 
 template <bool A_KC, bool B_KC, int WGM, int WGN, int STAGES, int DIST>
@@ -554,11 +573,15 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
 
-  // K steps of this workgroup: all of them, or slice `split` of a split contraction
+  // K steps of this workgroup: all whole ones, or slice `split` of a split contraction.  What is
+  // left of K beyond its last whole step (K % 16 indices) is an extra first tile of slice 0, copied
+  // into stage 0 by ordinary masked loads; the whole steps follow through the DMA pipeline.
   const int nk_all = p.K / BK;
   const int kt0 = split * p.steps_per_split;
-  const int nk = (p.split_k > 1) ? ((nk_all - kt0 < p.steps_per_split) ? nk_all - kt0 : p.steps_per_split)
-                                 : nk_all;
+  const int nk_dma = (p.split_k > 1) ? ((nk_all - kt0 < p.steps_per_split) ? nk_all - kt0 : p.steps_per_split)
+                                     : nk_all;
+  const bool k_tail = (p.K % BK) != 0 && split == 0;
+  const int nk = nk_dma + (k_tail ? 1 : 0);
   a_ptr += (long)kt0 * a_step;
   b_ptr += (long)kt0 * b_step;
   auto issue = [&](int stage) {
@@ -588,12 +611,20 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
         __builtin_amdgcn_s_sleep(32);
     }
   }
-  // prologue: tiles 0 .. DIST-1 in flight, tile 0 landed
-#pragma unroll
-  for (int d = 0; d < DIST; ++d)
-    if (d < nk) issue(d);
-  if (nk >= DIST) wait_vmcnt((DIST - 1) * 2 * CH); else wait_vmcnt(0);
-  __builtin_amdgcn_s_barrier();
+  // prologue: tile 0 in stage 0
+  static_assert(DIST == 1, "the prologue puts exactly one tile in flight");
+  if (k_tail) {
+    v2d ra[(BM * BK / 2) / (NW * 64)], rb[(BN * BK / 2) / (NW * 64)];
+    load_tile<BM, A_KC, true, true, NW * 64>(ra, p.A, p.lda, m0, p.M, nk_all * BK, p.K, tid);
+    load_tile<BN, B_KC, true, true, NW * 64>(rb, p.B, p.ldb, n0, p.N, nk_all * BK, p.K, tid);
+    store_tile_dma<BM, A_KC, NW * 64>(lds_a, ra, tid);
+    store_tile_dma<BN, B_KC, NW * 64>(lds_b, rb, tid);
+    __syncthreads();
+  } else {
+    if (nk > 0) issue(0);
+    wait_vmcnt(0);
+    __builtin_amdgcn_s_barrier();
+  }
 
   const bool do_colsum = !A_KC && p.colsum != nullptr && tile_n == 0;
   double colsum_partial = 0.0;
@@ -861,8 +892,7 @@ int launch_layout(hipStream_t stream, const GemmParams& p) {
     return (long long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
   };
   // (leading dimensions below 2^22 doubles keep the 32-bit lane offsets of the tile DMA in range)
-  const bool dma_ok = VEC && p.K % BK == 0 && p.K > 0 && p.M >= 2 && p.N >= 2 && p.lda < (1L << 22) &&
-                      p.ldb < (1L << 22);
+  const bool dma_ok = VEC && p.K > 0 && p.M >= 2 && p.N >= 2 && p.lda < (1L << 22) && p.ldb < (1L << 22);
   const long long t128 = tiles(128, 128);
   if (t128 >= 256) {
     if (dma_ok) return launch_dma<A_KC, B_KC>(stream, p);

@@ -33,6 +33,8 @@ SHAPES = [
     # (forward 128 tiles x 4 slices, input gradient 64 tiles x 8; ragged: 128 tiles x 4; weight
     # gradient with its bias gradient over 4 slices)
     (512, 2048, 4096), (498, 2048, 4094), (2048, 1024, 1000),
+    # the same with a K remainder (a masked extra tile in slice 0), and K below one whole step
+    (512, 2056, 4096), (2048, 1000, 4096), (2048, 10, 2048),
     # small outputs with a long contraction: the split-K path (with and without a K tail)
     (8192, 784, 100), (8192, 100, 10), (32, 4099, 24), (4100, 7, 9), (16384, 33, 65),
 ]
