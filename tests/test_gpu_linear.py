@@ -169,3 +169,44 @@ def test_backward_twice_raises(engine):
         lin.backward(np.ones((4, 2)))  # cache consumed (linear.rs:61)
     with pytest.raises(rs.ShapeError):
         lin.forward(np.ones((4, 5)))
+
+
+def _sweep_cases():
+    rng = np.random.default_rng(12345)
+    cases = []
+    for _ in range(36):
+        kind = int(rng.integers(0, 4))
+        if kind == 0:    # hundreds of 128x128 tiles, dimensions a little off the tile grid
+            b, k, n = (int(rng.integers(3, 36)) * 64 + int(rng.choice([0, 2, 6, 14])) for _ in range(3))
+        elif kind == 1:  # few tiles and a long contraction (K slices), with and without a K remainder
+            b = int(rng.integers(1, 8)) * 128 + int(rng.choice([0, 2, 30]))
+            n = int(rng.integers(2, 20)) * 128 - int(rng.choice([0, 2, 100]))
+            k = int(rng.integers(20, 300)) * 16 + int(rng.choice([0, 2, 8, 14]))
+        elif kind == 2:  # odd sizes: nothing is aligned
+            b, k, n = (int(rng.integers(1, 900)) for _ in range(3))
+        else:            # long batch, narrow layers
+            b = int(rng.integers(100, 5000)) * 2
+            k = int(rng.integers(1, 60)) * 2
+            n = int(rng.integers(1, 60)) * 2
+        cases.append((b, k, n))
+    return cases
+
+
+@pytest.mark.parametrize("batch,k,n", _sweep_cases())
+def test_seeded_shape_sweep_matches_numpy(engine, batch, k, n):
+    """Every kernel-selection path (tile sizes, K slices, K remainder, unaligned fallbacks) on seeded
+    random shapes, forward with fused ReLU and backward with the fused mask, against numpy float64."""
+    import rstorch_amd as rs
+    rng = np.random.default_rng(batch * 31 + k * 17 + n)
+    x = rng.standard_normal((batch, k))
+    w = rng.standard_normal((n, k)) / np.sqrt(k)
+    b = rng.standard_normal((1, n))
+    g = rng.standard_normal((batch, n))
+    lin = _linear(rs, w, b)
+    out = lin._forward(x, True).to_numpy()
+    gx = lin._backward(g, True).to_numpy()
+    params = list(lin.parameters())
+    assert rel_err(out, np.maximum(x @ w.T + b, 0.0)) <= TOL
+    assert rel_err(gx, (g @ w) * (x > 0)) <= TOL
+    assert rel_err(params[0].grad.to_numpy(), g.T @ x / batch) <= TOL
+    assert rel_err(params[1].grad.to_numpy(), g.sum(0, keepdims=True) / batch) <= TOL
