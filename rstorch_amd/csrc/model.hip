@@ -88,6 +88,7 @@ struct rst_model {
   // profiling
   bool profiling = false;
   bool slot_open = false;
+  bool chain_open = false;  // the last slot's stop event is the latest thing on the stream
   std::vector<ProfileSlot> slots;
   std::vector<hipEvent_t> event_pool;
   size_t events_used = 0;
@@ -144,9 +145,15 @@ int prof_begin(rst_model* m, int kind, int layer, double flops, double bytes) {
   }
   ProfileSlot s;
   s.kind = kind; s.layer = layer; s.flops = flops; s.bytes = bytes;
-  s.start = m->event_pool[m->events_used++];
+  // launches that follow each other inside one call share an event: the stop of one is the start
+  // of the next (one marker between two kernels instead of two)
+  if (m->chain_open) {
+    s.start = m->slots.back().stop;
+  } else {
+    s.start = m->event_pool[m->events_used++];
+    RST_HIP(hipEventRecord(s.start, m->engine->stream));
+  }
   s.stop = m->event_pool[m->events_used++];
-  RST_HIP(hipEventRecord(s.start, m->engine->stream));
   m->slots.push_back(s);
   m->slot_open = true;
   return RST_OK;
@@ -156,12 +163,14 @@ int prof_end(rst_model* m) {
   if (!m->slot_open) return RST_OK;
   m->slot_open = false;
   RST_HIP(hipEventRecord(m->slots.back().stop, m->engine->stream));
+  m->chain_open = true;
   return RST_OK;
 }
 
 void prof_reset(rst_model* m) {
   m->slots.clear();
   m->events_used = 0;
+  m->chain_open = false;
 }
 
 int prev_non_identity(const rst_model* m, int i) {
@@ -545,6 +554,7 @@ int rst_model_init_kaiming(rst_model* m, uint64_t seed, uint64_t first_stream) {
 
 int rst_model_forward(rst_model* m, const double* x, size_t batch, const double** logits) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->chain_open = false;  // whatever ran on the stream since the last profiled launch is not ours
   RST_TRY(engine_activate(m->engine));
   if (!x && batch) return fail(RST_ERR_INVALID_ARGUMENT, "x is null");
   RST_TRY(do_forward(m, x, batch));
@@ -554,6 +564,7 @@ int rst_model_forward(rst_model* m, const double* x, size_t batch, const double*
 
 int rst_model_loss(rst_model* m, const double* truth, double* host_loss) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->chain_open = false;  // whatever ran on the stream since the last profiled launch is not ours
   RST_TRY(engine_activate(m->engine));
   return do_loss(m, truth, host_loss);
 }
@@ -561,12 +572,14 @@ int rst_model_loss(rst_model* m, const double* truth, double* host_loss) {
 int rst_model_backward(rst_model* m, const double* grad, int need_input_grad,
                        const double** input_grad) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->chain_open = false;
   RST_TRY(engine_activate(m->engine));
   return do_backward(m, grad, need_input_grad, input_grad, nullptr);
 }
 
 int rst_model_sgd_step(rst_model* m, double lr) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->chain_open = false;  // whatever ran on the stream since the last profiled launch is not ours
   RST_TRY(engine_activate(m->engine));
   return do_sgd(m, lr);
 }
@@ -627,6 +640,7 @@ extern "C" {
 int rst_model_train_step(rst_model* m, const double* x, const double* truth, size_t batch,
                          double lr, double* host_loss) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->chain_open = false;
   rst_engine* e = m->engine;
   RST_TRY(engine_activate(e));
   if (!x || !truth) return fail(RST_ERR_INVALID_ARGUMENT, "x or truth is null");
