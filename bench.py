@@ -112,6 +112,33 @@ def summarise(recs, steps):
     return out
 
 
+def bench_relu(rs, eng, iters=20):
+    """The standalone ReLU kernels (what the module API runs when a ReLU does not follow or precede a
+    Linear layer) over 2^27 doubles: 16 B per element forward, 24 B per element backward."""
+    from rstorch_amd import _ffi
+    n = 1 << 27
+    x = eng.normal(1, n, SEED, 3100)
+    g = eng.normal(1, n, SEED, 3101)
+    out = eng.empty(1, n)
+    res = {"elements": n}
+    for name, nbytes, call in (
+            ("forward", 16 * n, lambda: _ffi.check(eng.lib.rst_relu_forward(eng.handle, x.ptr, out.ptr, n))),
+            ("backward", 24 * n, lambda: _ffi.check(eng.lib.rst_relu_backward(eng.handle, g.ptr, x.ptr, out.ptr, n)))):
+        for _ in range(3):
+            call()
+        eng.synchronize()
+        ev0, ev1 = eng.event(), eng.event()
+        ev0.record()
+        for _ in range(iters):
+            call()
+        ev1.record()
+        eng.synchronize()
+        ms = ev0.elapsed_ms(ev1) / iters
+        res[name] = {"ms": ms, "achieved_gbps": nbytes / (ms * 1e-3) / 1e9,
+                     "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS}
+    return res
+
+
 def bench_sgd_c3(rs, eng, iters=20):
     """configs[3]: SGD::step alone over 64 x (Linear(2048,2048) weight + bias), ~268.6M params."""
     import ctypes
@@ -319,6 +346,7 @@ def main():
     if not args.no_extra:
         log("SGD alone (configs[3]) ...")
         result["sgd_c3"] = bench_sgd_c3(rs, eng)
+        result["relu_standalone"] = bench_relu(rs, eng)
         log("other configurations ...")
         result["other_configs"] = {
             "C0_readme_b32": bench_small(rs, eng, C01_SPEC, 32, False, 2000, 100),

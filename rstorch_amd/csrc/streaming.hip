@@ -8,6 +8,9 @@ namespace {
 
 typedef double v2d __attribute__((ext_vector_type(2)));
 constexpr int kBlock = 256;
+// one wavefront per workgroup streams a few per cent faster for the wide element-wise passes
+// (measured on MI355X for ReLU and SGD alike)
+constexpr int kStreamBlock = 64;
 
 inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
 
@@ -19,9 +22,9 @@ inline unsigned grid_for(size_t work_items, size_t per_block) {
 
 // ---- ReLU -----------------------------------------------------------------------------------
 // forward: out = max(x, 0); fmax returns the non-NaN operand, like f64::max in the reference.
-__global__ __launch_bounds__(kBlock) void relu_forward_v2(const v2d* __restrict__ x,
+__global__ __launch_bounds__(kStreamBlock) void relu_forward_v2(const v2d* __restrict__ x,
                                                          v2d* __restrict__ out, size_t n2) {
-  size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  size_t i = (size_t)blockIdx.x * kStreamBlock + threadIdx.x;
   if (i < n2) {
     v2d v = __builtin_nontemporal_load(x + i);
     v.x = fmax(v.x, 0.0);
@@ -35,10 +38,10 @@ __global__ __launch_bounds__(kBlock) void relu_forward_s(const double* __restric
   if (i < n) out[i] = fmax(x[i], 0.0);
 }
 // backward: out = g * (x > 0 ? 1 : 0), a real multiply so that inf * 0 stays NaN.
-__global__ __launch_bounds__(kBlock) void relu_backward_v2(const v2d* __restrict__ g,
+__global__ __launch_bounds__(kStreamBlock) void relu_backward_v2(const v2d* __restrict__ g,
                                                           const v2d* __restrict__ x,
                                                           v2d* __restrict__ out, size_t n2) {
-  size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+  size_t i = (size_t)blockIdx.x * kStreamBlock + threadIdx.x;
   if (i < n2) {
     v2d gv = __builtin_nontemporal_load(g + i);
     v2d xv = __builtin_nontemporal_load(x + i);
@@ -203,7 +206,7 @@ __global__ void zero_hits_kernel(unsigned long long* hits) { hits[0] = 0ull; }
 int launch_relu_forward(hipStream_t s, const double* x, double* out, size_t n) {
   if (n == 0) return RST_OK;
   if (n % 2 == 0 && aligned16(x) && aligned16(out)) {
-    hipLaunchKernelGGL(relu_forward_v2, dim3(grid_for(n / 2, kBlock)), dim3(kBlock), 0, s,
+    hipLaunchKernelGGL(relu_forward_v2, dim3(grid_for(n / 2, kStreamBlock)), dim3(kStreamBlock), 0, s,
                        reinterpret_cast<const v2d*>(x), reinterpret_cast<v2d*>(out), n / 2);
   } else {
     hipLaunchKernelGGL(relu_forward_s, dim3(grid_for(n, kBlock)), dim3(kBlock), 0, s, x, out, n);
@@ -215,7 +218,7 @@ int launch_relu_forward(hipStream_t s, const double* x, double* out, size_t n) {
 int launch_relu_backward(hipStream_t s, const double* g, const double* x, double* out, size_t n) {
   if (n == 0) return RST_OK;
   if (n % 2 == 0 && aligned16(g) && aligned16(x) && aligned16(out)) {
-    hipLaunchKernelGGL(relu_backward_v2, dim3(grid_for(n / 2, kBlock)), dim3(kBlock), 0, s,
+    hipLaunchKernelGGL(relu_backward_v2, dim3(grid_for(n / 2, kStreamBlock)), dim3(kStreamBlock), 0, s,
                        reinterpret_cast<const v2d*>(g), reinterpret_cast<const v2d*>(x),
                        reinterpret_cast<v2d*>(out), n / 2);
   } else {
