@@ -240,8 +240,10 @@ int rst_model_pair_gradients(rst_model* model, int enabled);
  * (x, truth, batch, lr) and replays the graph afterwards; a different argument re-records.
  * enabled == 0 switches to plain launches (profiling does so by itself).  Default: enabled. */
 int rst_model_graph_enable(rst_model* model, int enabled);
-/* Per-launch timing of the model's kernels: when enabled every launch is bracketed by events
- * on the engine's stream (this serialises nothing, the stream is already in order).  Records
+/* Per-launch timing of the model's kernels: when enabled an event is recorded on the engine's
+ * stream after every launch (and one before the first launch of a call); a launch's duration runs
+ * from the previous event to its own, so it includes the few microseconds between the previous
+ * kernel's end and its own start.  Records
  * accumulate over calls (up to 65536) until rst_model_profile_read, which waits for the stream,
  * copies up to `capacity` of them (host_records == NULL: only counts) and clears the list. */
 typedef struct rst_kernel_record {
