@@ -229,7 +229,7 @@ def bench_staged(rs, eng, spec, batch, normal, steps, warmup, in_place=False):
             "host_bytes_per_step": batch * (8 * n_in + 4), "final_loss": loss}
 
 
-def cpu_baseline(sample_batches=(32, 96)):
+def cpu_baseline(sample_batches=(64, 256)):
     """The oracle (CPU restatement of the reference) on the C4 network at two reduced batches.
     A step costs t(B) = a + b*B (a: SGD and operand packing, independent of the batch; b: the
     per-row contraction and loss work), so two timed steps give t(1024) = a + 1024*b."""
