@@ -6,8 +6,10 @@
 // gradient = -(truth - p).  Where truth is exactly 0 the term is 0 unless p is 0 or NaN
 // (0 * -inf = NaN in the reference), so ln is only evaluated where truth is non-zero.
 //
-// A row is kept in registers between the three phases, so each logit and each truth value is
-// read once and each gradient written once: 24 bytes per logit.
+// Rows of up to 2048 logits are kept in registers between the three phases, so each logit and
+// each truth value is read once and each gradient written once: 24 bytes per logit.  Wider rows
+// are walked twice (running maximum and sum first, then the probabilities); the second walk goes
+// backwards so that the most recently read part of the row is still in L2.
 #include <cfloat>
 
 #include "common.h"
@@ -58,11 +60,6 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
   constexpr int BLOCK = TPR > 256 ? TPR : 256;
   constexpr int RPB = BLOCK / TPR;
   __shared__ double red[3][TPR > 64 ? TPR / 64 : 1];
-  // Widest rows only (one 1024-thread workgroup per row, so one workgroup per compute unit and
-  // nothing else to overlap with): the first PF truth vectors of every thread are fetched
-  // straight into LDS (16 bytes per lane, no registers) while the exponentials are computed.
-  constexpr int PF = (CE && VEC == 2 && TPR == 1024 && IPT == 16) ? 8 : 0;
-  __shared__ __attribute__((aligned(1024))) double tstage[PF ? PF * TPR * 2 : 2];
 
   const int sub = threadIdx.x % TPR;
   const size_t row = (size_t)blockIdx.x * RPB + threadIdx.x / TPR;
@@ -92,18 +89,6 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
       }
     }
   }
-  if (PF) {
-    // wavefront w, vector i -> 1 KiB at tstage[(w*PF + i)*128]; lane l lands 16*l bytes in
-    double* wave_base = tstage + (size_t)(threadIdx.x >> 6) * PF * 128;
-#pragma unroll
-    for (int i = 0; i < PF; ++i) {
-      const size_t c = (size_t)(sub + i * TPR) * VEC;
-      if (row_ok && c < cols)
-        __builtin_amdgcn_global_load_lds(
-            (const __attribute__((address_space(1))) void*)(truth + base + c),
-            (__attribute__((address_space(3))) void*)(uintptr_t)(wave_base + i * 128), 16, 0, 0);
-    }
-  }
   mx = group_reduce<TPR, MaxOp>(mx, red[0]);
 
   double s = 0.0;
@@ -119,11 +104,6 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
     }
   }
   s = group_reduce<TPR, SumOp>(s, red[1]);
-  if (PF) {
-    // every direct-to-LDS load of this wavefront has landed before its slots are read
-    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
-    asm volatile("" ::: "memory");
-  }
 
   double lsum = 0.0;
 #pragma unroll
@@ -136,12 +116,7 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
     for (int e = 0; e < VEC; ++e) p[e] = x[i][e] / s;
     if (CE) {
       double t[VEC];
-      if (PF && i < PF) {
-        const v2d tv = *reinterpret_cast<const v2d*>(
-            tstage + ((size_t)(threadIdx.x >> 6) * PF + i) * 128 + 2 * (threadIdx.x & 63));
-        t[0] = tv.x;
-        t[VEC - 1] = tv.y;
-      } else if (VEC == 2) {
+      if (VEC == 2) {
         v2d tv = __builtin_nontemporal_load(reinterpret_cast<const v2d*>(truth + base + c));
         t[0] = tv.x;
         t[VEC - 1] = tv.y;
@@ -179,40 +154,135 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
   }
 }
 
-// Rows too long for registers: one 1024-thread workgroup per row, three passes over memory.
-template <bool CE>
-__global__ __launch_bounds__(1024) void softmax_long_rows_kernel(
+template <int VEC>
+__device__ __forceinline__ void load_vec(const double* p, double (&v)[VEC]) {
+  if (VEC == 2) {
+    const v2d t = *reinterpret_cast<const v2d*>(p);
+    v[0] = t.x;
+    v[VEC - 1] = t.y;
+  } else {
+    v[0] = *p;
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void load_vec_nt(const double* p, double (&v)[VEC]) {
+  if (VEC == 2) {
+    const v2d t = __builtin_nontemporal_load(reinterpret_cast<const v2d*>(p));
+    v[0] = t.x;
+    v[VEC - 1] = t.y;
+  } else {
+    v[0] = __builtin_nontemporal_load(p);
+  }
+}
+template <int VEC>
+__device__ __forceinline__ void store_vec_nt(double* p, const double (&v)[VEC]) {
+  if (VEC == 2) {
+    const v2d t = {v[0], v[VEC - 1]};
+    __builtin_nontemporal_store(t, reinterpret_cast<v2d*>(p));
+  } else {
+    __builtin_nontemporal_store(v[0], p);
+  }
+}
+
+// Rows wider than 2048 logits: one workgroup of BLOCK threads per row, several workgroups per
+// compute unit (128 registers per thread), so that the arithmetic of one row overlaps the memory
+// traffic of another.  First walk: every thread folds its share of the row into a running
+// maximum m and the sum s of exp(z - m), rescaling s when m grows; the workgroup then agrees on
+// the row maximum M and the row sum S = sum of s * exp(m - M).  Second walk, backwards: p =
+// exp(z - M) / S with the same operations as the register kernel, then the loss term and the
+// gradient.  S differs from a left-to-right sum only by rounding (relative 1e-16).
+template <int BLOCK, int VEC, bool CE>
+__global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) void softmax_wide_rows_kernel(
     const double* __restrict__ z, const double* __restrict__ truth, double* __restrict__ grad,
-    double* __restrict__ prob, double* __restrict__ row_loss, double* __restrict__ loss,
-    int* __restrict__ flags, size_t rows, size_t cols) {
-  constexpr int TPR = 1024;
-  __shared__ double red[3][TPR / 64];
+    double* __restrict__ prob, double* __restrict__ row_loss, int* __restrict__ flags, size_t cols) {
+  constexpr int UNR = 4;
+  constexpr size_t CHUNK = (size_t)UNR * BLOCK;
+  __shared__ double red[3][BLOCK / 64];
   const size_t row = blockIdx.x;
   const size_t base = row * cols;
-  (void)rows;
+  const double* zr = z + base;
+  const size_t units = cols / VEC;
+  const size_t full = units / CHUNK * CHUNK;
+
   bool saw_nan = false;
-  double mx = -DBL_MAX;
-  for (size_t c = threadIdx.x; c < cols; c += TPR) {
-    double v = z[base + c];
-    saw_nan |= (v != v);
-    mx = MaxOp::apply(mx, v);
-  }
-  mx = group_reduce<TPR, MaxOp>(mx, red[0]);
-  double s = 0.0;
-  for (size_t c = threadIdx.x; c < cols; c += TPR) s += exp(z[base + c] - mx);
-  s = group_reduce<TPR, SumOp>(s, red[1]);
-  double lsum = 0.0;
-  for (size_t c = threadIdx.x; c < cols; c += TPR) {
-    double p = exp(z[base + c] - mx) / s;
-    if (CE) {
-      double t = truth[base + c];
-      lsum += loss_term(t, p);
-      grad[base + c] = -(t - p);
+  double m = -DBL_MAX, s = 0.0;
+  for (size_t u0 = 0; u0 < full; u0 += CHUNK) {
+    double v[UNR][VEC];
+#pragma unroll
+    for (int i = 0; i < UNR; ++i) load_vec<VEC>(zr + (u0 + threadIdx.x + (size_t)i * BLOCK) * VEC, v[i]);
+    double cm = m;
+#pragma unroll
+    for (int i = 0; i < UNR; ++i) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        saw_nan |= (v[i][e] != v[i][e]);
+        cm = MaxOp::apply(cm, v[i][e]);
+      }
     }
-    if (prob) prob[base + c] = p;
+    if (cm > m) {
+      s *= exp(m - cm);
+      m = cm;
+    }
+#pragma unroll
+    for (int i = 0; i < UNR; ++i) {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) s += exp(v[i][e] - m);
+    }
+  }
+  for (size_t u = full + threadIdx.x; u < units; u += BLOCK) {
+    double v[VEC];
+    load_vec<VEC>(zr + u * VEC, v);
+    double cm = m;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      saw_nan |= (v[e] != v[e]);
+      cm = MaxOp::apply(cm, v[e]);
+    }
+    if (cm > m) {
+      s *= exp(m - cm);
+      m = cm;
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) s += exp(v[e] - m);
+  }
+  const double M = group_reduce<BLOCK, MaxOp>(m, red[0]);
+  s *= exp(m - M);
+  const double S = group_reduce<BLOCK, SumOp>(s, red[1]);
+
+  double lsum = 0.0;
+  auto finish = [&](size_t u, const double (&v)[VEC], const double (&t)[VEC]) {
+    double p[VEC], g[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      p[e] = exp(v[e] - M) / S;
+      if (CE) {
+        lsum += loss_term(t[e], p[e]);
+        g[e] = -(t[e] - p[e]);
+      }
+    }
+    if (CE) store_vec_nt<VEC>(grad + base + u * VEC, g);
+    if (prob) store_vec_nt<VEC>(prob + base + u * VEC, p);
+  };
+  for (size_t u = full + threadIdx.x; u < units; u += BLOCK) {
+    double v[VEC], t[VEC] = {};
+    load_vec<VEC>(zr + u * VEC, v);
+    if (CE) load_vec_nt<VEC>(truth + base + u * VEC, t);
+    finish(u, v, t);
+  }
+  for (size_t u0 = full; u0 > 0; u0 -= CHUNK) {
+    const size_t ub = u0 - CHUNK + threadIdx.x;
+    double v[UNR][VEC], t[UNR][VEC] = {};
+#pragma unroll
+    for (int i = UNR - 1; i >= 0; --i) load_vec<VEC>(zr + (ub + (size_t)i * BLOCK) * VEC, v[i]);
+    if (CE) {
+#pragma unroll
+      for (int i = UNR - 1; i >= 0; --i) load_vec_nt<VEC>(truth + base + (ub + (size_t)i * BLOCK) * VEC, t[i]);
+    }
+#pragma unroll
+    for (int i = UNR - 1; i >= 0; --i) finish(ub + (size_t)i * BLOCK, v[i], t[i]);
   }
   if (CE) {
-    lsum = group_reduce<TPR, SumOp>(lsum, red[2]);
+    lsum = group_reduce<BLOCK, SumOp>(lsum, red[2]);
     if (threadIdx.x == 0) row_loss[row] = lsum;
     if (saw_nan) atomicOr(&flags[0], 1);
   } else {
@@ -289,6 +359,20 @@ int launch_rows(hipStream_t s, const double* z, const double* t, double* grad, d
   return RST_OK;
 }
 
+template <int BLOCK, int VEC>
+int launch_wide(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
+                double* row_loss, int* flags, size_t rows, size_t cols, bool ce) {
+  if (rows > 0x7fffffffull) return fail(RST_ERR_UNSUPPORTED, "too many rows for one launch");
+  if (ce)
+    hipLaunchKernelGGL((softmax_wide_rows_kernel<BLOCK, VEC, true>), dim3((unsigned)rows), dim3(BLOCK), 0,
+                       s, z, t, grad, prob, row_loss, flags, cols);
+  else
+    hipLaunchKernelGGL((softmax_wide_rows_kernel<BLOCK, VEC, false>), dim3((unsigned)rows), dim3(BLOCK), 0,
+                       s, z, t, grad, prob, row_loss, flags, cols);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
+}
+
 template <int VEC>
 int dispatch(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
              double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce) {
@@ -296,17 +380,9 @@ int dispatch(hipStream_t s, const double* z, const double* t, double* grad, doub
   if (units <= 16 * 2) return launch_rows<16, 2, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
   if (units <= 64 * 4) return launch_rows<64, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
   if (units <= 256 * 4) return launch_rows<256, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
-  if (units <= 1024 * 4) return launch_rows<1024, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
-  if (units <= 1024 * 16) return launch_rows<1024, 16, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
-  if (rows > 0x7fffffffull) return fail(RST_ERR_UNSUPPORTED, "too many rows for one launch");
-  if (ce)
-    hipLaunchKernelGGL(softmax_long_rows_kernel<true>, dim3((unsigned)rows), dim3(1024), 0, s, z, t,
-                       grad, prob, row_loss, loss, flags, rows, cols);
-  else
-    hipLaunchKernelGGL(softmax_long_rows_kernel<false>, dim3((unsigned)rows), dim3(1024), 0, s, z, t,
-                       grad, prob, row_loss, loss, flags, rows, cols);
-  RST_HIP(hipGetLastError());
-  return RST_OK;
+  // measured on 32 Mi logits: 256 threads per row are ahead below about 12 Ki columns, 512 above
+  if (cols < 12288) return launch_wide<256, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
+  return launch_wide<512, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
 }
 
 inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }

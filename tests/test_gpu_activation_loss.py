@@ -80,8 +80,9 @@ def test_softmax_reference_known_answer(engine):
 
 
 @pytest.mark.parametrize("rows,cols", [(1, 1), (3, 2), (32, 10), (33, 11), (8, 64), (5, 100),
-                                       (17, 257), (64, 1000), (7, 1001), (4, 4096), (3, 8190),
-                                       (2, 32768), (2, 32770), (2, 40001)])
+                                       (17, 257), (64, 1000), (7, 1001), (9, 2048), (5, 2050), (6, 2051),
+                                       (4, 4096), (3, 8190), (3, 12288), (2, 12301), (2, 32768),
+                                       (2, 32770), (2, 40001), (1, 300000)])
 def test_softmax_matches_oracle(engine, oracle, rows, cols):
     rng = np.random.default_rng(rows * 65537 + cols)
     x = rng.standard_normal((rows, cols)) * 3.0
@@ -92,7 +93,7 @@ def test_softmax_matches_oracle(engine, oracle, rows, cols):
 
 
 def test_softmax_uniform_power_of_two_is_exact(engine):
-    for cols in (2, 16, 256, 4096):
+    for cols in (2, 16, 256, 4096, 32768):
         p = _softmax(engine, np.full((3, cols), 0.37))
         np.testing.assert_array_equal(p, np.full((3, cols), 1.0 / cols))
 
@@ -116,6 +117,32 @@ def test_softmax_nan_is_an_error(engine):
     y = np.zeros((2, 6)); y[0, 1] = -np.inf
     p = _softmax(engine, y)
     assert p[0, 1] == 0.0 and abs(p[0].sum() - 1.0) < 1e-15
+
+
+@pytest.mark.parametrize("cols", [2050, 4099, 16384, 33001])
+def test_softmax_wide_rows_special_values(engine, oracle, cols):
+    """Rows wider than 2048 logits are walked twice with a running maximum: the special values
+    must come out as in the reference's max-then-sum order."""
+    import rstorch_amd as rs
+    rng = np.random.default_rng(cols)
+    x = rng.standard_normal((6, cols))
+    x[0, cols // 3] = -np.inf                      # contributes exp(-inf) = 0
+    x[1, :] = -np.inf                              # all -inf: maximum stays at the lowest finite double, 0/0
+    x[2, cols - 1] = 700.0                         # the maximum arrives last: every partial sum is rescaled
+    x[3, 0] = 700.0                                # ... and first
+    x[4, :] = np.sort(x[4, :])                     # ever growing maximum
+    x[5, 5] = np.inf                               # inf - inf = NaN through the whole row (no NaN input)
+    got = _softmax(engine, x)
+    want = oracle.softmax(x)
+    assert got[0, cols // 3] == 0.0
+    assert np.all(np.isnan(got[1])) and np.all(np.isnan(want[1]))
+    assert np.all(np.isnan(got[5])) and np.all(np.isnan(want[5]))
+    ok = [0, 2, 3, 4]
+    assert rel_err(got[ok], want[ok]) <= TOL
+    assert np.all(np.abs(got[ok].sum(axis=1) - 1.0) <= 1e-12)
+    y = x[:1].copy(); y[0, cols // 2] = np.nan
+    with pytest.raises(rs.NanError):
+        _softmax(engine, y)
 
 
 # ---- the Softmax module (forward on both axes, batch-summed Jacobian backward) -----------------
@@ -152,7 +179,8 @@ def test_softmax_module_matches_oracle(engine, oracle, rows, cols, axis):
 
 # ---- CrossEntropyLoss ---------------------------------------------------------------------------
 @pytest.mark.parametrize("rows,cols", [(1, 2), (32, 10), (33, 11), (64, 100), (128, 1000),
-                                       (16, 4096), (4, 32768), (3, 33000)])
+                                       (9, 2048), (7, 2050), (5, 2051), (16, 4096), (6, 10000),
+                                       (5, 12289), (4, 32768), (3, 33000), (2, 100001)])
 def test_cross_entropy_matches_oracle(engine, oracle, rows, cols):
     import rstorch_amd as rs
     rng = np.random.default_rng(rows + 17 * cols)
@@ -180,6 +208,38 @@ def test_cross_entropy_soft_labels(engine, oracle):
     want, prob = oracle.cross_entropy_forward(z, t)
     assert abs(got - want) <= TOL * abs(want)
     assert rel_err(loss.backward().to_numpy(), prob - t) <= TOL
+
+
+@pytest.mark.parametrize("cols", [3000, 20000])
+def test_cross_entropy_soft_labels_wide_rows(engine, oracle, cols):
+    import rstorch_amd as rs
+    rng = np.random.default_rng(cols)
+    z = rng.standard_normal((5, cols)) * 3.0
+    t = rng.random((5, cols)); t /= t.sum(axis=1, keepdims=True)
+    loss = rs.CrossEntropyLoss.new()
+    got = loss.forward(z, t)
+    want, prob = oracle.cross_entropy_forward(z, t)
+    assert abs(got - want) <= TOL * abs(want)
+    assert rel_err(loss.backward().to_numpy(), prob - t) <= TOL
+
+
+@pytest.mark.parametrize("cols", [4100, 16384])
+def test_cross_entropy_wide_rows_underflow_and_nan(engine, oracle, cols):
+    """The wide-row kernel keeps the reference's 0 * ln(0) = NaN and its NaN-logit error."""
+    import rstorch_amd as rs
+    rng = np.random.default_rng(cols)
+    z = rng.standard_normal((3, cols))
+    t = np.zeros((3, cols)); t[np.arange(3), [1, 2, 3]] = 1.0
+    want, _ = oracle.cross_entropy_forward(z, t)
+    got = rs.CrossEntropyLoss.new().forward(z, t)
+    assert abs(got - want) <= TOL * abs(want)
+    z[1, cols - 7] = -900.0  # probability underflows to 0 where truth is 0
+    want, _ = oracle.cross_entropy_forward(z, t)
+    got = rs.CrossEntropyLoss.new().forward(z, t)
+    assert math.isnan(want) and math.isnan(got)
+    z[1, cols - 7] = np.nan
+    with pytest.raises(rs.NanError):
+        rs.CrossEntropyLoss.new().forward(z, t)
 
 
 def test_cross_entropy_closed_forms(engine):
