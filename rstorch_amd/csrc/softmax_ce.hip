@@ -190,26 +190,43 @@ __device__ __forceinline__ void store_vec_nt(double* p, const double (&v)[VEC]) 
 // maximum m and the sum s of exp(z - m), rescaling s when m grows; the workgroup then agrees on
 // the row maximum M and the row sum S = sum of s * exp(m - M).  Second walk, backwards: p =
 // exp(z - M) / S with the same operations as the register kernel, then the loss term and the
-// gradient.  S differs from a left-to-right sum only by rounding (relative 1e-16).
+// gradient.  S differs from a left-to-right sum only by rounding (relative 1e-16).  The first
+// PARK chunks of the row (PARK * 4 * BLOCK vectors, 32 KiB with 256 threads, 64 KiB with 512)
+// wait in LDS between the walks instead of being read again.
 template <int BLOCK, int VEC, bool CE>
 __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) void softmax_wide_rows_kernel(
     const double* __restrict__ z, const double* __restrict__ truth, double* __restrict__ grad,
     double* __restrict__ prob, double* __restrict__ row_loss, int* __restrict__ flags, size_t cols) {
   constexpr int UNR = 4;
+  constexpr int PARK = 2;
   constexpr size_t CHUNK = (size_t)UNR * BLOCK;
   __shared__ double red[3][BLOCK / 64];
+  __shared__ __attribute__((aligned(16))) double park[PARK * UNR * BLOCK * VEC];
   const size_t row = blockIdx.x;
   const size_t base = row * cols;
   const double* zr = z + base;
   const size_t units = cols / VEC;
-  const size_t full = units / CHUNK * CHUNK;
+  const size_t nchunk = units / CHUNK;
+  const size_t full = nchunk * CHUNK;
 
   bool saw_nan = false;
   double m = -DBL_MAX, s = 0.0;
-  for (size_t u0 = 0; u0 < full; u0 += CHUNK) {
+  for (size_t c = 0; c < nchunk; ++c) {
     double v[UNR][VEC];
+    const double* src = zr + (c * CHUNK + threadIdx.x) * VEC;
+    if (c < PARK) {
 #pragma unroll
-    for (int i = 0; i < UNR; ++i) load_vec<VEC>(zr + (u0 + threadIdx.x + (size_t)i * BLOCK) * VEC, v[i]);
+      for (int i = 0; i < UNR; ++i) load_vec_nt<VEC>(src + (size_t)i * BLOCK * VEC, v[i]);
+#pragma unroll
+      for (int i = 0; i < UNR; ++i) {
+        double* slot = park + ((c * UNR + i) * BLOCK + threadIdx.x) * VEC;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) slot[e] = v[i][e];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < UNR; ++i) load_vec<VEC>(src + (size_t)i * BLOCK * VEC, v[i]);
+    }
     double cm = m;
 #pragma unroll
     for (int i = 0; i < UNR; ++i) {
@@ -269,11 +286,21 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) v
     if (CE) load_vec_nt<VEC>(truth + base + u * VEC, t);
     finish(u, v, t);
   }
-  for (size_t u0 = full; u0 > 0; u0 -= CHUNK) {
-    const size_t ub = u0 - CHUNK + threadIdx.x;
+  for (size_t c = nchunk; c > 0; --c) {
+    const size_t cc = c - 1;
+    const size_t ub = cc * CHUNK + threadIdx.x;
     double v[UNR][VEC], t[UNR][VEC] = {};
+    if (cc < PARK) {
 #pragma unroll
-    for (int i = UNR - 1; i >= 0; --i) load_vec<VEC>(zr + (ub + (size_t)i * BLOCK) * VEC, v[i]);
+      for (int i = UNR - 1; i >= 0; --i) {
+        const double* slot = park + ((cc * UNR + i) * BLOCK + threadIdx.x) * VEC;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[i][e] = slot[e];
+      }
+    } else {
+#pragma unroll
+      for (int i = UNR - 1; i >= 0; --i) load_vec<VEC>(zr + (ub + (size_t)i * BLOCK) * VEC, v[i]);
+    }
     if (CE) {
 #pragma unroll
       for (int i = UNR - 1; i >= 0; --i) load_vec_nt<VEC>(truth + base + (ub + (size_t)i * BLOCK) * VEC, t[i]);
