@@ -762,14 +762,27 @@ __global__ __launch_bounds__(512, 4) void gemm_f64_mfma_dma_pair(const GemmParam
   }
 }
 
+// Sum of `count` values `stride` doubles apart, added in order; 32 loads are in flight at a time
+// (the slices were written by other XCDs, so every load is a trip to memory).
+__device__ __forceinline__ double ordered_slice_sum(const double* __restrict__ first, size_t stride, int count) {
+  double v = 0.0;
+  for (int s0 = 0; s0 < count; s0 += 32) {
+    double t[32];
+#pragma unroll
+    for (int j = 0; j < 32; ++j) t[j] = s0 + j < count ? first[(size_t)(s0 + j) * stride] : 0.0;
+#pragma unroll
+    for (int j = 0; j < 32; ++j)
+      if (s0 + j < count) v += t[j];
+  }
+  return v;
+}
+
 // Adds the K slices of a split contraction in slice order and applies the epilogue.
 __global__ __launch_bounds__(256) void split_reduce_kernel(const GemmParams p) {
   const size_t mn = (size_t)p.M * p.N;
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i < mn) {
-    double v = 0.0;
-#pragma unroll 8
-    for (int s = 0; s < p.split_k; ++s) v += p.ws[(size_t)s * mn + i];
+    double v = ordered_slice_sum(p.ws + i, mn, p.split_k);
     const int row = (int)(i / p.N), col = (int)(i - (size_t)row * p.N);
     switch (p.epilogue) {
       case EPI_BIAS: v = v + p.bias[col]; break;
@@ -786,8 +799,7 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const GemmParams p) {
     }
   }
   if (p.colsum != nullptr && i < (size_t)p.M) {
-    double t = 0.0;
-    for (int s = 0; s < p.split_k; ++s) t += p.ws_colsum[(size_t)s * p.M + i];
+    const double t = ordered_slice_sum(p.ws_colsum + i, (size_t)p.M, p.split_k);
     const double g = t / p.colsum_div;
     p.colsum[i] = g;
     if (p.sgd_bias) p.sgd_bias[i] = sgd_apply(p.sgd_bias[i], g, p.sgd_lr);
@@ -853,7 +865,7 @@ int launch_dma(hipStream_t stream, GemmParams p, int want_split = 0) {
 }
 
 template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
-int launch_one(hipStream_t stream, GemmParams p) {
+int launch_one(hipStream_t stream, GemmParams p, long long split_below = 256, long long want_blocks = 2048) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   long long blocks = (long long)p.tiles_m * p.tiles_n;
@@ -861,8 +873,8 @@ int launch_one(hipStream_t stream, GemmParams p) {
   const int nk = (p.K + BK - 1) / BK;
   p.split_k = 1;
   p.steps_per_split = nk;
-  if (blocks < 256 && nk >= 8 && p.ws != nullptr) {
-    long long want = (2048 + blocks - 1) / blocks;           // about eight workgroups per CU
+  if (blocks < split_below && nk >= 8 && p.ws != nullptr) {
+    long long want = (want_blocks + blocks - 1) / blocks;    // about eight workgroups per CU
     if (want > 64) want = 64;                                // keep the ordered reduction short
     long long max_by_steps = nk / 4;                         // at least 4 K steps per slice
     long long max_by_ws = (long long)(p.ws_capacity / ((size_t)p.M * p.N + (size_t)p.M));
