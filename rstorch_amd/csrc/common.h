@@ -78,6 +78,11 @@ int launch_gemm(hipStream_t stream, const GemmDesc& d);
 // under-fill the chip (fewer than 512 tiles).
 bool can_pair_gemm(const GemmDesc& input_grad, const GemmDesc& weight_grad);
 int launch_gemm_pair(hipStream_t stream, const GemmDesc& input_grad, const GemmDesc& weight_grad);
+// Several small weight gradients (both operands output-contiguous, each one unsplit launch of
+// fewer than 256 tiles of 32x32 on its own) in one grid; same results as launch_gemm on each.
+bool can_group_gemm(const GemmDesc& d);
+int max_gemm_group();
+int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count);
 
 // ---- streaming kernels -----------------------------------------------------------------------
 int launch_relu_forward(hipStream_t s, const double* x, double* out, size_t n);

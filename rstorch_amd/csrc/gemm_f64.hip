@@ -304,9 +304,9 @@ __device__ __forceinline__ void colsum_finish(double partial, double* __restrict
   }
 }
 
+// One output tile of the register-staged product: workgroup number `block` of problem p.
 template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
-__global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm_f64_mfma(
-    const GemmParams p) {
+__device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block) {
   constexpr int kThreads = WGM * WGN * 64;
   using GA = TileGeom<BM, A_KC, kThreads>;
   using GB = TileGeom<BN, B_KC, kThreads>;
@@ -321,10 +321,10 @@ __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm
   // its private L2) works on one compact patch of the tile grid, then walk the patch in
   // groups of 8 tile rows so that concurrently resident workgroups share operand panels.
   const int n_blocks = p.tiles_m * p.tiles_n;
-  const int split = blockIdx.x / n_blocks;  // K slice of this workgroup (0 without split-K)
+  const int split = block / n_blocks;  // K slice of this workgroup (0 without split-K)
   int logical;
   {
-    const int pid = blockIdx.x - split * n_blocks;
+    const int pid = block - split * n_blocks;
     const int xcd = pid & 7, local = pid >> 3;
     const int base = n_blocks >> 3, rem = n_blocks & 7;
     logical = xcd * base + (xcd < rem ? xcd : rem) + local;
@@ -414,6 +414,29 @@ __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm
   }
 
   write_block<TM, TN>(p, &acc[0][0], m0 + wm * WM, n0 + wn * WN, lr, lk, split);
+}
+
+template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
+__global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm_f64_mfma(
+    const GemmParams p) {
+  gemm_tile<BM, BN, WGM, WGN, A_KC, B_KC, VEC>(p, (int)blockIdx.x);
+}
+
+// Up to kMaxGroup small products of the same operand layouts in one grid of 32x32 tiles (the
+// weight gradients of a small network: each is a handful of tiles, and a launch of its own costs
+// more than its arithmetic).  Workgroups [first_block[i], first_block[i+1]) belong to problem i.
+constexpr int kMaxGroup = 8;
+struct GemmGroup {
+  int count;
+  int first_block[kMaxGroup + 1];
+  GemmParams p[kMaxGroup];
+};
+
+template <bool A_KC, bool B_KC>
+__global__ __launch_bounds__(256, 2) void gemm_f64_mfma_group(const GemmGroup g) {
+  int i = 0;
+  while (i + 1 < g.count && (int)blockIdx.x >= g.first_block[i + 1]) ++i;
+  gemm_tile<32, 32, 2, 2, A_KC, B_KC, true>(g.p[i], (int)blockIdx.x - g.first_block[i]);
 }
 
 // ---- 128x128 tiles fed by direct global -> LDS loads ------------------------------------------
@@ -864,28 +887,34 @@ int launch_dma(hipStream_t stream, GemmParams p, int want_split = 0) {
   return RST_OK;
 }
 
+// Few output tiles (`blocks` < split_below) but a long contraction: the number of K slices that
+// fills the chip (want_blocks workgroups, about eight per CU), 1 = none.
+long long small_tile_slices(const GemmParams& p, long long blocks, long long split_below, long long want_blocks) {
+  const int nk = (p.K + BK - 1) / BK;
+  if (!(blocks < split_below && nk >= 8 && p.ws != nullptr)) return 1;
+  long long want = (want_blocks + blocks - 1) / blocks;
+  if (want > 64) want = 64;                                // keep the ordered reduction short
+  const long long max_by_steps = nk / 4;                   // at least 4 K steps per slice
+  const long long max_by_ws = (long long)(p.ws_capacity / ((size_t)p.M * p.N + (size_t)p.M));
+  long long s = want < max_by_steps ? want : max_by_steps;
+  if (s > max_by_ws) s = max_by_ws;
+  return s > 1 ? s : 1;
+}
+
 template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
 int launch_one(hipStream_t stream, GemmParams p, long long split_below = 256, long long want_blocks = 2048) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   long long blocks = (long long)p.tiles_m * p.tiles_n;
-  // Few output tiles but a long contraction: cut K into slices so that the chip fills up.
   const int nk = (p.K + BK - 1) / BK;
   p.split_k = 1;
   p.steps_per_split = nk;
-  if (blocks < split_below && nk >= 8 && p.ws != nullptr) {
-    long long want = (want_blocks + blocks - 1) / blocks;    // about eight workgroups per CU
-    if (want > 64) want = 64;                                // keep the ordered reduction short
-    long long max_by_steps = nk / 4;                         // at least 4 K steps per slice
-    long long max_by_ws = (long long)(p.ws_capacity / ((size_t)p.M * p.N + (size_t)p.M));
-    long long s = want < max_by_steps ? want : max_by_steps;
-    if (s > max_by_ws) s = max_by_ws;
-    if (s > 1) {
-      p.steps_per_split = (int)((nk + s - 1) / s);
-      p.split_k = (nk + p.steps_per_split - 1) / p.steps_per_split;
-      p.ws_colsum = p.ws + (size_t)p.split_k * p.M * p.N;
-      blocks *= p.split_k;
-    }
+  const long long s = small_tile_slices(p, blocks, split_below, want_blocks);
+  if (s > 1) {
+    p.steps_per_split = (int)((nk + s - 1) / s);
+    p.split_k = (nk + p.steps_per_split - 1) / p.steps_per_split;
+    p.ws_colsum = p.ws + (size_t)p.split_k * p.M * p.N;
+    blocks *= p.split_k;
   }
   if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
   hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, WGM, WGN, A_KC, B_KC, VEC>), dim3((unsigned)blocks),
@@ -895,21 +924,20 @@ int launch_one(hipStream_t stream, GemmParams p, long long split_below = 256, lo
   return RST_OK;
 }
 
-template <bool A_KC, bool B_KC, bool VEC>
-int launch_layout(hipStream_t stream, const GemmParams& p) {
-  // 128x128 tiles once they fill the 256 compute units, 64x64 while that still leaves about
-  // four workgroups per CU to overlap each other's load latency, else 32x32 (which cuts the
-  // contraction into slices when even that gives too few workgroups).
+// Which kernel a product goes to.  128x128 tiles once they fill the 256 compute units, 64x64 while
+// that still leaves about four workgroups per CU to overlap each other's load latency, else 32x32
+// (which cuts the contraction into slices when even that gives too few workgroups).
+enum class Route { kDma, kDmaSliced, kTile128, kTile64, kTile32 };
+
+Route choose_route(const GemmParams& p, bool vec, int* dma_slices) {
   auto tiles = [&](int bm, int bn) {
     return (long long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
   };
   // (leading dimensions below 2^22 doubles keep the 32-bit lane offsets of the tile DMA in range)
-  const bool dma_ok = VEC && p.K > 0 && p.M >= 2 && p.N >= 2 && p.lda < (1L << 22) && p.ldb < (1L << 22);
+  const bool dma_ok = vec && p.K > 0 && p.M >= 2 && p.N >= 2 && p.lda < (1L << 22) && p.ldb < (1L << 22);
   const long long t128 = tiles(128, 128);
-  if (t128 >= 256) {
-    if (dma_ok) return launch_dma<A_KC, B_KC>(stream, p);
-    return launch_one<128, 128, 2, 4, A_KC, B_KC, VEC>(stream, p);
-  }
+  *dma_slices = 0;
+  if (t128 >= 256) return dma_ok ? Route::kDma : Route::kTile128;
   // 32..255 tiles of 128x128 with a long contraction: the direct-to-LDS kernel on up to eight K
   // slices (about two workgroups per CU, at least 32 K steps each) plus the ordered reduction
   // beats the smaller register-staged tiles by far (128 tiles, K = 4096: 87 % of the MFMA peak
@@ -920,10 +948,24 @@ int launch_layout(hipStream_t stream, const GemmParams& p) {
     if (s > 8) s = 8;
     while (s > 1 && nk / s < 32) --s;
     while (s > 1 && p.ws_capacity < (size_t)s * ((size_t)p.M * p.N + (size_t)p.M)) --s;
-    if (s > 1 && t128 * s >= 256) return launch_dma<A_KC, B_KC>(stream, p, s);
+    if (s > 1 && t128 * s >= 256) {
+      *dma_slices = s;
+      return Route::kDmaSliced;
+    }
   }
-  if (tiles(64, 64) >= 1024) return launch_one<64, 64, 2, 2, A_KC, B_KC, VEC>(stream, p);
-  return launch_one<32, 32, 2, 2, A_KC, B_KC, VEC>(stream, p);
+  return tiles(64, 64) >= 1024 ? Route::kTile64 : Route::kTile32;
+}
+
+template <bool A_KC, bool B_KC, bool VEC>
+int launch_layout(hipStream_t stream, const GemmParams& p) {
+  int slices = 0;
+  switch (choose_route(p, VEC, &slices)) {
+    case Route::kDma: return launch_dma<A_KC, B_KC>(stream, p);
+    case Route::kDmaSliced: return launch_dma<A_KC, B_KC>(stream, p, slices);
+    case Route::kTile128: return launch_one<128, 128, 2, 4, A_KC, B_KC, VEC>(stream, p);
+    case Route::kTile64: return launch_one<64, 64, 2, 2, A_KC, B_KC, VEC>(stream, p);
+    default: return launch_one<32, 32, 2, 2, A_KC, B_KC, VEC>(stream, p);
+  }
 }
 
 }  // namespace
@@ -980,6 +1022,40 @@ int launch_gemm(hipStream_t stream, const GemmDesc& d) {
   if (d.a_kc && !d.b_kc)
     return vec ? launch_layout<true, false, true>(stream, p) : launch_layout<true, false, false>(stream, p);
   return vec ? launch_layout<false, true, true>(stream, p) : launch_layout<false, true, false>(stream, p);
+}
+
+int max_gemm_group() { return kMaxGroup; }
+
+bool can_group_gemm(const GemmDesc& d) {
+  // the grouped kernel exists for the weight-gradient layouts with 16-byte loads
+  if (d.M <= 0 || d.N <= 0 || d.a_kc || d.b_kc || !desc_vec_ok(d)) return false;
+  const GemmParams p = make_params(d);
+  int slices = 0;
+  if (choose_route(p, true, &slices) != Route::kTile32) return false;
+  const long long blocks = (long long)((p.M + 31) / 32) * ((p.N + 31) / 32);
+  return small_tile_slices(p, blocks, 256, 2048) == 1;
+}
+
+int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count) {
+  if (count < 1 || count > kMaxGroup) return fail(RST_ERR_INVALID_ARGUMENT, "a group holds 1..%d contractions", kMaxGroup);
+  GemmGroup g{};
+  g.count = count;
+  long long blocks = 0;
+  for (int i = 0; i < count; ++i) {
+    if (!can_group_gemm(d[i])) return fail(RST_ERR_INVALID_ARGUMENT, "contraction %d cannot join a group", i);
+    GemmParams p = make_params(d[i]);
+    p.tiles_m = (p.M + 31) / 32;
+    p.tiles_n = (p.N + 31) / 32;
+    p.split_k = 1;
+    p.steps_per_split = (p.K + BK - 1) / BK;
+    g.first_block[i] = (int)blocks;
+    blocks += (long long)p.tiles_m * p.tiles_n;  // < 256 each
+    g.p[i] = p;
+  }
+  g.first_block[count] = (int)blocks;
+  hipLaunchKernelGGL((gemm_f64_mfma_group<false, false>), dim3((unsigned)blocks), dim3(256), 0, stream, g);
+  RST_HIP(hipGetLastError());
+  return RST_OK;
 }
 
 bool can_pair_gemm(const GemmDesc& input_grad, const GemmDesc& weight_grad) {

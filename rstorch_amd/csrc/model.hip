@@ -269,28 +269,51 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
   for (int i = 0; i < n; ++i)
     if (m->layers[i].kind == RST_LAYER_LINEAR) { first_linear = i; break; }
 
-  // the weight gradient that has been described but not launched yet
-  struct {
+  // a weight gradient that has been described but not launched yet
+  struct Pending {
     bool active = false;
     GemmDesc d{};
     int layer = -1;
     double flops = 0.0, bytes = 0.0;
     bool fused_bias = false;
     const double* grad = nullptr;  // gradient w.r.t. that layer's output
-  } pend;
-  auto flush_pending = [&]() -> int {
-    if (!pend.active) return RST_OK;
-    pend.active = false;
-    Layer& pl = m->layers[pend.layer];
-    RST_TRY(prof_begin(m, RST_KERNEL_GRAD_WEIGHT, pend.layer, pend.flops, pend.bytes));
-    RST_TRY(launch_gemm(e->stream, pend.d));
+  };
+  Pending pend;
+  // Small weight gradients (a launch each would cost more than their arithmetic) wait here for one
+  // shared grid at the end; their operands - the layer's cached input and the gradient buffer of
+  // the layer above - stay untouched until then.  Not while profiling: every layer keeps its record.
+  std::vector<Pending> held;
+  const bool may_hold = !m->profiling;
+  auto launch_pending = [&](const Pending& q) -> int {
+    Layer& pl = m->layers[q.layer];
+    RST_TRY(prof_begin(m, RST_KERNEL_GRAD_WEIGHT, q.layer, q.flops, q.bytes));
+    RST_TRY(launch_gemm(e->stream, q.d));
     RST_TRY(prof_end(m));
-    if (!pend.fused_bias) {
-      RST_TRY(prof_begin(m, RST_KERNEL_GRAD_BIAS, pend.layer, 0.0, 8.0 * ((double)batch * pl.out + pl.out)));
-      RST_TRY(launch_column_mean(e->stream, pend.grad, pl.gb, batch, pl.out, n_rows));
+    if (!q.fused_bias) {
+      RST_TRY(prof_begin(m, RST_KERNEL_GRAD_BIAS, q.layer, 0.0, 8.0 * ((double)batch * pl.out + pl.out)));
+      RST_TRY(launch_column_mean(e->stream, q.grad, pl.gb, batch, pl.out, n_rows));
       RST_TRY(prof_end(m));
       if (fused_lr) RST_TRY(launch_sgd_flat(e->stream, pl.b, pl.gb, pl.out, *fused_lr));
     }
+    return RST_OK;
+  };
+  auto flush_pending = [&]() -> int {
+    if (!pend.active) return RST_OK;
+    pend.active = false;
+    if (may_hold && pend.fused_bias && (int)held.size() < max_gemm_group() && can_group_gemm(pend.d)) {
+      held.push_back(pend);
+      return RST_OK;
+    }
+    return launch_pending(pend);
+  };
+  auto flush_held = [&]() -> int {
+    if (held.size() == 1) RST_TRY(launch_pending(held[0]));
+    if (held.size() > 1) {
+      std::vector<GemmDesc> descs;
+      for (const Pending& q : held) descs.push_back(q.d);
+      RST_TRY(launch_gemm_group(e->stream, descs.data(), (int)descs.size()));
+    }
+    held.clear();
     return RST_OK;
   };
 
@@ -371,6 +394,7 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
     cur = l.grad_in_buf;
   }
   RST_TRY(flush_pending());
+  RST_TRY(flush_held());
   if (input_grad) *input_grad = cur;
   // the caches are consumed (Option::take in linear.rs:61, relu.rs:26, cross_entropy.rs:46)
   m->forward_valid = false;

@@ -145,6 +145,40 @@ def test_profile_records_cover_every_launch(engine, oracle):
     dm.profile_enable(False)
 
 
+GROUP_CASES = [
+    ("readme_b32", README_MLP, 32),
+    # more small layers than one shared grid holds (eight), so two grids and a leftover
+    ("twelve_small_layers", [("linear", 20, 34), ("relu",)] + [("linear", 34, 34), ("relu",)] * 10 +
+     [("linear", 34, 6)], 16),
+    # a layer large enough for the 128x128 kernels between small ones, and an odd width that
+    # rules out 16-byte loads
+    ("mixed", [("linear", 64, 2048), ("relu",), ("linear", 2048, 2048), ("relu",), ("linear", 2048, 33),
+               ("relu",), ("linear", 33, 10)], 64),
+]
+
+
+@pytest.mark.parametrize("name,spec,batch", GROUP_CASES, ids=[c[0] for c in GROUP_CASES])
+@pytest.mark.parametrize("fused", [True, False])
+def test_shared_grid_of_small_weight_gradients_is_bit_identical(engine, oracle, name, spec, batch, fused):
+    """Small weight gradients share one grid at the end of backward; with profiling on every layer
+    launches on its own.  Losses, parameters and gradients must agree bit for bit."""
+    import rstorch_amd as rs
+    models = [pair(rs, oracle, spec, 77)[0] for _ in range(2)]
+    models[1].profile_enable(True)
+    for dm in models:
+        dm.fuse_sgd(fused)
+    for step in range(3):
+        x, y = batch_data(oracle, batch, models[0].in_width, models[0].out_width, 5, step, True)
+        losses = [dm.train_step(x, y, 0.05) for dm in models]
+        assert losses[0] == losses[1], "step %d" % step
+        for (p, g), (q, h) in zip(models[0].parameters(), models[1].parameters()):
+            assert np.array_equal(p.to_numpy(), q.to_numpy()), "step %d" % step
+            assert np.array_equal(g.to_numpy(), h.to_numpy()), "step %d" % step
+    kinds = [r["kernel"] for r in models[1].profile_read()]
+    assert kinds.count("grad_weight") == 3 * sum(1 for l in spec if l[0] == "linear")
+    models[1].profile_enable(False)
+
+
 def test_graph_replay_equals_eager_launches(engine, oracle):
     """The captured step must give bit-identical results on every replay, with other eager work
     and synchronisations between replays, and must re-record when an argument changes."""
