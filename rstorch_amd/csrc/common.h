@@ -78,9 +78,12 @@ int launch_gemm(hipStream_t stream, const GemmDesc& d);
 // under-fill the chip (fewer than 512 tiles).
 bool can_pair_gemm(const GemmDesc& input_grad, const GemmDesc& weight_grad);
 int launch_gemm_pair(hipStream_t stream, const GemmDesc& input_grad, const GemmDesc& weight_grad);
-// Several small weight gradients (both operands output-contiguous, each one unsplit launch of
-// fewer than 256 tiles of 32x32 on its own) in one grid; same results as launch_gemm on each.
+// Several small weight gradients (both operands output-contiguous, each a launch of 32x32 tiles
+// on its own, with or without K slices) in one grid, plus one shared reduction grid for the
+// sliced ones; same results as launch_gemm on each.  The descriptors share one workspace, of
+// which each sliced contraction takes gemm_group_workspace(d) doubles.
 bool can_group_gemm(const GemmDesc& d);
+size_t gemm_group_workspace(const GemmDesc& d);
 int max_gemm_group();
 int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count);
 

@@ -424,11 +424,14 @@ __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm
 
 // Up to kMaxGroup small products of the same operand layouts in one grid of 32x32 tiles (the
 // weight gradients of a small network: each is a handful of tiles, and a launch of its own costs
-// more than its arithmetic).  Workgroups [first_block[i], first_block[i+1]) belong to problem i.
+// more than its arithmetic).  Workgroups [first_block[i], first_block[i+1]) belong to problem i;
+// problems cut into K slices are finished by one shared reduction grid, whose workgroups
+// [first_reduce_block[i], first_reduce_block[i+1]) belong to problem i.
 constexpr int kMaxGroup = 8;
 struct GemmGroup {
   int count;
   int first_block[kMaxGroup + 1];
+  int first_reduce_block[kMaxGroup + 1];
   GemmParams p[kMaxGroup];
 };
 
@@ -800,10 +803,11 @@ __device__ __forceinline__ double ordered_slice_sum(const double* __restrict__ f
   return v;
 }
 
-// Adds the K slices of a split contraction in slice order and applies the epilogue.
-__global__ __launch_bounds__(256) void split_reduce_kernel(const GemmParams p) {
+// Adds the K slices of a split contraction in slice order and applies the epilogue: workgroup
+// `block` (256 threads) of problem p.
+__device__ __forceinline__ void split_reduce_body(const GemmParams& p, const size_t block) {
   const size_t mn = (size_t)p.M * p.N;
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t i = block * 256 + threadIdx.x;
   if (i < mn) {
     double v = ordered_slice_sum(p.ws + i, mn, p.split_k);
     const int row = (int)(i / p.N), col = (int)(i - (size_t)row * p.N);
@@ -827,6 +831,16 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const GemmParams p) {
     p.colsum[i] = g;
     if (p.sgd_bias) p.sgd_bias[i] = sgd_apply(p.sgd_bias[i], g, p.sgd_lr);
   }
+}
+
+__global__ __launch_bounds__(256) void split_reduce_kernel(const GemmParams p) {
+  split_reduce_body(p, blockIdx.x);
+}
+
+__global__ __launch_bounds__(256) void split_reduce_group_kernel(const GemmGroup g) {
+  int i = 0;
+  while (i + 1 < g.count && (int)blockIdx.x >= g.first_reduce_block[i + 1]) ++i;
+  split_reduce_body(g.p[i], (size_t)((int)blockIdx.x - g.first_reduce_block[i]));
 }
 
 int launch_split_reduce(hipStream_t stream, const GemmParams& p) {
@@ -901,11 +915,8 @@ long long small_tile_slices(const GemmParams& p, long long blocks, long long spl
   return s > 1 ? s : 1;
 }
 
-template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
-int launch_one(hipStream_t stream, GemmParams p, long long split_below = 256, long long want_blocks = 2048) {
-  p.tiles_m = (p.M + BM - 1) / BM;
-  p.tiles_n = (p.N + BN - 1) / BN;
-  long long blocks = (long long)p.tiles_m * p.tiles_n;
+// Fills in split_k, steps_per_split and ws_colsum of a small-tile launch of `blocks` output tiles.
+void plan_slices(GemmParams& p, long long blocks, long long split_below, long long want_blocks) {
   const int nk = (p.K + BK - 1) / BK;
   p.split_k = 1;
   p.steps_per_split = nk;
@@ -914,8 +925,16 @@ int launch_one(hipStream_t stream, GemmParams p, long long split_below = 256, lo
     p.steps_per_split = (int)((nk + s - 1) / s);
     p.split_k = (nk + p.steps_per_split - 1) / p.steps_per_split;
     p.ws_colsum = p.ws + (size_t)p.split_k * p.M * p.N;
-    blocks *= p.split_k;
   }
+}
+
+template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
+int launch_one(hipStream_t stream, GemmParams p, long long split_below = 256, long long want_blocks = 2048) {
+  p.tiles_m = (p.M + BM - 1) / BM;
+  p.tiles_n = (p.N + BN - 1) / BN;
+  long long blocks = (long long)p.tiles_m * p.tiles_n;
+  plan_slices(p, blocks, split_below, want_blocks);
+  blocks *= p.split_k;
   if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
   hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, WGM, WGN, A_KC, B_KC, VEC>), dim3((unsigned)blocks),
                      dim3(WGM * WGN * 64), 0, stream, p);
@@ -1026,35 +1045,64 @@ int launch_gemm(hipStream_t stream, const GemmDesc& d) {
 
 int max_gemm_group() { return kMaxGroup; }
 
+namespace {
+// the slices of a group member: what launch_gemm would choose for it alone
+void plan_group_member(GemmParams& p) {
+  p.tiles_m = (p.M + 31) / 32;
+  p.tiles_n = (p.N + 31) / 32;
+  plan_slices(p, (long long)p.tiles_m * p.tiles_n, 256, 2048);
+}
+}  // namespace
+
 bool can_group_gemm(const GemmDesc& d) {
   // the grouped kernel exists for the weight-gradient layouts with 16-byte loads
   if (d.M <= 0 || d.N <= 0 || d.a_kc || d.b_kc || !desc_vec_ok(d)) return false;
   const GemmParams p = make_params(d);
   int slices = 0;
-  if (choose_route(p, true, &slices) != Route::kTile32) return false;
-  const long long blocks = (long long)((p.M + 31) / 32) * ((p.N + 31) / 32);
-  return small_tile_slices(p, blocks, 256, 2048) == 1;
+  return choose_route(p, true, &slices) == Route::kTile32;
+}
+
+size_t gemm_group_workspace(const GemmDesc& d) {
+  GemmParams p = make_params(d);
+  plan_group_member(p);
+  return p.split_k > 1 ? (size_t)p.split_k * ((size_t)p.M * p.N + (size_t)p.M) : 0;
 }
 
 int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count) {
   if (count < 1 || count > kMaxGroup) return fail(RST_ERR_INVALID_ARGUMENT, "a group holds 1..%d contractions", kMaxGroup);
   GemmGroup g{};
   g.count = count;
-  long long blocks = 0;
+  long long blocks = 0, reduce_blocks = 0;
+  size_t ws_used = 0;
   for (int i = 0; i < count; ++i) {
     if (!can_group_gemm(d[i])) return fail(RST_ERR_INVALID_ARGUMENT, "contraction %d cannot join a group", i);
+    if (d[i].workspace != d[0].workspace || d[i].workspace_count != d[0].workspace_count)
+      return fail(RST_ERR_INVALID_ARGUMENT, "the contractions of a group share one workspace");
     GemmParams p = make_params(d[i]);
-    p.tiles_m = (p.M + 31) / 32;
-    p.tiles_n = (p.N + 31) / 32;
-    p.split_k = 1;
-    p.steps_per_split = (p.K + BK - 1) / BK;
+    plan_group_member(p);
     g.first_block[i] = (int)blocks;
-    blocks += (long long)p.tiles_m * p.tiles_n;  // < 256 each
+    g.first_reduce_block[i] = (int)reduce_blocks;
+    blocks += (long long)p.tiles_m * p.tiles_n * p.split_k;
+    if (p.split_k > 1) {
+      // every problem gets a region of its own in the shared workspace
+      const size_t need = (size_t)p.split_k * ((size_t)p.M * p.N + (size_t)p.M);
+      if (ws_used + need > p.ws_capacity) return fail(RST_ERR_INVALID_ARGUMENT, "group workspace exhausted");
+      p.ws += ws_used;
+      p.ws_colsum = p.ws + (size_t)p.split_k * p.M * p.N;
+      ws_used += need;
+      reduce_blocks += (long long)(((size_t)p.M * p.N + 255) / 256);
+    }
     g.p[i] = p;
   }
+  if (blocks > 0x7fffffffLL || reduce_blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
   g.first_block[count] = (int)blocks;
+  g.first_reduce_block[count] = (int)reduce_blocks;
   hipLaunchKernelGGL((gemm_f64_mfma_group<false, false>), dim3((unsigned)blocks), dim3(256), 0, stream, g);
   RST_HIP(hipGetLastError());
+  if (reduce_blocks > 0) {
+    hipLaunchKernelGGL(split_reduce_group_kernel, dim3((unsigned)reduce_blocks), dim3(256), 0, stream, g);
+    RST_HIP(hipGetLastError());
+  }
   return RST_OK;
 }
 

@@ -283,6 +283,7 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
   // shared grid at the end; their operands - the layer's cached input and the gradient buffer of
   // the layer above - stay untouched until then.  Not while profiling: every layer keeps its record.
   std::vector<Pending> held;
+  size_t held_ws = 0;  // doubles of the split-K workspace that the held ones will take
   const bool may_hold = !m->profiling;
   auto launch_pending = [&](const Pending& q) -> int {
     Layer& pl = m->layers[q.layer];
@@ -301,8 +302,12 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
     if (!pend.active) return RST_OK;
     pend.active = false;
     if (may_hold && pend.fused_bias && (int)held.size() < max_gemm_group() && can_group_gemm(pend.d)) {
-      held.push_back(pend);
-      return RST_OK;
+      const size_t need = gemm_group_workspace(pend.d);
+      if (held_ws + need <= e->gemm_ws_count) {
+        held_ws += need;
+        held.push_back(pend);
+        return RST_OK;
+      }
     }
     return launch_pending(pend);
   };
@@ -314,6 +319,7 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
       RST_TRY(launch_gemm_group(e->stream, descs.data(), (int)descs.size()));
     }
     held.clear();
+    held_ws = 0;
     return RST_OK;
   };
 

@@ -147,6 +147,9 @@ def test_profile_records_cover_every_launch(engine, oracle):
 
 GROUP_CASES = [
     ("readme_b32", README_MLP, 32),
+    # long batch: every weight gradient is cut into K slices, which share the reduction grid too
+    ("readme_b8192", README_MLP, 8192),
+    ("readme_b500", README_MLP, 500),
     # more small layers than one shared grid holds (eight), so two grids and a leftover
     ("twelve_small_layers", [("linear", 20, 34), ("relu",)] + [("linear", 34, 34), ("relu",)] * 10 +
      [("linear", 34, 6)], 16),
