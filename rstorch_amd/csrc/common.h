@@ -108,15 +108,13 @@ int launch_sgd_multi(hipStream_t s, const SgdTensor* device_table, size_t n_tens
 unsigned long long sgd_blocks_for(unsigned long long count);
 
 // softmax / cross entropy.  grad_out != NULL: cross entropy (row kernel + a one-workgroup
-// reduction) - row_loss is [rows] scratch, loss[0] receives -(sum)/rows, flags[1] the NaN flag of
-// this call (flags[0] is a working word left at zero).  grad_out == NULL: softmax only, prob_out
-// is written and flags[2] is set on a NaN input.
+// reduction; a batch of at most 64 rows that fits one workgroup is finished by the row kernel) -
+// row_loss is [rows] scratch, loss[0] receives -(sum)/rows, flags[1] the NaN flag of this call
+// (flags[0] is a working word left at zero).  grad_out == NULL: softmax only, prob_out is written
+// and flags[2] is set on a NaN input.
 int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* grad_out,
                       double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
                       size_t cols);
-int launch_softmax_rows(hipStream_t s, const double* z, const double* t, double* grad_out,
-                        double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
-                        size_t cols);
 int launch_softmax_columns(hipStream_t s, const double* z, double* out, int* flags, size_t rows,
                            size_t cols);
 int launch_softmax_jacobian(hipStream_t s, double* jac, size_t cols);

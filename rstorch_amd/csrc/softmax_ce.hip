@@ -51,13 +51,16 @@ __device__ __forceinline__ double loss_term(double truth, double p) {
   return truth * log(p);
 }
 
-// Register-resident rows: TPR threads per row, IPT vectors of VEC doubles per thread.
-template <int TPR, int IPT, int VEC, bool CE>
-__global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
+// Register-resident rows: TPR threads per row, IPT vectors of VEC doubles per thread, BLOCK / TPR
+// rows per workgroup.  SOLO: the whole batch (at most 64 rows) sits in one workgroup of 1024
+// threads, which then also finishes the loss the way loss_reduce_kernel would (same order of
+// additions, same bits), so that a small batch needs one launch instead of two.
+template <int TPR, int IPT, int VEC, bool CE, int BLOCK = 256, bool SOLO = false>
+__global__ __launch_bounds__(BLOCK) void softmax_rows_kernel(
     const double* __restrict__ z, const double* __restrict__ truth, double* __restrict__ grad,
     double* __restrict__ prob, double* __restrict__ row_loss, double* __restrict__ loss,
     int* __restrict__ flags, size_t rows, size_t cols) {
-  constexpr int BLOCK = TPR > 256 ? TPR : 256;
+  static_assert(BLOCK % TPR == 0 && (TPR <= 64 || BLOCK == TPR) && (!SOLO || (CE && BLOCK == 1024)), "unsupported shape");
   constexpr int RPB = BLOCK / TPR;
   __shared__ double red[3][TPR > 64 ? TPR / 64 : 1];
 
@@ -145,7 +148,29 @@ __global__ __launch_bounds__((TPR > 256 ? TPR : 256)) void softmax_rows_kernel(
       }
     }
   }
-  if (CE) {
+  if (CE && SOLO) {
+    __shared__ double solo_sum[64];
+    __shared__ int solo_nan;
+    lsum = group_reduce<TPR, SumOp>(lsum, red[2]);
+    if (threadIdx.x < 64) solo_sum[threadIdx.x] = 0.0;
+    if (threadIdx.x == 0) solo_nan = 0;
+    __syncthreads();
+    if (sub == 0 && row_ok) solo_sum[row] = lsum;
+    if (saw_nan) atomicOr(&solo_nan, 1);
+    __syncthreads();
+    if (threadIdx.x < 64) {
+      // loss_reduce_kernel on at most 64 rows: one value per lane of wavefront 0, the butterfly
+      // of group_reduce, then the (zero) sums of the other fifteen wavefronts
+      double v = solo_sum[threadIdx.x];
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) v = SumOp::apply(v, __shfl_xor(v, off));
+      if (threadIdx.x == 0) {
+        v = v + 0.0;
+        loss[0] = -v / (double)rows;
+        flags[1] = solo_nan;
+      }
+    }
+  } else if (CE) {
     lsum = group_reduce<TPR, SumOp>(lsum, red[2]);
     if (sub == 0 && row_ok) row_loss[row] = lsum;
     if (saw_nan) atomicOr(&flags[0], 1);
@@ -371,11 +396,22 @@ __global__ __launch_bounds__(256) void softmax_jacobian_kernel(double* __restric
 
 template <int TPR, int IPT, int VEC>
 int launch_rows(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
-                double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce) {
-  constexpr int BLOCK = TPR > 256 ? TPR : 256;
+                double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce,
+                bool* loss_done) {
+  constexpr int BLOCK = 256;
   constexpr int RPB = BLOCK / TPR;
   size_t blocks = (rows + RPB - 1) / RPB;
   if (blocks > 0x7fffffffull) return fail(RST_ERR_UNSUPPORTED, "too many rows for one launch");
+  // (rows that span several wavefronts reduce through per-row scratch that exists once per workgroup)
+  if constexpr (TPR <= 64) {
+    if (ce && rows * TPR <= 1024) {
+      hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, true, 1024, true>), dim3(1), dim3(1024), 0, s,
+                         z, t, grad, prob, row_loss, loss, flags, rows, cols);
+      *loss_done = true;
+      RST_HIP(hipGetLastError());
+      return RST_OK;
+    }
+  }
   if (ce)
     hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, true>), dim3((unsigned)blocks),
                        dim3(BLOCK), 0, s, z, t, grad, prob, row_loss, loss, flags, rows, cols);
@@ -402,17 +438,28 @@ int launch_wide(hipStream_t s, const double* z, const double* t, double* grad, d
 
 template <int VEC>
 int dispatch(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
-             double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce) {
+             double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce, bool* loss_done) {
   const size_t units = cols / VEC;  // vectors per row
-  if (units <= 16 * 2) return launch_rows<16, 2, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
-  if (units <= 64 * 4) return launch_rows<64, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
-  if (units <= 256 * 4) return launch_rows<256, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce);
+  if (units <= 16 * 2) return launch_rows<16, 2, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, loss_done);
+  if (units <= 64 * 4) return launch_rows<64, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, loss_done);
+  if (units <= 256 * 4) return launch_rows<256, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, loss_done);
   // measured on 32 Mi logits: 256 threads per row are ahead below about 12 Ki columns, 512 above
   if (cols < 12288) return launch_wide<256, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
   return launch_wide<512, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
 }
 
 inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; }
+
+// The row kernel of a softmax or cross entropy; *loss_done tells whether it finished the loss too.
+int launch_row_kernel(hipStream_t s, const double* z, const double* t, double* grad_out, double* prob_out,
+                      double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool* loss_done) {
+  const bool ce = grad_out != nullptr;
+  const bool vec = cols % 2 == 0 && aligned16(z) && (!ce || (aligned16(t) && aligned16(grad_out))) &&
+                   (!prob_out || aligned16(prob_out));
+  *loss_done = false;
+  if (vec) return dispatch<2>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, loss_done);
+  return dispatch<1>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, loss_done);
+}
 
 }  // namespace
 
@@ -421,8 +468,9 @@ int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* g
                       size_t cols) {
   if (rows == 0 || cols == 0) return RST_OK;
   const bool ce = grad_out != nullptr;
-  RST_TRY(launch_softmax_rows(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols));
-  if (ce) {
+  bool loss_done = false;
+  RST_TRY(launch_row_kernel(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, &loss_done));
+  if (ce && !loss_done) {
     hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(1024), 0, s, row_loss, loss, flags, rows);
     RST_HIP(hipGetLastError());
   }
@@ -444,16 +492,6 @@ int launch_softmax_jacobian(hipStream_t s, double* jac, size_t cols) {
                      0, s, jac, cols);
   RST_HIP(hipGetLastError());
   return RST_OK;
-}
-
-int launch_softmax_rows(hipStream_t s, const double* z, const double* t, double* grad_out,
-                        double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
-                        size_t cols) {
-  const bool ce = grad_out != nullptr;
-  const bool vec = cols % 2 == 0 && aligned16(z) && (!ce || (aligned16(t) && aligned16(grad_out))) &&
-                   (!prob_out || aligned16(prob_out));
-  if (vec) return dispatch<2>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce);
-  return dispatch<1>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce);
 }
 
 }  // namespace rst

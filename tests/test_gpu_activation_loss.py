@@ -179,6 +179,8 @@ def test_softmax_module_matches_oracle(engine, oracle, rows, cols, axis):
 
 # ---- CrossEntropyLoss ---------------------------------------------------------------------------
 @pytest.mark.parametrize("rows,cols", [(1, 2), (32, 10), (33, 11), (64, 100), (128, 1000),
+                                       # either side of what one workgroup finishes on its own
+                                       (64, 10), (65, 10), (16, 500), (17, 500), (4, 2000), (5, 2000),
                                        (9, 2048), (7, 2050), (5, 2051), (16, 4096), (6, 10000),
                                        (5, 12289), (4, 32768), (3, 33000), (2, 100001)])
 def test_cross_entropy_matches_oracle(engine, oracle, rows, cols):
