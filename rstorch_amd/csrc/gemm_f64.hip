@@ -305,7 +305,12 @@ __device__ __forceinline__ void colsum_finish(double partial, double* __restrict
 }
 
 // One output tile of the register-staged product: workgroup number `block` of problem p.
-template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
+// BURST = 0: the operand tiles of K step kt+1 travel while step kt is multiplied (two LDS stages).
+// BURST = D > 0, for grids of at most one workgroup per CU, where nothing else hides a load's
+// latency: the tiles of D K steps are requested together, land in D LDS stages and are multiplied
+// in K order, so a short contraction pays one trip to memory instead of one per step.  The
+// accumulation order, and with it every bit of the result, is the same either way.
+template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC, int BURST = 0>
 __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block) {
   constexpr int kThreads = WGM * WGN * 64;
   using GA = TileGeom<BM, A_KC, kThreads>;
@@ -314,8 +319,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block) 
   constexpr int TM = WM / 16, TN = WN / 16;  // MFMA tiles per wavefront
   static_assert(WM % 16 == 0 && WN % 16 == 0, "wave block must be whole MFMA tiles");
 
-  __shared__ __attribute__((aligned(16))) double lds_a[2][GA::size];
-  __shared__ __attribute__((aligned(16))) double lds_b[2][GB::size];
+  constexpr int kStages = BURST > 0 ? BURST : 2;
+  __shared__ __attribute__((aligned(16))) double lds_a[kStages][GA::size];
+  __shared__ __attribute__((aligned(16))) double lds_b[kStages][GB::size];
 
   // Workgroups are handed to the 8 XCDs round-robin; renumber them so that each XCD (and
   // its private L2) works on one compact patch of the tile grid, then walk the patch in
@@ -353,7 +359,6 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block) 
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
 
-  v2d ra[GA::loads], rb[GB::loads];
   const int nk_full = p.K / BK;                     // K steps that need no bounds handling
   const int nk_all = nk_full + (p.K % BK != 0 ? 1 : 0);
   const int kt0 = split * p.steps_per_split;        // this workgroup's K steps: [kt0, nk)
@@ -361,7 +366,7 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block) 
                                                                       : nk_all;
 
   // Loads the operand tiles of K step `kt` into registers; only the last step can be partial.
-  auto fetch = [&](int kt) {
+  auto fetch = [&](int kt, v2d* ra, v2d* rb) {
     if (kt < nk_full) {
       load_tile<BM, A_KC, VEC, false, kThreads>(ra, p.A, p.lda, m0, p.M, kt * BK, p.K, tid);
       load_tile<BN, B_KC, VEC, false, kThreads>(rb, p.B, p.ldb, n0, p.N, kt * BK, p.K, tid);
@@ -370,23 +375,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block) 
       load_tile<BN, B_KC, VEC, true, kThreads>(rb, p.B, p.ldb, n0, p.N, kt * BK, p.K, tid);
     }
   };
-
-  if (nk > kt0) {
-    fetch(kt0);
-    store_tile<BM, A_KC, kThreads>(lds_a[0], ra, tid);
-    store_tile<BN, B_KC, kThreads>(lds_b[0], rb, tid);
-  }
-  __syncthreads();
-
   const bool do_colsum = !A_KC && p.colsum != nullptr && tile_n == 0;
   double colsum_partial = 0.0;
-
-  for (int kt = kt0; kt < nk; ++kt) {
-    const int cur = (kt - kt0) & 1;
-    const bool more = kt + 1 < nk;
-    if (more) fetch(kt + 1);  // in flight while this step is multiplied
-    const double* __restrict__ sa = lds_a[cur];
-    const double* __restrict__ sb = lds_b[cur];
+  // One K step out of LDS stage (sa, sb).
+  auto multiply = [&](const double* __restrict__ sa, const double* __restrict__ sb) {
     if (!A_KC) {
       if (do_colsum) colsum_accumulate<BM, kThreads>(colsum_partial, sa, tid);
     }
@@ -403,11 +395,45 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block) 
         for (int j = 0; j < TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[i], fb[j], acc[i][j], 0, 0, 0);
     }
-    if (more) {
-      store_tile<BM, A_KC, kThreads>(lds_a[cur ^ 1], ra, tid);
-      store_tile<BN, B_KC, kThreads>(lds_b[cur ^ 1], rb, tid);
+  };
+
+  if (BURST > 0) {
+    v2d ra[kStages][GA::loads], rb[kStages][GB::loads];
+    for (int k0 = kt0; k0 < nk; k0 += kStages) {
+#pragma unroll
+      for (int d = 0; d < kStages; ++d)
+        if (k0 + d < nk) fetch(k0 + d, ra[d], rb[d]);
+#pragma unroll
+      for (int d = 0; d < kStages; ++d)
+        if (k0 + d < nk) {
+          store_tile<BM, A_KC, kThreads>(lds_a[d], ra[d], tid);
+          store_tile<BN, B_KC, kThreads>(lds_b[d], rb[d], tid);
+        }
+      __syncthreads();
+#pragma unroll
+      for (int d = 0; d < kStages; ++d)
+        if (k0 + d < nk) multiply(lds_a[d], lds_b[d]);
+      __syncthreads();
+    }
+  } else {
+    v2d ra[GA::loads], rb[GB::loads];
+    if (nk > kt0) {
+      fetch(kt0, ra, rb);
+      store_tile<BM, A_KC, kThreads>(lds_a[0], ra, tid);
+      store_tile<BN, B_KC, kThreads>(lds_b[0], rb, tid);
     }
     __syncthreads();
+    for (int kt = kt0; kt < nk; ++kt) {
+      const int cur = (kt - kt0) & 1;
+      const bool more = kt + 1 < nk;
+      if (more) fetch(kt + 1, ra, rb);  // in flight while this step is multiplied
+      multiply(lds_a[cur], lds_b[cur]);
+      if (more) {
+        store_tile<BM, A_KC, kThreads>(lds_a[cur ^ 1], ra, tid);
+        store_tile<BN, B_KC, kThreads>(lds_b[cur ^ 1], rb, tid);
+      }
+      __syncthreads();
+    }
   }
   if (!A_KC) {
     if (do_colsum) colsum_finish<BM, kThreads>(colsum_partial, lds_b[0], tid, m0, split, p);
@@ -416,10 +442,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block) 
   write_block<TM, TN>(p, &acc[0][0], m0 + wm * WM, n0 + wn * WN, lr, lk, split);
 }
 
-template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC>
+template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC, int BURST = 0>
 __global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm_f64_mfma(
     const GemmParams p) {
-  gemm_tile<BM, BN, WGM, WGN, A_KC, B_KC, VEC>(p, (int)blockIdx.x);
+  gemm_tile<BM, BN, WGM, WGN, A_KC, B_KC, VEC, BURST>(p, (int)blockIdx.x);
 }
 
 // Up to kMaxGroup small products of the same operand layouts in one grid of 32x32 tiles (the
@@ -435,11 +461,11 @@ struct GemmGroup {
   GemmParams p[kMaxGroup];
 };
 
-template <bool A_KC, bool B_KC>
+template <bool A_KC, bool B_KC, int BURST>
 __global__ __launch_bounds__(256, 2) void gemm_f64_mfma_group(const GemmGroup g) {
   int i = 0;
   while (i + 1 < g.count && (int)blockIdx.x >= g.first_block[i + 1]) ++i;
-  gemm_tile<32, 32, 2, 2, A_KC, B_KC, true>(g.p[i], (int)blockIdx.x - g.first_block[i]);
+  gemm_tile<32, 32, 2, 2, A_KC, B_KC, true, BURST>(g.p[i], (int)blockIdx.x - g.first_block[i]);
 }
 
 // ---- 128x128 tiles fed by direct global -> LDS loads ------------------------------------------
@@ -915,6 +941,10 @@ long long small_tile_slices(const GemmParams& p, long long blocks, long long spl
   return s > 1 ? s : 1;
 }
 
+// 32x32 tiles on at most one workgroup per CU: K steps are fetched eight at a time (gemm_tile)
+constexpr int kBurst = 8;
+constexpr long long kBurstMaxBlocks = 256;
+
 // Fills in split_k, steps_per_split and ws_colsum of a small-tile launch of `blocks` output tiles.
 void plan_slices(GemmParams& p, long long blocks, long long split_below, long long want_blocks) {
   const int nk = (p.K + BK - 1) / BK;
@@ -936,8 +966,12 @@ int launch_one(hipStream_t stream, GemmParams p, long long split_below = 256, lo
   plan_slices(p, blocks, split_below, want_blocks);
   blocks *= p.split_k;
   if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
-  hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, WGM, WGN, A_KC, B_KC, VEC>), dim3((unsigned)blocks),
-                     dim3(WGM * WGN * 64), 0, stream, p);
+  if (BM == 32 && BN == 32 && blocks <= kBurstMaxBlocks)
+    hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, WGM, WGN, A_KC, B_KC, VEC, (BM == 32 ? kBurst : 0)>),
+                       dim3((unsigned)blocks), dim3(WGM * WGN * 64), 0, stream, p);
+  else
+    hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, WGM, WGN, A_KC, B_KC, VEC>), dim3((unsigned)blocks),
+                       dim3(WGM * WGN * 64), 0, stream, p);
   RST_HIP(hipGetLastError());
   if (p.split_k > 1) RST_TRY(launch_split_reduce(stream, p));
   return RST_OK;
@@ -1097,7 +1131,10 @@ int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count) {
   if (blocks > 0x7fffffffLL || reduce_blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
   g.first_block[count] = (int)blocks;
   g.first_reduce_block[count] = (int)reduce_blocks;
-  hipLaunchKernelGGL((gemm_f64_mfma_group<false, false>), dim3((unsigned)blocks), dim3(256), 0, stream, g);
+  if (blocks <= kBurstMaxBlocks)
+    hipLaunchKernelGGL((gemm_f64_mfma_group<false, false, kBurst>), dim3((unsigned)blocks), dim3(256), 0, stream, g);
+  else
+    hipLaunchKernelGGL((gemm_f64_mfma_group<false, false, 0>), dim3((unsigned)blocks), dim3(256), 0, stream, g);
   RST_HIP(hipGetLastError());
   if (reduce_blocks > 0) {
     hipLaunchKernelGGL(split_reduce_group_kernel, dim3((unsigned)reduce_blocks), dim3(256), 0, stream, g);
