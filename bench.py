@@ -34,9 +34,9 @@ PEAK_HBM_GBPS = 8000.0
 # gradient), the reduction of the two partial results (134.3 MB); the weight gradient carries the SGD
 # update of its layer.
 C4_TRAFFIC_BYTES_PER_LAUNCH = {
-    "linear_forward": (8 * 436.4e6 + 3855.9e6) / 9,
-    "grad_weight": (8 * 858.6e6 + 6976.9e6) / 9,
-    "grad_input": (7 * 470.0e6 + 3354.0e6 + 134.3e6) / 8,
+    "linear_forward": (8 * 436.4e6 + 3847.5e6) / 9,
+    "grad_weight": (8 * 859.2e6 + 6972.6e6) / 9,
+    "grad_input": (7 * 470.0e6 + 3357.2e6 + 134.3e6) / 8,
 }
 
 C4_SPEC = [("linear", 4096, 4096), ("relu",)] * 8 + [("linear", 4096, 32768)]

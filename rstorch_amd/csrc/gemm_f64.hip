@@ -814,17 +814,32 @@ __global__ __launch_bounds__(512, 4) void gemm_f64_mfma_dma_pair(const GemmParam
   }
 }
 
-// Sum of `count` values `stride` doubles apart, added in order; 32 loads are in flight at a time
-// (the slices were written by other XCDs, so every load is a trip to memory).
+// Sum of `count` values `stride` doubles apart, added in order; up to 32 loads are in flight at a
+// time (the slices were written by other XCDs, so every load is a trip to memory).
 __device__ __forceinline__ double ordered_slice_sum(const double* __restrict__ first, size_t stride, int count) {
   double v = 0.0;
-  for (int s0 = 0; s0 < count; s0 += 32) {
+  int s = 0;
+  for (; s + 32 <= count; s += 32) {
     double t[32];
 #pragma unroll
-    for (int j = 0; j < 32; ++j) t[j] = s0 + j < count ? first[(size_t)(s0 + j) * stride] : 0.0;
+    for (int j = 0; j < 32; ++j) t[j] = first[(size_t)(s + j) * stride];
 #pragma unroll
-    for (int j = 0; j < 32; ++j)
-      if (s0 + j < count) v += t[j];
+    for (int j = 0; j < 32; ++j) v += t[j];
+  }
+  for (; s + 8 <= count; s += 8) {
+    double t[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t[j] = first[(size_t)(s + j) * stride];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v += t[j];
+  }
+  if (s < count) {
+    double t[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t[j] = s + j < count ? first[(size_t)(s + j) * stride] : 0.0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      if (s + j < count) v += t[j];
   }
   return v;
 }
@@ -943,7 +958,6 @@ long long small_tile_slices(const GemmParams& p, long long blocks, long long spl
 
 // 32x32 tiles on at most one workgroup per CU: K steps are fetched eight at a time (gemm_tile)
 constexpr int kBurst = 8;
-constexpr long long kBurstMaxBlocks = 256;
 
 // Fills in split_k, steps_per_split and ws_colsum of a small-tile launch of `blocks` output tiles.
 void plan_slices(GemmParams& p, long long blocks, long long split_below, long long want_blocks) {
@@ -966,7 +980,7 @@ int launch_one(hipStream_t stream, GemmParams p, long long split_below = 256, lo
   plan_slices(p, blocks, split_below, want_blocks);
   blocks *= p.split_k;
   if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
-  if (BM == 32 && BN == 32 && blocks <= kBurstMaxBlocks)
+  if (BM == 32 && BN == 32 && blocks <= compute_units())
     hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, WGM, WGN, A_KC, B_KC, VEC, (BM == 32 ? kBurst : 0)>),
                        dim3((unsigned)blocks), dim3(WGM * WGN * 64), 0, stream, p);
   else
@@ -1131,7 +1145,7 @@ int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count) {
   if (blocks > 0x7fffffffLL || reduce_blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
   g.first_block[count] = (int)blocks;
   g.first_reduce_block[count] = (int)reduce_blocks;
-  if (blocks <= kBurstMaxBlocks)
+  if (blocks <= compute_units())
     hipLaunchKernelGGL((gemm_f64_mfma_group<false, false, kBurst>), dim3((unsigned)blocks), dim3(256), 0, stream, g);
   else
     hipLaunchKernelGGL((gemm_f64_mfma_group<false, false, 0>), dim3((unsigned)blocks), dim3(256), 0, stream, g);
