@@ -460,6 +460,7 @@ struct GemmGroup {
   int first_reduce_block[kMaxGroup + 1];
   GemmParams p[kMaxGroup];
 };
+static_assert(sizeof(GemmGroup) <= 4096, "a group travels as one kernel argument");
 
 template <bool A_KC, bool B_KC, int BURST>
 __global__ __launch_bounds__(256, 2) void gemm_f64_mfma_group(const GemmGroup g) {
