@@ -1012,11 +1012,20 @@ Route choose_route(const GemmParams& p, bool vec, int* dma_slices) {
   // against 62 %), as long as the slices still fill the chip.
   if (dma_ok && p.ws != nullptr) {
     const int nk = p.K / BK;
+    auto fits = [&](int s) { return p.ws_capacity >= (size_t)s * ((size_t)p.M * p.N + (size_t)p.M); };
     int s = (int)((512 + t128 - 1) / t128);
     if (s > 8) s = 8;
-    while (s > 1 && nk / s < 32) --s;
-    while (s > 1 && p.ws_capacity < (size_t)s * ((size_t)p.M * p.N + (size_t)p.M)) --s;
-    if (s > 1 && t128 * s >= 256) {
+    while (s > 1 && (nk / s < 32 || !fits(s))) --s;
+    if (!(s > 1 && t128 * s >= 256)) {
+      // a shorter contraction: one round of workgroups (at most one per CU, at least three CUs in
+      // four busy) on slices of 12 K steps or more still beats the register-staged small tiles
+      // (8192 x 100 x 784 on 64 tiles: 39 us on four slices against 47 us); a round and a bit
+      // does not (64 tiles on five slices: 70 us against 60 us)
+      s = (int)(256 / t128);
+      if (s > 8) s = 8;
+      if (!(s > 1 && t128 * s >= 192 && nk / s >= 12 && fits(s))) s = 1;
+    }
+    if (s > 1) {
       *dma_slices = s;
       return Route::kDmaSliced;
     }
