@@ -959,6 +959,9 @@ long long small_tile_slices(const GemmParams& p, long long blocks, long long spl
 
 // 32x32 tiles on at most one workgroup per CU: K steps are fetched eight at a time (gemm_tile)
 constexpr int kBurst = 8;
+// 32x32 tiles are cut into K slices while they give fewer than two workgroups per CU (a 1024 x 256
+// output at K = 4096, 256 tiles: 110 us unsplit, one chain of 256 K steps per workgroup)
+constexpr long long kSmallTileSplitBelow = 512;
 
 // Fills in split_k, steps_per_split and ws_colsum of a small-tile launch of `blocks` output tiles.
 void plan_slices(GemmParams& p, long long blocks, long long split_below, long long want_blocks) {
@@ -1041,7 +1044,7 @@ int launch_layout(hipStream_t stream, const GemmParams& p) {
     case Route::kDmaSliced: return launch_dma<A_KC, B_KC>(stream, p, slices);
     case Route::kTile128: return launch_one<128, 128, 2, 4, A_KC, B_KC, VEC>(stream, p);
     case Route::kTile64: return launch_one<64, 64, 2, 2, A_KC, B_KC, VEC>(stream, p);
-    default: return launch_one<32, 32, 2, 2, A_KC, B_KC, VEC>(stream, p);
+    default: return launch_one<32, 32, 2, 2, A_KC, B_KC, VEC>(stream, p, kSmallTileSplitBelow);
   }
 }
 
@@ -1108,7 +1111,7 @@ namespace {
 void plan_group_member(GemmParams& p) {
   p.tiles_m = (p.M + 31) / 32;
   p.tiles_n = (p.N + 31) / 32;
-  plan_slices(p, (long long)p.tiles_m * p.tiles_n, 256, 2048);
+  plan_slices(p, (long long)p.tiles_m * p.tiles_n, kSmallTileSplitBelow, 2048);
 }
 }  // namespace
 
