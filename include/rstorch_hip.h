@@ -243,7 +243,9 @@ int rst_model_graph_enable(rst_model* model, int enabled);
 /* Per-launch timing of the model's kernels: when enabled an event is recorded on the engine's
  * stream after every launch (and one before the first launch of a call); a launch's duration runs
  * from the previous event to its own, so it includes the few microseconds between the previous
- * kernel's end and its own start.  Records
+ * kernel's end and its own start.  While enabled, every layer's weight gradient is a launch of
+ * its own (small ones otherwise share one grid at the end of backward; the results are the same
+ * bit for bit).  Records
  * accumulate over calls (up to 65536) until rst_model_profile_read, which waits for the stream,
  * copies up to `capacity` of them (host_records == NULL: only counts) and clears the list. */
 typedef struct rst_kernel_record {
