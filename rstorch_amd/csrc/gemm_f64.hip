@@ -377,11 +377,15 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block) 
   };
   const bool do_colsum = !A_KC && p.colsum != nullptr && tile_n == 0;
   double colsum_partial = 0.0;
+  // a wavefront whose whole block lies beyond the edge of the output (M = 100 in 32-row tiles:
+  // rows 112..127) copies its share of the tiles but multiplies nothing
+  const bool wave_live = m0 + wm * WM < p.M && n0 + wn * WN < p.N;
   // One K step out of LDS stage (sa, sb).
   auto multiply = [&](const double* __restrict__ sa, const double* __restrict__ sb) {
     if (!A_KC) {
       if (do_colsum) colsum_accumulate<BM, kThreads>(colsum_partial, sa, tid);
     }
+    if (!wave_live) return;
 #pragma unroll
     for (int ks = 0; ks < BK / 4; ++ks) {
       double fa[TM], fb[TN];
