@@ -298,19 +298,6 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
     }
     return RST_OK;
   };
-  auto flush_pending = [&]() -> int {
-    if (!pend.active) return RST_OK;
-    pend.active = false;
-    if (may_hold && pend.fused_bias && (int)held.size() < max_gemm_group() && can_group_gemm(pend.d)) {
-      const size_t need = gemm_group_workspace(pend.d);
-      if (held_ws + need <= e->gemm_ws_count) {
-        held_ws += need;
-        held.push_back(pend);
-        return RST_OK;
-      }
-    }
-    return launch_pending(pend);
-  };
   auto flush_held = [&]() -> int {
     if (held.size() == 1) RST_TRY(launch_pending(held[0]));
     if (held.size() > 1) {
@@ -323,6 +310,21 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
     return RST_OK;
   };
 
+  auto flush_pending = [&]() -> int {
+    if (!pend.active) return RST_OK;
+    pend.active = false;
+    if (may_hold && pend.fused_bias && can_group_gemm(pend.d)) {
+      const size_t need = gemm_group_workspace(pend.d);
+      // a full grid (or a full workspace) goes out, and the next one starts
+      if ((int)held.size() == max_gemm_group() || held_ws + need > e->gemm_ws_count) RST_TRY(flush_held());
+      if (need <= e->gemm_ws_count) {
+        held_ws += need;
+        held.push_back(pend);
+        return RST_OK;
+      }
+    }
+    return launch_pending(pend);
+  };
   for (int i = n - 1; i >= 0; --i) {
     Layer& l = m->layers[i];
     if (l.kind == RST_LAYER_IDENTITY) continue;  // identity.rs:22-24

@@ -150,7 +150,7 @@ GROUP_CASES = [
     # long batch: every weight gradient is cut into K slices, which share the reduction grid too
     ("readme_b8192", README_MLP, 8192),
     ("readme_b500", README_MLP, 500),
-    # more small layers than one shared grid holds (eight): the others launch on their own
+    # more small layers than one shared grid holds (eight): two grids
     ("twelve_small_layers", [("linear", 20, 34), ("relu",)] + [("linear", 34, 34), ("relu",)] * 10 +
      [("linear", 34, 6)], 16),
     # a layer large enough for the 128x128 kernels between small ones, and an odd width that
