@@ -112,15 +112,25 @@ unsigned long long sgd_blocks_for(unsigned long long count);
 // row_loss is [rows] scratch, loss[0] receives -(sum)/rows, flags[1] the NaN flag of this call
 // (flags[0] is a working word left at zero).  grad_out == NULL: softmax only, prob_out is written
 // and flags[2] is set on a NaN input.
+// LossMirror: device-visible addresses of pinned host words that receive the loss and flags[1]
+// as well (written by the thread that finishes the loss), so that the host can read them after a
+// stream synchronisation without a copy in between.  Null members: no mirror.
+struct LossMirror {
+  double* loss = nullptr;
+  int* flags = nullptr;
+};
 int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* grad_out,
                       double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
-                      size_t cols);
+                      size_t cols, LossMirror mirror = LossMirror());
 int launch_softmax_columns(hipStream_t s, const double* z, double* out, int* flags, size_t rows,
                            size_t cols);
 int launch_softmax_jacobian(hipStream_t s, double* jac, size_t cols);
 // hits[0] = number of rows whose first arg-max agrees
+// hits_mirror: device-visible address of a pinned host word; *mirrored tells whether the count
+// was also written there (small inputs, counted by one workgroup without atomics)
 int launch_accuracy(hipStream_t s, const double* pred, const double* truth, size_t rows,
-                    size_t cols, unsigned long long* hits);
+                    size_t cols, unsigned long long* hits, unsigned long long* hits_mirror = nullptr,
+                    bool* mirrored = nullptr);
 
 int launch_fill_uniform(hipStream_t s, double* dst, size_t n, uint64_t seed, uint64_t stream,
                         double lo, double hi);
@@ -143,6 +153,10 @@ struct rst_engine {
   double* h_loss = nullptr;  // pinned
   int* h_flags = nullptr;    // pinned
   unsigned long long* h_hits = nullptr;  // pinned
+  // the same three words as the device addresses them (kernels store scalar results there)
+  double* hd_loss = nullptr;
+  int* hd_flags = nullptr;
+  unsigned long long* hd_hits = nullptr;
   bool loss_valid = false;
   // split-K scratch of the contraction kernels (fixed size, allocated with the engine)
   double* d_gemm_ws = nullptr;

@@ -103,6 +103,14 @@ int rst_engine_create(int device, rst_engine** out) {
   if (err == hipSuccess) err = hipHostMalloc(&e->h_flags, 4 * sizeof(int), hipHostMallocDefault);
   if (err == hipSuccess)
     err = hipHostMalloc(&e->h_hits, sizeof(unsigned long long), hipHostMallocDefault);
+  if (err == hipSuccess) err = hipHostGetDevicePointer((void**)&e->hd_loss, e->h_loss, 0);
+  if (err == hipSuccess) err = hipHostGetDevicePointer((void**)&e->hd_flags, e->h_flags, 0);
+  if (err == hipSuccess) err = hipHostGetDevicePointer((void**)&e->hd_hits, e->h_hits, 0);
+  if (err == hipSuccess) {
+    *e->h_loss = 0.0;
+    e->h_flags[0] = e->h_flags[1] = e->h_flags[2] = e->h_flags[3] = 0;
+    *e->h_hits = 0;
+  }
   if (err == hipSuccess) err = hipMemsetAsync(e->d_flags, 0, 4 * sizeof(int), e->stream);
   if (err == hipSuccess) err = hipStreamSynchronize(e->stream);
   if (err != hipSuccess) {

@@ -23,8 +23,11 @@ int engine_cross_entropy(rst_engine* e, const double* pred, const double* truth,
                          double* prob_out, size_t rows, size_t cols, double* host_loss) {
   RST_TRY(engine_reserve_row_loss(e, rows));
   if (rows == 0 || cols == 0) return fail(RST_ERR_SHAPE, "cross entropy of an empty batch");
+  LossMirror mirror;
+  mirror.loss = e->hd_loss;
+  mirror.flags = e->hd_flags;
   RST_TRY(launch_softmax_ce(e->stream, pred, truth, grad_out, prob_out, e->d_row_loss, e->d_loss,
-                            e->d_flags, rows, cols));
+                            e->d_flags, rows, cols, mirror));
   e->loss_valid = true;
   if (host_loss) return rst_loss_value(e, host_loss);
   return RST_OK;
@@ -190,11 +193,10 @@ int rst_loss_value(rst_engine* e, double* host_loss) {
   RST_TRY(engine_activate(e));
   if (!host_loss) return fail(RST_ERR_INVALID_ARGUMENT, "host_loss is null");
   if (!e->loss_valid) return fail(RST_ERR_STATE, "no loss has been computed on this engine");
-  RST_HIP(hipMemcpyAsync(e->h_loss, e->d_loss, sizeof(double), hipMemcpyDeviceToHost, e->stream));
-  RST_HIP(hipMemcpyAsync(e->h_flags, e->d_flags, 4 * sizeof(int), hipMemcpyDeviceToHost, e->stream));
+  // the kernel that finished the loss stored it, and the NaN flag, in the pinned words as well
   RST_HIP(hipStreamSynchronize(e->stream));
-  *host_loss = *e->h_loss;
-  if (e->h_flags[1] & 1)
+  *host_loss = *static_cast<volatile double*>(e->h_loss);
+  if (static_cast<volatile int*>(e->h_flags)[1] & 1)
     return fail(RST_ERR_NAN, "cross entropy: NaN logits (the reference panics in softmax.rs:38)");
   return RST_OK;
 }
@@ -254,11 +256,13 @@ int rst_accuracy(rst_engine* e, const double* pred, const double* truth, size_t 
   RST_TRY(engine_activate(e));
   if (!pred || !truth || !host_accuracy)
     return fail(RST_ERR_INVALID_ARGUMENT, "accuracy: null operand");
-  RST_TRY(launch_accuracy(e->stream, pred, truth, rows, cols, e->d_hits));
-  RST_HIP(hipMemcpyAsync(e->h_hits, e->d_hits, sizeof(unsigned long long), hipMemcpyDeviceToHost,
-                         e->stream));
+  bool mirrored = false;
+  RST_TRY(launch_accuracy(e->stream, pred, truth, rows, cols, e->d_hits, e->hd_hits, &mirrored));
+  if (!mirrored)
+    RST_HIP(hipMemcpyAsync(e->h_hits, e->d_hits, sizeof(unsigned long long), hipMemcpyDeviceToHost,
+                           e->stream));
   RST_HIP(hipStreamSynchronize(e->stream));
-  *host_accuracy = (double)(*e->h_hits) / (double)rows;
+  *host_accuracy = (double)(*static_cast<volatile unsigned long long*>(e->h_hits)) / (double)rows;
   return RST_OK;
 }
 

@@ -59,7 +59,7 @@ template <int TPR, int IPT, int VEC, bool CE, int BLOCK = 256, bool SOLO = false
 __global__ __launch_bounds__(BLOCK) void softmax_rows_kernel(
     const double* __restrict__ z, const double* __restrict__ truth, double* __restrict__ grad,
     double* __restrict__ prob, double* __restrict__ row_loss, double* __restrict__ loss,
-    int* __restrict__ flags, size_t rows, size_t cols) {
+    int* __restrict__ flags, size_t rows, size_t cols, LossMirror mirror) {
   static_assert(BLOCK % TPR == 0 && (TPR <= 64 || BLOCK == TPR) && (!SOLO || (CE && BLOCK == 1024)), "unsupported shape");
   constexpr int RPB = BLOCK / TPR;
   __shared__ double red[3][TPR > 64 ? TPR / 64 : 1];
@@ -166,8 +166,13 @@ __global__ __launch_bounds__(BLOCK) void softmax_rows_kernel(
       for (int off = 32; off > 0; off >>= 1) v = SumOp::apply(v, __shfl_xor(v, off));
       if (threadIdx.x == 0) {
         v = v + 0.0;
-        loss[0] = -v / (double)rows;
+        const double l = -v / (double)rows;
+        loss[0] = l;
         flags[1] = solo_nan;
+        if (mirror.loss) {
+          mirror.loss[0] = l;
+          mirror.flags[1] = solo_nan;
+        }
       }
     }
   } else if (CE) {
@@ -347,15 +352,22 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) v
 // flags[0], so no reset launch is needed.
 __global__ __launch_bounds__(1024) void loss_reduce_kernel(const double* __restrict__ row_loss,
                                                           double* __restrict__ loss,
-                                                          int* __restrict__ flags, size_t rows) {
+                                                          int* __restrict__ flags, size_t rows,
+                                                          LossMirror mirror) {
   __shared__ double red[1024 / 64];
   double s = 0.0;
   for (size_t r = threadIdx.x; r < rows; r += 1024) s += row_loss[r];
   s = group_reduce<1024, SumOp>(s, red);
   if (threadIdx.x == 0) {
-    loss[0] = -s / (double)rows;
-    flags[1] = flags[0];
+    const double l = -s / (double)rows;
+    const int nan_seen = flags[0];
+    loss[0] = l;
+    flags[1] = nan_seen;
     flags[0] = 0;
+    if (mirror.loss) {
+      mirror.loss[0] = l;
+      mirror.flags[1] = nan_seen;
+    }
   }
 }
 
@@ -397,7 +409,7 @@ __global__ __launch_bounds__(256) void softmax_jacobian_kernel(double* __restric
 template <int TPR, int IPT, int VEC>
 int launch_rows(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
                 double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce,
-                bool* loss_done) {
+                LossMirror mirror, bool* loss_done) {
   constexpr int BLOCK = 256;
   constexpr int RPB = BLOCK / TPR;
   size_t blocks = (rows + RPB - 1) / RPB;
@@ -406,7 +418,7 @@ int launch_rows(hipStream_t s, const double* z, const double* t, double* grad, d
   if constexpr (TPR <= 64) {
     if (ce && rows * TPR <= 1024) {
       hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, true, 1024, true>), dim3(1), dim3(1024), 0, s,
-                         z, t, grad, prob, row_loss, loss, flags, rows, cols);
+                         z, t, grad, prob, row_loss, loss, flags, rows, cols, mirror);
       *loss_done = true;
       RST_HIP(hipGetLastError());
       return RST_OK;
@@ -414,10 +426,10 @@ int launch_rows(hipStream_t s, const double* z, const double* t, double* grad, d
   }
   if (ce)
     hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, true>), dim3((unsigned)blocks),
-                       dim3(BLOCK), 0, s, z, t, grad, prob, row_loss, loss, flags, rows, cols);
+                       dim3(BLOCK), 0, s, z, t, grad, prob, row_loss, loss, flags, rows, cols, mirror);
   else
     hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, false>), dim3((unsigned)blocks),
-                       dim3(BLOCK), 0, s, z, t, grad, prob, row_loss, loss, flags, rows, cols);
+                       dim3(BLOCK), 0, s, z, t, grad, prob, row_loss, loss, flags, rows, cols, mirror);
   RST_HIP(hipGetLastError());
   return RST_OK;
 }
@@ -438,11 +450,12 @@ int launch_wide(hipStream_t s, const double* z, const double* t, double* grad, d
 
 template <int VEC>
 int dispatch(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
-             double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce, bool* loss_done) {
+             double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce,
+             LossMirror mirror, bool* loss_done) {
   const size_t units = cols / VEC;  // vectors per row
-  if (units <= 16 * 2) return launch_rows<16, 2, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, loss_done);
-  if (units <= 64 * 4) return launch_rows<64, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, loss_done);
-  if (units <= 256 * 4) return launch_rows<256, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, loss_done);
+  if (units <= 16 * 2) return launch_rows<16, 2, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done);
+  if (units <= 64 * 4) return launch_rows<64, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done);
+  if (units <= 256 * 4) return launch_rows<256, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done);
   // measured on 32 Mi logits: 256 threads per row are ahead below about 12 Ki columns, 512 above
   if (cols < 12288) return launch_wide<256, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
   return launch_wide<512, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
@@ -452,26 +465,27 @@ inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 1
 
 // The row kernel of a softmax or cross entropy; *loss_done tells whether it finished the loss too.
 int launch_row_kernel(hipStream_t s, const double* z, const double* t, double* grad_out, double* prob_out,
-                      double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool* loss_done) {
+                      double* row_loss, double* loss, int* flags, size_t rows, size_t cols,
+                      LossMirror mirror, bool* loss_done) {
   const bool ce = grad_out != nullptr;
   const bool vec = cols % 2 == 0 && aligned16(z) && (!ce || (aligned16(t) && aligned16(grad_out))) &&
                    (!prob_out || aligned16(prob_out));
   *loss_done = false;
-  if (vec) return dispatch<2>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, loss_done);
-  return dispatch<1>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, loss_done);
+  if (vec) return dispatch<2>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, mirror, loss_done);
+  return dispatch<1>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, mirror, loss_done);
 }
 
 }  // namespace
 
 int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* grad_out,
                       double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
-                      size_t cols) {
+                      size_t cols, LossMirror mirror) {
   if (rows == 0 || cols == 0) return RST_OK;
   const bool ce = grad_out != nullptr;
   bool loss_done = false;
-  RST_TRY(launch_row_kernel(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, &loss_done));
+  RST_TRY(launch_row_kernel(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, mirror, &loss_done));
   if (ce && !loss_done) {
-    hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(1024), 0, s, row_loss, loss, flags, rows);
+    hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(1024), 0, s, row_loss, loss, flags, rows, mirror);
     RST_HIP(hipGetLastError());
   }
   return RST_OK;

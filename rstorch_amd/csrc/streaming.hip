@@ -281,8 +281,43 @@ int launch_sgd_multi(hipStream_t s, const SgdTensor* device_table, size_t n_tens
   return RST_OK;
 }
 
+// Small inputs: one workgroup of 16 wavefronts counts every row (wavefront w takes rows w, w+16,
+// ...), adds the sixteen counts in order and stores the total in the device word and in its host
+// mirror - one launch, no atomics, nothing to copy back.
+__global__ __launch_bounds__(1024) void accuracy_small_kernel(const double* __restrict__ pred,
+                                                             const double* __restrict__ truth,
+                                                             size_t rows, size_t cols,
+                                                             unsigned long long* hits,
+                                                             unsigned long long* hits_mirror) {
+  __shared__ unsigned counts[16];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  unsigned mine = 0;
+  for (size_t row = wave; row < rows; row += 16) {
+    const unsigned a = row_argmax(pred + row * cols, cols, lane);
+    const unsigned b = row_argmax(truth + row * cols, cols, lane);
+    mine += a == b ? 1u : 0u;
+  }
+  if (lane == 0) counts[wave] = mine;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned long long total = 0;
+    for (int w = 0; w < 16; ++w) total += counts[w];
+    hits[0] = total;
+    if (hits_mirror) hits_mirror[0] = total;
+  }
+}
+
 int launch_accuracy(hipStream_t s, const double* pred, const double* truth, size_t rows,
-                    size_t cols, unsigned long long* hits) {
+                    size_t cols, unsigned long long* hits, unsigned long long* hits_mirror,
+                    bool* mirrored) {
+  if (mirrored) *mirrored = false;
+  if (hits_mirror && mirrored && rows * cols <= (size_t)1 << 16) {
+    hipLaunchKernelGGL(accuracy_small_kernel, dim3(1), dim3(1024), 0, s, pred, truth, rows, cols, hits,
+                       hits_mirror);
+    RST_HIP(hipGetLastError());
+    *mirrored = true;
+    return RST_OK;
+  }
   hipLaunchKernelGGL(zero_hits_kernel, dim3(1), dim3(1), 0, s, hits);
   if (rows && cols)
     hipLaunchKernelGGL(accuracy_kernel, dim3(grid_for(rows, kBlock / 64)), dim3(kBlock), 0, s, pred,
