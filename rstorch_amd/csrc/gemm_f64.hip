@@ -310,8 +310,10 @@ __device__ __forceinline__ void colsum_finish(double partial, double* __restrict
 // latency: the tiles of D K steps are requested together, land in D LDS stages and are multiplied
 // in K order, so a short contraction pays one trip to memory instead of one per step.  The
 // accumulation order, and with it every bit of the result, is the same either way.
+// lds_a / lds_b: room for kStages tiles of the respective operand (tile_lds_doubles).
 template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC, int BURST = 0>
-__device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block) {
+__device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block, double* __restrict__ lds_a_base,
+                                          double* __restrict__ lds_b_base) {
   constexpr int kThreads = WGM * WGN * 64;
   using GA = TileGeom<BM, A_KC, kThreads>;
   using GB = TileGeom<BN, B_KC, kThreads>;
@@ -320,8 +322,8 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block) 
   static_assert(WM % 16 == 0 && WN % 16 == 0, "wave block must be whole MFMA tiles");
 
   constexpr int kStages = BURST > 0 ? BURST : 2;
-  __shared__ __attribute__((aligned(16))) double lds_a[kStages][GA::size];
-  __shared__ __attribute__((aligned(16))) double lds_b[kStages][GB::size];
+  auto lds_a = [&](int stage) { return lds_a_base + stage * GA::size; };
+  auto lds_b = [&](int stage) { return lds_b_base + stage * GB::size; };
 
   // Workgroups are handed to the 8 XCDs round-robin; renumber them so that each XCD (and
   // its private L2) works on one compact patch of the tile grid, then walk the patch in
@@ -410,46 +412,52 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block) 
 #pragma unroll
       for (int d = 0; d < kStages; ++d)
         if (k0 + d < nk) {
-          store_tile<BM, A_KC, kThreads>(lds_a[d], ra[d], tid);
-          store_tile<BN, B_KC, kThreads>(lds_b[d], rb[d], tid);
+          store_tile<BM, A_KC, kThreads>(lds_a(d), ra[d], tid);
+          store_tile<BN, B_KC, kThreads>(lds_b(d), rb[d], tid);
         }
       __syncthreads();
 #pragma unroll
       for (int d = 0; d < kStages; ++d)
-        if (k0 + d < nk) multiply(lds_a[d], lds_b[d]);
+        if (k0 + d < nk) multiply(lds_a(d), lds_b(d));
       __syncthreads();
     }
   } else {
     v2d ra[GA::loads], rb[GB::loads];
     if (nk > kt0) {
       fetch(kt0, ra, rb);
-      store_tile<BM, A_KC, kThreads>(lds_a[0], ra, tid);
-      store_tile<BN, B_KC, kThreads>(lds_b[0], rb, tid);
+      store_tile<BM, A_KC, kThreads>(lds_a(0), ra, tid);
+      store_tile<BN, B_KC, kThreads>(lds_b(0), rb, tid);
     }
     __syncthreads();
     for (int kt = kt0; kt < nk; ++kt) {
       const int cur = (kt - kt0) & 1;
       const bool more = kt + 1 < nk;
       if (more) fetch(kt + 1, ra, rb);  // in flight while this step is multiplied
-      multiply(lds_a[cur], lds_b[cur]);
+      multiply(lds_a(cur), lds_b(cur));
       if (more) {
-        store_tile<BM, A_KC, kThreads>(lds_a[cur ^ 1], ra, tid);
-        store_tile<BN, B_KC, kThreads>(lds_b[cur ^ 1], rb, tid);
+        store_tile<BM, A_KC, kThreads>(lds_a(cur ^ 1), ra, tid);
+        store_tile<BN, B_KC, kThreads>(lds_b(cur ^ 1), rb, tid);
       }
       __syncthreads();
     }
   }
   if (!A_KC) {
-    if (do_colsum) colsum_finish<BM, kThreads>(colsum_partial, lds_b[0], tid, m0, split, p);
+    if (do_colsum) colsum_finish<BM, kThreads>(colsum_partial, lds_b(0), tid, m0, split, p);
   }
 
   write_block<TM, TN>(p, &acc[0][0], m0 + wm * WM, n0 + wn * WN, lr, lk, split);
 }
 
+// LDS doubles that gemm_tile needs for one operand
+template <int EXT, bool KC, int THREADS, int BURST>
+constexpr int tile_lds_doubles() { return (BURST > 0 ? BURST : 2) * TileGeom<EXT, KC, THREADS>::size; }
+
 template <int BM, int BN, int WGM, int WGN, bool A_KC, bool B_KC, bool VEC, int BURST = 0>
-__global__ __launch_bounds__(WGM * WGN * 64, (WGM * WGN >= 8 ? 4 : 2)) void gemm_f64_mfma(
+__global__ __launch_bounds__(WGM * WGN * 64, (BURST > 0 ? 1 : WGM * WGN >= 8 ? 4 : 2)) void gemm_f64_mfma(
     const GemmParams p) {
-  gemm_tile<BM, BN, WGM, WGN, A_KC, B_KC, VEC, BURST>(p, (int)blockIdx.x);
+  __shared__ __attribute__((aligned(16))) double lds_a[tile_lds_doubles<BM, A_KC, WGM * WGN * 64, BURST>()];
+  __shared__ __attribute__((aligned(16))) double lds_b[tile_lds_doubles<BN, B_KC, WGM * WGN * 64, BURST>()];
+  gemm_tile<BM, BN, WGM, WGN, A_KC, B_KC, VEC, BURST>(p, (int)blockIdx.x, lds_a, lds_b);
 }
 
 // Up to kMaxGroup small products of the same operand layouts in one grid of 32x32 tiles (the
@@ -462,15 +470,35 @@ struct GemmGroup {
   int count;
   int first_block[kMaxGroup + 1];
   int first_reduce_block[kMaxGroup + 1];
+  unsigned char layout[kMaxGroup];  // bit 0: A contraction-contiguous, bit 1: B (the mixed kernel reads it)
   GemmParams p[kMaxGroup];
 };
 static_assert(sizeof(GemmGroup) <= 4096, "a group travels as one kernel argument");
 
 template <bool A_KC, bool B_KC, int BURST>
-__global__ __launch_bounds__(256, 2) void gemm_f64_mfma_group(const GemmGroup g) {
+__global__ __launch_bounds__(256, (BURST > 0 ? 1 : 2)) void gemm_f64_mfma_group(const GemmGroup g) {
+  __shared__ __attribute__((aligned(16))) double lds_a[tile_lds_doubles<32, A_KC, 256, BURST>()];
+  __shared__ __attribute__((aligned(16))) double lds_b[tile_lds_doubles<32, B_KC, 256, BURST>()];
   int i = 0;
   while (i + 1 < g.count && (int)blockIdx.x >= g.first_block[i + 1]) ++i;
-  gemm_tile<32, 32, 2, 2, A_KC, B_KC, true, BURST>(g.p[i], (int)blockIdx.x - g.first_block[i]);
+  gemm_tile<32, 32, 2, 2, A_KC, B_KC, true, BURST>(g.p[i], (int)blockIdx.x - g.first_block[i], lds_a, lds_b);
+}
+
+// The same with a layout per problem (a layer's input gradient next to its weight gradient).
+template <int BURST>
+__global__ __launch_bounds__(256, (BURST > 0 ? 1 : 2)) void gemm_f64_mfma_mixed_group(const GemmGroup g) {
+  // an output-contiguous tile is the larger of the two layouts
+  __shared__ __attribute__((aligned(16))) double lds_a[tile_lds_doubles<32, false, 256, BURST>()];
+  __shared__ __attribute__((aligned(16))) double lds_b[tile_lds_doubles<32, false, 256, BURST>()];
+  int i = 0;
+  while (i + 1 < g.count && (int)blockIdx.x >= g.first_block[i + 1]) ++i;
+  const int block = (int)blockIdx.x - g.first_block[i];
+  switch (g.layout[i]) {
+    case 0: gemm_tile<32, 32, 2, 2, false, false, true, BURST>(g.p[i], block, lds_a, lds_b); break;
+    case 1: gemm_tile<32, 32, 2, 2, true, false, true, BURST>(g.p[i], block, lds_a, lds_b); break;
+    case 2: gemm_tile<32, 32, 2, 2, false, true, true, BURST>(g.p[i], block, lds_a, lds_b); break;
+    default: gemm_tile<32, 32, 2, 2, true, true, true, BURST>(g.p[i], block, lds_a, lds_b); break;
+  }
 }
 
 // ---- 128x128 tiles fed by direct global -> LDS loads ------------------------------------------
@@ -1120,8 +1148,8 @@ void plan_group_member(GemmParams& p) {
 }  // namespace
 
 bool can_group_gemm(const GemmDesc& d) {
-  // the grouped kernel exists for the weight-gradient layouts with 16-byte loads
-  if (d.M <= 0 || d.N <= 0 || d.a_kc || d.b_kc || !desc_vec_ok(d)) return false;
+  // the grouped kernels use 16-byte loads
+  if (d.M <= 0 || d.N <= 0 || !desc_vec_ok(d)) return false;
   const GemmParams p = make_params(d);
   int slices = 0;
   return choose_route(p, true, &slices) == Route::kTile32;
@@ -1139,6 +1167,7 @@ int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count) {
   g.count = count;
   long long blocks = 0, reduce_blocks = 0;
   size_t ws_used = 0;
+  bool mixed = false;  // anything but weight-gradient layouts
   for (int i = 0; i < count; ++i) {
     if (!can_group_gemm(d[i])) return fail(RST_ERR_INVALID_ARGUMENT, "contraction %d cannot join a group", i);
     if (d[i].workspace != d[0].workspace || d[i].workspace_count != d[0].workspace_count)
@@ -1147,6 +1176,8 @@ int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count) {
     plan_group_member(p);
     g.first_block[i] = (int)blocks;
     g.first_reduce_block[i] = (int)reduce_blocks;
+    g.layout[i] = (unsigned char)((d[i].a_kc ? 1 : 0) | (d[i].b_kc ? 2 : 0));
+    mixed = mixed || g.layout[i] != 0;
     blocks += (long long)p.tiles_m * p.tiles_n * p.split_k;
     if (p.split_k > 1) {
       // every problem gets a region of its own in the shared workspace
@@ -1162,7 +1193,12 @@ int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count) {
   if (blocks > 0x7fffffffLL || reduce_blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
   g.first_block[count] = (int)blocks;
   g.first_reduce_block[count] = (int)reduce_blocks;
-  if (blocks <= compute_units())
+  const bool burst = blocks <= compute_units();
+  if (mixed && burst)
+    hipLaunchKernelGGL((gemm_f64_mfma_mixed_group<kBurst>), dim3((unsigned)blocks), dim3(256), 0, stream, g);
+  else if (mixed)
+    hipLaunchKernelGGL((gemm_f64_mfma_mixed_group<0>), dim3((unsigned)blocks), dim3(256), 0, stream, g);
+  else if (burst)
     hipLaunchKernelGGL((gemm_f64_mfma_group<false, false, kBurst>), dim3((unsigned)blocks), dim3(256), 0, stream, g);
   else
     hipLaunchKernelGGL((gemm_f64_mfma_group<false, false, 0>), dim3((unsigned)blocks), dim3(256), 0, stream, g);

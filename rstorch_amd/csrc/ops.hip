@@ -70,32 +70,35 @@ int rst_linear_backward(rst_engine* e, const double* grad, const double* x, cons
   RST_TRY(check_dim(in_features, "in_features"));
   RST_TRY(check_dim(out_features, "out_features"));
   const double n = (double)batch;
-  {  // grad_weight[out,in] = (grad^T . x) / n
-    GemmDesc d{};
-    d.A = grad; d.B = x; d.C = grad_weight;
-    d.M = (int)out_features; d.N = (int)in_features; d.K = (int)batch;
-    d.lda = (long)out_features; d.ldb = (long)in_features; d.ldc = (long)in_features;
-    d.a_kc = false; d.b_kc = false;
-    d.epilogue = EPI_DIVIDE; d.divisor = n;
-    // grad_bias[1,out] = colsum(grad) / n rides along in the same launch
-    d.colsum = (in_features > 0 && batch > 0) ? grad_bias : nullptr;
-    d.colsum_div = n;
-    d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
-      RST_TRY(launch_gemm(e->stream, d));
-    if (grad_bias && !d.colsum)
-      RST_TRY(launch_column_mean(e->stream, grad, grad_bias, batch, out_features, n));
+  GemmDesc dw{};  // grad_weight[out,in] = (grad^T . x) / n
+  dw.A = grad; dw.B = x; dw.C = grad_weight;
+  dw.M = (int)out_features; dw.N = (int)in_features; dw.K = (int)batch;
+  dw.lda = (long)out_features; dw.ldb = (long)in_features; dw.ldc = (long)in_features;
+  dw.a_kc = false; dw.b_kc = false;
+  dw.epilogue = EPI_DIVIDE; dw.divisor = n;
+  // grad_bias[1,out] = colsum(grad) / n rides along in the same launch
+  dw.colsum = (in_features > 0 && batch > 0) ? grad_bias : nullptr;
+  dw.colsum_div = n;
+  dw.workspace = e->d_gemm_ws; dw.workspace_count = e->gemm_ws_count;
+  GemmDesc dx{};  // grad_input[batch,in] = grad . weight
+  dx.A = grad; dx.B = weight; dx.C = grad_input;
+  dx.M = (int)batch; dx.N = (int)in_features; dx.K = (int)out_features;
+  dx.lda = (long)out_features; dx.ldb = (long)in_features; dx.ldc = (long)in_features;
+  dx.a_kc = true; dx.b_kc = false;
+  dx.epilogue = relu_mask_source ? EPI_MASK : EPI_NONE;
+  dx.mask = relu_mask_source; dx.ldmask = (long)in_features;
+  dx.workspace = e->d_gemm_ws; dx.workspace_count = e->gemm_ws_count;
+  // two small products that do not depend on each other: one grid
+  if (grad_input && can_group_gemm(dw) && can_group_gemm(dx) &&
+      gemm_group_workspace(dw) + gemm_group_workspace(dx) <= e->gemm_ws_count) {
+    const GemmDesc both[2] = {dw, dx};
+    RST_TRY(launch_gemm_group(e->stream, both, 2));
+  } else {
+    RST_TRY(launch_gemm(e->stream, dw));
+    if (grad_input) RST_TRY(launch_gemm(e->stream, dx));
   }
-  if (grad_input) {  // grad_input[batch,in] = grad . weight
-    GemmDesc d{};
-    d.A = grad; d.B = weight; d.C = grad_input;
-    d.M = (int)batch; d.N = (int)in_features; d.K = (int)out_features;
-    d.lda = (long)out_features; d.ldb = (long)in_features; d.ldc = (long)in_features;
-    d.a_kc = true; d.b_kc = false;
-    d.epilogue = relu_mask_source ? EPI_MASK : EPI_NONE;
-    d.mask = relu_mask_source; d.ldmask = (long)in_features;
-    d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
-      RST_TRY(launch_gemm(e->stream, d));
-  }
+  if (grad_bias && !dw.colsum)
+    RST_TRY(launch_column_mean(e->stream, grad, grad_bias, batch, out_features, n));
   return RST_OK;
 }
 
