@@ -313,7 +313,7 @@ def main():
     d = kernels[dominant]
     launches = [r for r in recs if r["kernel"] == dominant]
     flops_per_launch = sum(r["flops"] for r in launches) / len(launches)
-    roofline = {"kernel": "gemm_f64_mfma (" + dominant + ")", "bound": "mfma",
+    roofline = {"kernel": "gemm_f64_mfma_dma (" + dominant + ")", "bound": "mfma",
                 "achieved": d["achieved_tflops"], "peak": PEAK_FP64_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": d["frac"], "traffic": C4_TRAFFIC_BYTES_PER_LAUNCH.get(dominant),
                 "traffic_unit": "bytes per launch (L2 misses + write-backs, rocprofv3 FETCH_SIZE/WRITE_SIZE)",
