@@ -178,6 +178,9 @@ struct rst_engine {
 namespace rst {
 int engine_activate(rst_engine* e);
 int engine_reserve_row_loss(rst_engine* e, size_t rows);
-int engine_cross_entropy(rst_engine* e, const double* pred, const double* truth, double* grad_out,
-                         double* prob_out, size_t rows, size_t cols, double* host_loss);
+// row_loss: [rows] scratch of the caller, or NULL for the engine's own (which is reallocated when
+// it grows: only for launches that are not recorded into a graph)
+int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, const double* truth,
+                         double* grad_out, double* prob_out, size_t rows, size_t cols,
+                         double* host_loss);
 }  // namespace rst

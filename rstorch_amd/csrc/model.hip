@@ -61,6 +61,9 @@ struct rst_model {
   size_t batch_capacity = 0;
   size_t batch = 0;
   double* loss_grad = nullptr;  // [batch, out_width]
+  // per-row loss terms [batch]: owned by the model, because a recorded step graph keeps the address
+  // (a buffer shared through the engine could be reallocated by another caller between two replays)
+  double* row_loss = nullptr;
   const double* logits = nullptr;
   // state machine (mirrors the Option::take() caches of the reference)
   bool forward_valid = false;
@@ -98,7 +101,10 @@ namespace {
 
 constexpr size_t kMaxStepGraphs = 8;
 
+// A graph executable is only destroyed once nothing enqueued on the stream can still be running it.
 void drop_graph(rst_model* m) {
+  if (m->graphs.empty()) return;
+  (void)hipStreamSynchronize(m->engine->stream);
   for (auto& g : m->graphs) (void)hipGraphExecDestroy(g.exec);
   m->graphs.clear();
 }
@@ -111,7 +117,8 @@ int free_activations(rst_model* m) {
     l.out_buf = l.grad_in_buf = nullptr;
   }
   if (m->loss_grad) RST_HIP(hipFree(m->loss_grad));
-  m->loss_grad = nullptr;
+  if (m->row_loss) RST_HIP(hipFree(m->row_loss));
+  m->loss_grad = m->row_loss = nullptr;
   m->batch_capacity = 0;
   return RST_OK;
 }
@@ -128,6 +135,7 @@ int reserve_activations(rst_model* m, size_t batch) {
   }
   size_t n = batch * m->out_width;
   RST_HIP(hipMalloc(&m->loss_grad, (n ? n : 1) * sizeof(double)));
+  RST_HIP(hipMalloc(&m->row_loss, (batch ? batch : 1) * sizeof(double)));
   m->batch_capacity = batch;
   return RST_OK;
 }
@@ -243,7 +251,7 @@ int do_loss(rst_model* m, const double* truth, double* host_loss) {
   if (!truth) return fail(RST_ERR_INVALID_ARGUMENT, "truth is null");
   const size_t rows = m->batch, cols = m->out_width;
   RST_TRY(prof_begin(m, RST_KERNEL_CROSS_ENTROPY, -1, 0.0, 24.0 * (double)rows * (double)cols));
-  RST_TRY(engine_cross_entropy(e, m->logits, truth, m->loss_grad, nullptr, rows, cols, nullptr));
+  RST_TRY(engine_cross_entropy(e, m->row_loss, m->logits, truth, m->loss_grad, nullptr, rows, cols, nullptr));
   RST_TRY(prof_end(m));
   m->loss_grad_valid = true;
   if (host_loss) return rst_loss_value(e, host_loss);
@@ -639,7 +647,6 @@ int capture_step(rst_model* m, const double* x, const double* truth, size_t batc
                  hipGraphExec_t* out) {
   rst_engine* e = m->engine;
   RST_TRY(reserve_activations(m, batch));  // drops every graph if the buffers move
-  RST_TRY(engine_reserve_row_loss(e, batch));
   RST_HIP(hipStreamBeginCapture(e->stream, hipStreamCaptureModeThreadLocal));
   const int status = run_step(m, x, truth, batch, lr);
   hipGraph_t graph = nullptr;
@@ -657,6 +664,7 @@ int capture_step(rst_model* m, const double* x, const double* truth, size_t batc
     size_t victim = 0;
     for (size_t i = 1; i < m->graphs.size(); ++i)
       if (m->graphs[i].last_use < m->graphs[victim].last_use) victim = i;
+    (void)hipStreamSynchronize(e->stream);  // it may be the graph launched a moment ago
     (void)hipGraphExecDestroy(m->graphs[victim].exec);
     m->graphs.erase(m->graphs.begin() + victim);
   }

@@ -19,14 +19,18 @@ int check_dim(size_t v, const char* what) {
 
 }  // namespace
 
-int engine_cross_entropy(rst_engine* e, const double* pred, const double* truth, double* grad_out,
-                         double* prob_out, size_t rows, size_t cols, double* host_loss) {
-  RST_TRY(engine_reserve_row_loss(e, rows));
+int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, const double* truth,
+                         double* grad_out, double* prob_out, size_t rows, size_t cols,
+                         double* host_loss) {
   if (rows == 0 || cols == 0) return fail(RST_ERR_SHAPE, "cross entropy of an empty batch");
+  if (!row_loss) {  // the engine's own scratch; it moves when it grows, so nothing may keep its address
+    RST_TRY(engine_reserve_row_loss(e, rows));
+    row_loss = e->d_row_loss;
+  }
   LossMirror mirror;
   mirror.loss = e->hd_loss;
   mirror.flags = e->hd_flags;
-  RST_TRY(launch_softmax_ce(e->stream, pred, truth, grad_out, prob_out, e->d_row_loss, e->d_loss,
+  RST_TRY(launch_softmax_ce(e->stream, pred, truth, grad_out, prob_out, row_loss, e->d_loss,
                             e->d_flags, rows, cols, mirror));
   e->loss_valid = true;
   if (host_loss) return rst_loss_value(e, host_loss);
@@ -189,7 +193,7 @@ int rst_cross_entropy(rst_engine* e, const double* pred, const double* truth, do
   RST_TRY(engine_activate(e));
   if (!pred || !truth || !grad_out)
     return fail(RST_ERR_INVALID_ARGUMENT, "cross_entropy: null operand");
-  return engine_cross_entropy(e, pred, truth, grad_out, prob_out, rows, cols, host_loss);
+  return engine_cross_entropy(e, nullptr, pred, truth, grad_out, prob_out, rows, cols, host_loss);
 }
 
 int rst_loss_value(rst_engine* e, double* host_loss) {

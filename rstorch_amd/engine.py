@@ -30,9 +30,10 @@ class Event:
 
     def __del__(self):
         try:
-            if self.handle:
+            # the native event points at its engine: once that is closed it has gone with it
+            if self.handle and self._engine.handle:
                 _ffi.load().rst_event_destroy(self.handle)
-                self.handle = None
+            self.handle = None
         except Exception:
             pass
 

@@ -237,8 +237,9 @@ class BatchStager:
     def __init__(self, max_rows, x_cols, classes, depth=2, engine=None):
         self.engine = engine or default_engine()
         self.x_cols, self.classes = int(x_cols), int(classes)
+        self.max_rows = int(max_rows)
         h = ctypes.c_void_p()
-        _ffi.check(self.engine.lib.rst_stager_create(self.engine.handle, int(max_rows), self.x_cols,
+        _ffi.check(self.engine.lib.rst_stager_create(self.engine.handle, self.max_rows, self.x_cols,
                                                      self.classes, int(depth), ctypes.byref(h)))
         self.handle = h
 
@@ -275,6 +276,10 @@ class BatchStager:
     def host_slot(self, rows):
         """numpy views (x [rows, x_cols], labels [rows]) onto the pinned memory of the next free
         slot, to be filled in place and sent with ``commit(rows)``: no intermediate copy."""
+        rows = int(rows)
+        if rows < 1 or rows > self.max_rows:  # the views must stay inside the pinned slot
+            raise _ffi.ShapeError(_ffi.RST_ERR_SHAPE, "%d rows requested from a slot of %d rows"
+                                  % (rows, self.max_rows))
         px = _ffi.c_double_p()
         pl = ctypes.POINTER(ctypes.c_uint32)()
         _ffi.check(self.engine.lib.rst_stager_acquire_host(self.handle, ctypes.byref(px), ctypes.byref(pl)))

@@ -298,3 +298,42 @@ def test_paired_gradient_launches_are_bit_identical(engine, oracle, name, spec, 
         dm.forward(xd); dm.loss(yd, want_value=False)
     gins = [dm.backward(None, need_input_grad=True).to_numpy() for dm in models]
     assert np.array_equal(gins[0], gins[1])
+
+
+def test_recorded_step_survives_other_users_of_the_engine(engine, oracle):
+    """A recorded step graph must not name a buffer that another caller on the same engine can
+    reallocate: model A replays its graph, a 4096-row cross entropy and a second model grow the
+    engine-side scratch, model A replays again - and stays bit-identical to a twin that launches
+    its kernels one by one."""
+    import ctypes
+    import rstorch_amd as rs
+    from rstorch_amd import _ffi
+    spec = [("linear", 64, 48), ("relu",), ("linear", 48, 24)]
+    weights = [oracle.fill_normal((48, 64), 3, 0, 0.0, 0.125), np.zeros((1, 48)),
+               oracle.fill_normal((24, 48), 3, 2, 0.0, 0.15), np.zeros((1, 24))]
+    x = engine.from_numpy(oracle.fill_normal((256, 64), 3, 10))
+    y = engine.from_numpy(oracle.fill_one_hot(256, 24, 3, 11))
+    a, twin = rs.DeviceModel(spec, engine), rs.DeviceModel(spec, engine)
+    a.load_parameters(weights); twin.load_parameters(weights)
+    twin.graph_enable(False)
+
+    def both():
+        la, lt = a.train_step(x, y, 0.05), twin.train_step(x, y, 0.05)
+        assert la == lt
+        for (p, _), (q, _) in zip(a.parameters(), twin.parameters()):
+            np.testing.assert_array_equal(p.to_numpy(), q.to_numpy())
+
+    both(); both()  # record, replay
+    big = engine.normal(4096, 50, 3, 12)
+    t = engine.one_hot(4096, 50, 3, 13)
+    g = engine.empty(4096, 50)
+    loss = ctypes.c_double()
+    _ffi.check(engine.lib.rst_cross_entropy(engine.handle, big.ptr, t.ptr, g.ptr, None, 4096, 50,
+                                            ctypes.byref(loss)))
+    other = rs.DeviceModel(spec, engine)
+    other.load_parameters(weights)
+    xb = engine.normal(8192, 64, 3, 14)
+    yb = engine.one_hot(8192, 24, 3, 15)
+    other.train_step(xb, yb, 0.05)
+    both(); both()
+    other.close(); a.close(); twin.close()

@@ -84,6 +84,10 @@ def test_fill_pinned_slot_in_place(engine):
         x, t = st.next()
         np.testing.assert_array_equal(x.to_numpy(), np.arange(60.0).reshape(12, 5) + k)
         np.testing.assert_array_equal(t.to_numpy(), np.eye(4)[np.arange(12) % 4])
+    for rows in (0, 17, 1 << 40):  # views never reach beyond the 16-row pinned slot
+        with pytest.raises(rs.ShapeError):
+            st.host_slot(rows)
+    st.close()
 
 
 def test_checkpoint_round_trip(engine, oracle, tmp_path):
