@@ -126,6 +126,18 @@ int rst_cross_entropy(rst_engine* engine, const double* pred, const double* trut
  * logit was NaN. */
 int rst_loss_value(rst_engine* engine, double* host_loss);
 
+/* No counterpart in the reference.  For callers that cannot allocate device memory at the time of
+ * the call (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * the same computation and the same bits as rst_cross_entropy without prob_out, but the per-row
+ * loss terms, the loss word and the NaN flags live in a fixed array inside the library's device
+ * image (RST_STATIC_CROSS_ENTROPY_MAX_ROWS doubles + 256 bytes on every GPU the library runs on,
+ * held until the process ends) instead of engine buffers that grow on demand.  The call allocates
+ * and frees nothing.  More rows than the maximum: RST_ERR_UNSUPPORTED.  Every call on one GPU
+ * shares that GPU's array: calls that overlap there (two engines, two threads) race. */
+#define RST_STATIC_CROSS_ENTROPY_MAX_ROWS 65536
+int rst_cross_entropy_static(rst_engine* engine, const double* pred, const double* truth,
+                             double* grad_out, size_t rows, size_t cols, double* host_loss);
+
 /* ---- SGD (src/optim/sgd.rs:19-24) -------------------------------------------------------- */
 /* parm[i] = parm[i] - (lr * grad[i]) for every tensor in ONE launch: the product is rounded,
  * then the difference (no fused multiply-add), as in the reference.  The arrays are HOST

@@ -16,7 +16,7 @@ OBJ_DIR = os.path.join(PKG_DIR, "build")
 LIB_PATH = os.path.join(LIB_DIR, "librstorch_hip.so")
 
 SOURCES = ["engine.hip", "gemm_f64.hip", "streaming.hip", "softmax_ce.hip", "rng_fill.hip",
-           "ops.hip", "model.hip", "staging.hip"]
+           "ops.hip", "model.hip", "staging.hip", "static_scratch.hip"]
 
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",

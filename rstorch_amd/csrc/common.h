@@ -178,6 +178,8 @@ struct rst_engine {
 namespace rst {
 int engine_activate(rst_engine* e);
 int engine_reserve_row_loss(rst_engine* e, size_t rows);
+// looks up, once per device, the address of the fixed scratch behind rst_cross_entropy_static
+int static_scratch_setup(int device, hipStream_t stream);
 // row_loss: [rows] scratch of the caller, or NULL for the engine's own (which is reallocated when
 // it grows: only for launches that are not recorded into a graph)
 int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, const double* truth,

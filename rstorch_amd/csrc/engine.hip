@@ -112,9 +112,15 @@ int rst_engine_create(int device, rst_engine** out) {
     *e->h_hits = 0;
   }
   if (err == hipSuccess) err = hipMemsetAsync(e->d_flags, 0, 4 * sizeof(int), e->stream);
-  if (err == hipSuccess) err = hipStreamSynchronize(e->stream);
   if (err != hipSuccess) {
     int status = fail_hip(err, "engine set-up", __FILE__, __LINE__);
+    rst_engine_destroy(e);
+    return status;
+  }
+  int status = static_scratch_setup(device, e->stream);
+  if (status == RST_OK && (err = hipStreamSynchronize(e->stream)) != hipSuccess)
+    status = fail_hip(err, "engine set-up", __FILE__, __LINE__);
+  if (status != RST_OK) {
     rst_engine_destroy(e);
     return status;
   }
