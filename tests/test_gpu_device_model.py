@@ -77,6 +77,24 @@ def test_hundred_fused_steps(engine, oracle):
         assert abs(got - want) <= 1e-8 * abs(want), "step %d" % step
 
 
+def test_hundred_fused_steps_at_batch_8192(engine, oracle):
+    """The 100-step criterion (loss within 1e-8 relative) on the README network at batch 8192, fresh
+    inputs every step; the parameters after the run within 1e-8 as well."""
+    import rstorch_amd as rs
+    dm, ref = pair(rs, oracle, README_MLP, 6)
+    oracle.set_threads(8)
+    try:
+        for step in range(100):
+            x, y = batch_data(oracle, 8192, 784, 10, 17, step)
+            got = dm.train_step(x, y, 0.01)
+            want = ref.train_step(x, y, 0.01)
+            assert abs(got - want) <= 1e-8 * abs(want), "step %d" % step
+    finally:
+        oracle.set_threads(1)
+    for (p, _), (rp, _) in zip(dm.parameters(), ref.parameters()):
+        assert rel_err(p.to_numpy(), rp) <= 1e-8
+
+
 def test_basic_model_from_sequential(engine, oracle):
     """BasicModel::step (src/model.rs:19-27) == the layer-by-layer README loop."""
     import rstorch_amd as rs
