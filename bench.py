@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the rstorch f64 training step on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra] [--eager]
 
 Workload (BASELINE.json configs[4], the one the target sentence is quoted on): the deep MLP
 (Linear(4096,4096)+ReLU) x 8 -> Linear(4096,32768), f64, batch 1024, CrossEntropyLoss,
@@ -12,11 +12,17 @@ backward, SGD through the C ABI (rst_model_train_step), inputs resident in HBM.
 Prints ONE JSON line.  `roofline` is for the FP64-MFMA contraction kernel instantiation with the
 largest share of the step; per-launch durations come from HIP events recorded on the engine's
 stream around every launch of the timed steps.  `cpu_baseline` is the CPU restatement (oracle)
-timed on this host: a bounded sample of the same network at a reduced batch, extrapolated.
+timed on this host, single thread like the reference: one whole C4 step at the full batch.
+`other_configs` holds, for configs[0..2], the graph-replay rate, a second pass with per-launch events
+(contraction TFLOP/s against the FP64 MFMA peak) and the oracle timed on the same configuration;
+`readme_loop_b32` is the reference's README loop shape (layer by layer, loss and accuracy read back
+every step) run by the C++ host mirror in a child process.
 """
 import argparse
 import json
 import os
+import re
+import subprocess
 import sys
 import time
 
@@ -33,6 +39,8 @@ PEAK_HBM_GBPS = 8000.0
 # A launch = the contraction plus, for the one that is contracted as two K slices (the head's input
 # gradient), the reduction of the two partial results (134.3 MB); the weight gradient carries the SGD
 # update of its layer.
+C4_TRAFFIC_SOURCE = {"profile": "profiles/c4_hbm_traffic.md",
+                     "kernels_as_of_commit": "379da82 (contraction kernels unchanged since)"}
 C4_TRAFFIC_BYTES_PER_LAUNCH = {
     "linear_forward": (8 * 436.4e6 + 3847.5e6) / 9,
     "grad_weight": (8 * 859.2e6 + 6972.6e6) / 9,
@@ -174,12 +182,62 @@ def bench_sgd_c3(rs, eng, iters=20):
     return res
 
 
-def bench_small(rs, eng, spec, batch, normal, steps, warmup):
+def contraction_summary(recs, steps):
+    """Contraction launches of a profiled pass: rate against the FP64 MFMA peak, the class with the
+    largest share, and the step's launch count."""
+    kernels = summarise(recs, steps)
+    kinds = [k for k in ("linear_forward", "grad_weight", "grad_input", "grad_pair") if k in kernels]
+    ms = sum(kernels[k]["ms_per_step"] for k in kinds)
+    flops = sum(r["flops"] for r in recs if r["kernel"] in kinds) / steps
+    dominant = max(kinds, key=lambda k: kernels[k]["ms_per_step"])
+    return kernels, {
+        "tflops": flops / (ms * 1e-3) / 1e12, "frac": flops / (ms * 1e-3) / 1e12 / PEAK_FP64_MFMA_TFLOPS,
+        "flops_per_step": flops, "ms_per_step": ms, "launches_per_step": len(recs) / steps,
+        "dominant": dominant, "dominant_tflops": kernels[dominant]["achieved_tflops"],
+        "dominant_frac": kernels[dominant]["frac"],
+        "dominant_avg_launch_ms": kernels[dominant]["avg_launch_ms"],
+        "first_layer_input_gradient": "skipped (the README loop discards it)"}
+
+
+def bench_small(rs, eng, spec, batch, normal, steps, warmup, eager, profile_steps):
+    """steps_per_s: the fused step as shipped (graph replay unless --eager).  `contractions`: a
+    second pass with an event after every launch (plain launches, one weight gradient per layer)."""
     dm, x, y = make_model(rs, eng, spec, batch, normal)
+    if eager:
+        dm.graph_enable(False)
     wall, dev_ms, loss, _ = time_steps(eng, dm, x, y, steps, warmup, False)
+    out = {"batch": batch, "steps": steps, "ms_per_step": wall * 1e3 / steps,
+           "steps_per_s": steps / wall, "samples_per_s": steps / wall * batch, "final_loss": loss,
+           "launch_mode": "plain launches" if eager else "graph replay"}
+    _, _, _, recs = time_steps(eng, dm, x, y, profile_steps, 2, True)
+    kernels, out["contractions"] = contraction_summary(recs, profile_steps)
+    out["kernels"] = {k: {"avg_launch_us": v["avg_launch_ms"] * 1e3, "launches_per_step": v["launches_per_step"],
+                          "frac": v["frac"], "bound": v["bound"]} for k, v in kernels.items()}
     dm.close()
-    return {"batch": batch, "steps": steps, "ms_per_step": wall * 1e3 / steps,
-            "steps_per_s": steps / wall, "samples_per_s": steps / wall * batch, "final_loss": loss}
+    return out
+
+
+def readme_loop_child():
+    """The README-shaped loop (README.md:64-74) through the C++ mirror of the module interface, in a
+    process of its own, started before this one touches the GPU."""
+    exe = os.path.join(ROOT, "rstorch_amd", "cpp", "bin", "readme_loop")
+    if not os.path.exists(exe):
+        return {"error": "rstorch_amd/cpp/bin/readme_loop is not built (__graft_entry__.build())"}
+    try:
+        proc = subprocess.run([exe, "3", "1875"], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                              text=True, timeout=120)
+    except subprocess.TimeoutExpired:
+        return {"error": "readme_loop did not finish in 120 s"}
+    rates = [float(m) for m in re.findall(r"\((\d+) steps/s\)", proc.stdout)]
+    losses = [float(m) for m in re.findall(r"Avarage loss ([0-9.]+)", proc.stdout)]
+    if proc.returncode != 0 or not rates:
+        return {"error": "readme_loop failed: %s" % (proc.stderr.strip() or proc.stdout.strip())[:200]}
+    return {"batch": 32, "steps_per_epoch": 1875, "epochs": len(rates), "steps_per_s": rates[-1],
+            "samples_per_s": rates[-1] * 32, "steps_per_s_per_epoch": rates,
+            "average_loss_per_epoch": losses,
+            "shape": "model.forward -> loss.forward(pred.clone(), y.clone()) -> accuracy(pred, y) -> "
+                     "model.backward(loss.backward()) -> optim.step(model), layer by layer; the loss and "
+                     "the accuracy are read back every step; the first layer's input gradient is computed"}
 
 
 def bench_staged(rs, eng, spec, batch, normal, steps, warmup, in_place=False):
@@ -229,10 +287,55 @@ def bench_staged(rs, eng, spec, batch, normal, steps, warmup, in_place=False):
             "host_bytes_per_step": batch * (8 * n_in + 4), "final_loss": loss}
 
 
+def cpu_baseline_small(spec, batch, normal, steps):
+    """The oracle, single thread, on one of the small configurations: `steps` whole steps timed."""
+    import numpy as np
+    import oracle
+    oracle.build()
+    oracle.set_threads(1)
+    ref = oracle.Model(spec)
+    for i, (p, _) in enumerate(ref.parameters()):
+        if p.shape[0] > 1:
+            p[...] = oracle.fill_normal(p.shape, SEED, i, 0.0, p.shape[1] ** -0.5)
+    n_in = next(l[1] for l in spec if l[0] == "linear")
+    n_out = [l[2] for l in spec if l[0] == "linear"][-1]
+    x = oracle.fill_normal((batch, n_in), SEED, 1000) if normal else oracle.fill_uniform((batch, n_in), SEED, 1000)
+    y = oracle.fill_one_hot(batch, n_out, SEED, 1001)
+    ref.train_step(x, y, LR)  # allocates the activation buffers
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        ref.train_step(x, y, LR)
+    dt = time.perf_counter() - t0
+    return {"value": steps / dt, "unit": "steps/s", "cores": 1, "kind": "port",
+            "sample": "%d whole steps of the oracle, single thread" % steps, "s_per_step": dt / steps}
+
+
+def cpu_baseline_sgd_c3(calls=10):
+    """configs[3] on the host: the oracle's SGD::step over 268.6 M parameters, single thread."""
+    import numpy as np
+    import oracle
+    total = 64 * (2048 * 2048 + 2048)
+    parm = np.full(total, 0.02)
+    grad = np.full(total, 1e-3)
+    L = oracle.lib()
+    oracle.set_threads(1)
+    L.rsto_sgd_step(oracle._ptr(parm), oracle._ptr(grad), total, LR)
+    t0 = time.perf_counter()
+    for _ in range(calls):
+        L.rsto_sgd_step(oracle._ptr(parm), oracle._ptr(grad), total, LR)
+    dt = (time.perf_counter() - t0) / calls
+    return {"value": 1.0 / dt, "unit": "steps/s", "cores": 1, "kind": "port",
+            "sample": "%d calls of the oracle's SGD::step over %d parameters" % (calls, total),
+            "achieved_gbps": 24.0 * total / dt / 1e9}
+
+
 def cpu_baseline(sample_batches=(64, 256)):
-    """The oracle (CPU restatement of the reference) on the C4 network at two reduced batches.
-    A step costs t(B) = a + b*B (a: SGD and operand packing, independent of the batch; b: the
-    per-row contraction and loss work), so two timed steps give t(1024) = a + 1024*b."""
+    """The oracle (CPU restatement of the reference) on the C4 network: one whole step at the full
+    batch of 1024, single thread, is the baseline.  Beside it, as a cross-check and for the all-cores
+    figure, two reduced batches: a step costs t(B) = a + b*B (a: SGD and operand packing, independent
+    of the batch; b: the per-row contraction and loss work), so two timed steps give t(1024).
+    The oracle's weights here are uniform with the variance of N(0, 1/fan_in) (cheaper to draw;
+    the timing does not depend on the distribution)."""
     import numpy as np
     import oracle
     oracle.build()
@@ -257,10 +360,16 @@ def cpu_baseline(sample_batches=(64, 256)):
         fixed = max(times[b_lo] - slope * b_lo, 0.0)
         t_full = fixed + slope * C4_BATCH
         out[label] = {"threads": threads, "t_step_s": {str(B): times[B] for B in sample_batches},
-                      "per_row_s": slope, "batch_independent_s": fixed, "t_full_step_s": t_full,
-                      "steps_per_s": 1.0 / t_full}
+                      "per_row_s": slope, "batch_independent_s": fixed, "t_full_step_s_fitted": t_full,
+                      "steps_per_s_fitted": 1.0 / t_full}
+    # the baseline proper: one whole step at the full batch, single thread
     oracle.set_threads(1)
-    del ref
+    full = (oracle.fill_normal((C4_BATCH, 4096), SEED, 1000), oracle.fill_one_hot(C4_BATCH, 32768, SEED, 1001))
+    t0 = time.perf_counter()
+    ref.train_step(*full, LR)
+    out["single"]["t_full_step_s"] = time.perf_counter() - t0
+    out["single"]["steps_per_s"] = 1.0 / out["single"]["t_full_step_s"]
+    del ref, full
     return out, sample_batches, cores
 
 
@@ -271,6 +380,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
+    ap.add_argument("--eager", action="store_true",
+                    help="plain kernel launches instead of graph replay (the library also does this by "
+                         "itself when a rocprofiler-sdk tool is attached to the process)")
     ap.add_argument("--sgd-only", action="store_true",
                     help="time only SGD::step over the configs[3] parameter set (for profiler runs)")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -280,6 +392,12 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this backend runs the training step on ONE GPU; --gpus %d is not "
                  "supported (no collectives are part of this build)" % args.gpus)
+
+    # a child process that uses the GPU runs before this process opens it
+    readme_loop = None
+    if not (args.no_extra or args.sgd_only):
+        log("README-shaped loop (C++ mirror, child process) ...")
+        readme_loop = readme_loop_child()
 
     import rstorch_amd as rs
     eng = rs.default_engine()
@@ -300,6 +418,8 @@ def main():
         del src, dst
 
     dm, x, y = make_model(rs, eng, C4_SPEC, C4_BATCH, True)
+    if args.eager:
+        dm.graph_enable(False)
     tensors, params = dm.parameter_count()
     wall, dev_ms, loss, recs = time_steps(eng, dm, x, y, args.steps, args.warmup, True)
     ms_per_step = wall * 1e3 / args.steps
@@ -317,6 +437,7 @@ def main():
                 "achieved": d["achieved_tflops"], "peak": PEAK_FP64_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": d["frac"], "traffic": C4_TRAFFIC_BYTES_PER_LAUNCH.get(dominant),
                 "traffic_unit": "bytes per launch (L2 misses + write-backs, rocprofv3 FETCH_SIZE/WRITE_SIZE)",
+                "traffic_source": C4_TRAFFIC_SOURCE,
                 "algorithmic_bytes_per_launch": sum(r["bytes"] for r in launches) / len(launches),
                 "avg_launch_ms": d["avg_launch_ms"], "flops_per_launch": flops_per_launch}
     gemm_ms = sum(kernels[k]["ms_per_step"] for k in gemm_kinds)
@@ -337,7 +458,11 @@ def main():
                    "device": info["name"], "device_ms_per_step": dev_ms / args.steps,
                    "device_ms_per_step_median": per_step[len(per_step) // 2],
                    "device_ms_per_step_min": per_step[0],
-                   "final_loss": loss, "per_launch_events": True},
+                   "final_loss": loss, "per_launch_events": True,
+                   # the loss is computed on the device every step but the host does not read it inside
+                   # the timed loop (one read after the last step); the README-shaped loop, which reads
+                   # the loss and the accuracy every step, is reported as readme_loop_b32
+                   "per_step_loss_read": False},
         "roofline": roofline,
         "contractions": all_gemm,
         "kernels": kernels,
@@ -349,10 +474,11 @@ def main():
         result["relu_standalone"] = bench_relu(rs, eng)
         log("other configurations ...")
         result["other_configs"] = {
-            "C0_readme_b32": bench_small(rs, eng, C01_SPEC, 32, False, 2000, 100),
-            "C1_readme_b8192": bench_small(rs, eng, C01_SPEC, 8192, False, 200, 20),
-            "C2_wide_b2048": bench_small(rs, eng, C2_SPEC, 2048, True, 20, 3),
+            "C0_readme_b32": bench_small(rs, eng, C01_SPEC, 32, False, 2000, 100, args.eager, 200),
+            "C1_readme_b8192": bench_small(rs, eng, C01_SPEC, 8192, False, 200, 20, args.eager, 50),
+            "C2_wide_b2048": bench_small(rs, eng, C2_SPEC, 2048, True, 20, 3, args.eager, 10),
         }
+        result["readme_loop_b32"] = readme_loop
         log("host-fed (PCIe-inclusive) runs ...")
         result["host_fed"] = {
             "C1_readme_b8192": bench_staged(rs, eng, C01_SPEC, 8192, False, 100, 10),
@@ -366,14 +492,24 @@ def main():
         result["cpu_baseline"] = {
             "value": cpu["single"]["steps_per_s"], "unit": "steps/s", "cores": 1, "kind": "port",
             "sample": "oracle (C restatement of the reference, single thread like the reference) on "
-                      "the same C4 network: one full step timed at batch %d and at batch %d, "
-                      "t(B) = a + b*B fitted and evaluated at batch 1024" % tuple(sample_batches),
+                      "the same C4 network: ONE whole step at the full batch of 1024, timed; beside it "
+                      "(detail) steps at batch %d and %d with t(B) = a + b*B fitted and evaluated at "
+                      "1024 as a cross-check" % tuple(sample_batches),
             "detail": cpu["single"],
         }
         result["cpu_baseline_all_cores"] = {
-            "value": cpu["all"]["steps_per_s"], "unit": "steps/s", "cores": cores, "kind": "port",
-            "sample": "same sample, OpenMP over the oracle's contraction blocks", "detail": cpu["all"],
+            "value": cpu["all"]["steps_per_s_fitted"], "unit": "steps/s", "cores": cores, "kind": "port",
+            "sample": "steps at batch %d and %d, OpenMP over the oracle's contraction blocks, "
+                      "t(B) = a + b*B fitted and evaluated at 1024" % tuple(sample_batches),
+            "detail": cpu["all"],
         }
+        if not args.no_extra:
+            log("CPU baselines of the other configurations ...")
+            oc = result["other_configs"]
+            oc["C0_readme_b32"]["cpu_baseline"] = cpu_baseline_small(C01_SPEC, 32, False, 1875)
+            oc["C1_readme_b8192"]["cpu_baseline"] = cpu_baseline_small(C01_SPEC, 8192, False, 20)
+            oc["C2_wide_b2048"]["cpu_baseline"] = cpu_baseline_small(C2_SPEC, 2048, True, 3)
+            result["sgd_c3"]["cpu_baseline"] = cpu_baseline_sgd_c3()
     print(json.dumps(result), flush=True)
 
 

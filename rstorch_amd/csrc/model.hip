@@ -9,6 +9,8 @@
 //             ([relu(z) > 0] == [z > 0], NaN included, both false);
 //   any ReLU not adjacent to a Linear runs the streaming kernels instead.
 #include <climits>
+#include <cstdlib>
+#include <cstring>
 #include <new>
 
 #include "common.h"
@@ -100,6 +102,22 @@ struct rst_model {
 namespace {
 
 constexpr size_t kMaxStepGraphs = 8;
+
+// Whether a new model records its step into a HIP graph.  RSTORCH_GRAPH=0/1 decides when set.
+// Otherwise graphs are on, except in a process that a rocprofiler-sdk tool is attached to (rocprofv3
+// announces itself through ROCP_TOOL_LIBRARIES): a profiled run once died inside the profiler's
+// queue-interception callback, called from the HIP runtime under the launch of a second model's
+// freshly instantiated graph after the first model's graph had been destroyed.  Nothing of this
+// library is on that stack below the runtime call, and unprofiled runs of the same sequence are
+// clean, so under a profiler the step is launched kernel by kernel - which is also what a kernel
+// trace wants to see.
+bool default_graph_enabled() {
+  if (const char* v = std::getenv("RSTORCH_GRAPH")) {
+    if (v[0] == '0' || v[0] == '1') return v[0] == '1';
+  }
+  const char* tools = std::getenv("ROCP_TOOL_LIBRARIES");
+  return !(tools && tools[0]);
+}
 
 // A graph executable is only destroyed once nothing enqueued on the stream can still be running it.
 void drop_graph(rst_model* m) {
@@ -442,6 +460,7 @@ int rst_model_create(rst_engine* e, const int* kinds, const size_t* in_features,
   rst_model* m = new (std::nothrow) rst_model();
   if (!m) return fail(RST_ERR_OUT_OF_MEMORY, "host allocation failed");
   m->engine = e;
+  m->graph_enabled = default_graph_enabled();
   m->layers.resize(layer_count);
   size_t offset = 0;
   size_t width = 0;
