@@ -383,6 +383,8 @@ def main():
     ap.add_argument("--eager", action="store_true",
                     help="plain kernel launches instead of graph replay (the library also does this by "
                          "itself when a rocprofiler-sdk tool is attached to the process)")
+    ap.add_argument("--only", choices=["C0", "C1", "C2"],
+                    help="run one of the small configurations alone (for profiler runs)")
     ap.add_argument("--sgd-only", action="store_true",
                     help="time only SGD::step over the configs[3] parameter set (for profiler runs)")
     ap.add_argument("--calibration-copy", action="store_true",
@@ -395,7 +397,7 @@ def main():
 
     # a child process that uses the GPU runs before this process opens it
     readme_loop = None
-    if not (args.no_extra or args.sgd_only):
+    if not (args.no_extra or args.sgd_only or args.only):
         log("README-shaped loop (C++ mirror, child process) ...")
         readme_loop = readme_loop_child()
 
@@ -406,6 +408,15 @@ def main():
 
     if args.sgd_only:
         print(json.dumps({"sgd_c3": bench_sgd_c3(rs, eng)}), flush=True)
+        return
+
+    small = {"C0": ("C0_readme_b32", C01_SPEC, 32, False, 2000, 100, 200),
+             "C1": ("C1_readme_b8192", C01_SPEC, 8192, False, 200, 20, 50),
+             "C2": ("C2_wide_b2048", C2_SPEC, 2048, True, 20, 3, 10)}
+    if args.only:
+        name, spec, batch, normal, steps, warmup, psteps = small[args.only]
+        print(json.dumps({name: bench_small(rs, eng, spec, batch, normal, steps, warmup, args.eager, psteps)}),
+              flush=True)
         return
 
     if args.calibration_copy:
@@ -474,10 +485,8 @@ def main():
         result["relu_standalone"] = bench_relu(rs, eng)
         log("other configurations ...")
         result["other_configs"] = {
-            "C0_readme_b32": bench_small(rs, eng, C01_SPEC, 32, False, 2000, 100, args.eager, 200),
-            "C1_readme_b8192": bench_small(rs, eng, C01_SPEC, 8192, False, 200, 20, args.eager, 50),
-            "C2_wide_b2048": bench_small(rs, eng, C2_SPEC, 2048, True, 20, 3, args.eager, 10),
-        }
+            name: bench_small(rs, eng, spec, batch, normal, steps, warmup, args.eager, psteps)
+            for name, spec, batch, normal, steps, warmup, psteps in small.values()}
         result["readme_loop_b32"] = readme_loop
         log("host-fed (PCIe-inclusive) runs ...")
         result["host_fed"] = {
