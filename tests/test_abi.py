@@ -32,6 +32,20 @@ def test_binding_and_header_agree():
     assert sorted(_ffi.EXPORTED_SYMBOLS) == declared_functions()
 
 
+def test_rust_extern_block_in_the_integration_notes_matches_the_header():
+    """INTEGRATION.md shows the Rust `extern "C"` block a maintainer of the reference would add; it
+    is generated from the header and must declare every entry point, with the current signatures."""
+    gen = os.path.join(ROOT, "include", "gen_rust_extern.py")
+    block = subprocess.run([sys.executable, gen], capture_output=True, text=True, check=True).stdout
+    assert sorted(re.findall(r"pub fn (rst_[a-z0-9_]+)", block)) == declared_functions()
+    assert block.strip() in open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    for c_type, rust in (("const double* const*", "*const *const f64"), ("double* const*", "*const *mut f64"),
+                         ("rst_engine**", "*mut *mut RstEngine"), ("const char*", "*const c_char")):
+        sys.path.insert(0, os.path.join(ROOT, "include"))
+        import gen_rust_extern
+        assert gen_rust_extern.rust_type(c_type) == rust
+
+
 def test_header_is_plain_c():
     src = '#include "rstorch_hip.h"\nint main(void){return (int)RST_OK + (int)sizeof(rst_kernel_record) * 0;}\n'
     out = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-pedantic", "-I", os.path.join(ROOT, "include"),

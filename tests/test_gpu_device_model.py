@@ -355,3 +355,98 @@ def test_recorded_step_survives_other_users_of_the_engine(engine, oracle):
     other.train_step(xb, yb, 0.05)
     both(); both()
     other.close(); a.close(); twin.close()
+
+
+# Heads far wider than the 2048 logits that the loss kernel keeps in registers (the two-walk kernel,
+# ragged widths), through the model: logits, loss, loss gradient, input and bias gradients.
+@pytest.mark.parametrize("batch,k,n", [(512, 64, 16386), (640, 48, 13000)])
+def test_wide_head_loss_through_the_model(engine, oracle, batch, k, n):
+    import ctypes
+    import rstorch_amd as rs
+    from rstorch_amd import _ffi
+    spec = [("linear", k, n)]
+    dm = rs.DeviceModel(spec)
+    w = oracle.fill_normal((n, k), 21, 0, 0.0, 1.5 * k ** -0.5)
+    b = oracle.fill_normal((1, n), 21, 1)
+    dm.load_parameters([w, b])
+    x = oracle.fill_normal((batch, k), 21, 2)
+    rng = np.random.default_rng(n)
+    y = np.zeros((batch, n))
+    y[np.arange(batch), rng.integers(0, n, batch)] = 1.0
+    y[3] = rng.random(n); y[3] /= y[3].sum()  # a soft-label row
+    logits = dm.forward(x).to_numpy()
+    oracle.set_threads(8)
+    try:
+        assert rel_err(logits, oracle.linear_forward(x, w, b)) <= TOL
+    finally:
+        oracle.set_threads(1)
+    got = dm.loss(y)
+    want, prob = oracle.cross_entropy_forward(logits, y)
+    assert abs(got - want) <= TOL * abs(want)
+    # the gradient the model keeps, against the oracle and against the operator-level call on the same logits
+    dl, dy = engine.from_numpy(logits), engine.from_numpy(y)
+    g2 = engine.empty(batch, n)
+    l2 = ctypes.c_double()
+    _ffi.check(engine.lib.rst_cross_entropy(engine.handle, dl.ptr, dy.ptr, g2.ptr, None, batch, n, ctypes.byref(l2)))
+    assert abs(got - l2.value) <= 1e-13 * abs(want)
+    gin = dm.backward(None, need_input_grad=True).to_numpy()
+    g = oracle.cross_entropy_backward(prob, y)
+    assert rel_err(gin, g @ w) <= TOL
+    assert rel_err(dm.parameters()[1][1].to_numpy(), g.sum(axis=0, keepdims=True) / batch) <= TOL
+    assert rel_err(g2.to_numpy(), g) <= TOL
+    dm.close()
+
+
+def test_wide_head_special_values(engine):
+    """-inf and +inf logits and NaN come out as in the reference's max-then-sum order
+    (softmax.rs:37-53): an all -inf row and a row holding +inf give NaN, NaN logits are an error."""
+    import rstorch_amd as rs
+    batch, k, n = 512, 32, 16384
+    dm = rs.DeviceModel([("linear", k, n)])
+    rng = np.random.default_rng(5)
+    w = rng.standard_normal((n, k)) * 0.1
+    x = rng.standard_normal((batch, k))
+    y = np.eye(n)[rng.integers(0, n, batch)]
+    b = np.zeros((1, n)); b[0, 100:9000] = -np.inf  # whole 128-column tiles of -inf: harmless
+    dm.load_parameters([w, b])
+    dm.forward(x)
+    # probabilities of exactly 0 under a zero truth are 0 * ln 0 = NaN in the reference's loss
+    # (cross_entropy.rs:38), while the gradient p - t stays finite
+    assert np.isnan(dm.loss(y))
+    logits = x @ w.T + b
+    e = np.exp(logits - logits.max(axis=1, keepdims=True))
+    g = e / e.sum(axis=1, keepdims=True) - y
+    gin = dm.backward(None, need_input_grad=True).to_numpy()
+    assert rel_err(gin, g @ w) <= TOL
+    b[0, 5] = np.inf
+    dm.load_parameters([w, b])
+    dm.forward(x)
+    assert np.isnan(dm.loss(y))  # exp(inf - inf)
+    b[...] = -np.inf
+    dm.load_parameters([w, b])
+    dm.forward(x)
+    assert np.isnan(dm.loss(y))  # 0 / 0
+    w[7, 3] = np.nan
+    dm.load_parameters([w, np.zeros((1, n))])
+    dm.forward(x)
+    with pytest.raises(rs.NanError):
+        dm.loss(y)
+    dm.close()
+
+
+def test_train_step_nan_logits(engine, oracle):
+    """NaN logits are an error (softmax.rs:38 panics) in the one-call step too; a NaN in the input
+    does not get there: max(NaN, 0) = 0 in the first ReLU, as with f64::max."""
+    import rstorch_amd as rs
+    dm, ref = pair(rs, oracle, README_MLP, 3)
+    x, y = batch_data(oracle, 32, 784, 10, 23, 0)
+    x[4, 7] = np.nan
+    got, want = dm.train_step(x, y, 0.01), ref.train_step(x, y, 0.01)
+    assert np.isfinite(got) and abs(got - want) <= TOL * abs(want)
+    params = dm.parameters()
+    bias = params[-1][0].to_numpy()
+    bias[0, 3] = np.nan
+    params[-1][0].assign(bias)
+    x[4, 7] = 0.5
+    with pytest.raises(rs.NanError):
+        dm.train_step(x, y, 0.01)
