@@ -381,8 +381,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
     ap.add_argument("--eager", action="store_true",
-                    help="plain kernel launches instead of graph replay (the library also does this by "
-                         "itself when a rocprofiler-sdk tool is attached to the process)")
+                    help="plain kernel launches instead of graph replay")
     ap.add_argument("--only", choices=["C0", "C1", "C2"],
                     help="run one of the small configurations alone (for profiler runs)")
     ap.add_argument("--sgd-only", action="store_true",

@@ -251,8 +251,7 @@ int rst_model_pair_gradients(rst_model* model, int enabled);
 /* rst_model_train_step records its launches into a HIP graph the first time it sees a given
  * (x, truth, batch, lr) and replays the graph afterwards; a different argument re-records.
  * enabled == 0 switches to plain launches (profiling does so by itself).  Default: enabled,
- * unless the environment says RSTORCH_GRAPH=0 or a rocprofiler-sdk tool is attached to the process
- * (ROCP_TOOL_LIBRARIES is set, as under rocprofv3): then plain launches. */
+ * unless the environment says RSTORCH_GRAPH=0. */
 int rst_model_graph_enable(rst_model* model, int enabled);
 /* Per-launch timing of the model's kernels: when enabled an event is recorded on the engine's
  * stream after every launch (and one before the first launch of a call); a launch's duration runs

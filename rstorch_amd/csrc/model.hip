@@ -103,20 +103,11 @@ namespace {
 
 constexpr size_t kMaxStepGraphs = 8;
 
-// Whether a new model records its step into a HIP graph.  RSTORCH_GRAPH=0/1 decides when set.
-// Otherwise graphs are on, except in a process that a rocprofiler-sdk tool is attached to (rocprofv3
-// announces itself through ROCP_TOOL_LIBRARIES): a profiled run once died inside the profiler's
-// queue-interception callback, called from the HIP runtime under the launch of a second model's
-// freshly instantiated graph after the first model's graph had been destroyed.  Nothing of this
-// library is on that stack below the runtime call, and unprofiled runs of the same sequence are
-// clean, so under a profiler the step is launched kernel by kernel - which is also what a kernel
-// trace wants to see.
+// Whether a new model records its step into a HIP graph: yes, unless RSTORCH_GRAPH=0 (plain
+// launches are handy for debuggers and for comparing the two launch modes from outside).
 bool default_graph_enabled() {
-  if (const char* v = std::getenv("RSTORCH_GRAPH")) {
-    if (v[0] == '0' || v[0] == '1') return v[0] == '1';
-  }
-  const char* tools = std::getenv("ROCP_TOOL_LIBRARIES");
-  return !(tools && tools[0]);
+  const char* v = std::getenv("RSTORCH_GRAPH");
+  return !(v && v[0] == '0');
 }
 
 // A graph executable is only destroyed once nothing enqueued on the stream can still be running it.
