@@ -19,6 +19,8 @@
 //
 // MFMA register layout (64 lanes): A fragment lane l holds A[l%16][l/16], B fragment lane l
 // holds B[l/16][l%16], and accumulator register r of lane l holds D[4*r + l/16][l%16].
+#include <cstdlib>
+
 #include "common.h"
 
 namespace rst {
@@ -818,6 +820,193 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
   dma_tile<A_KC, B_KC, WGM, WGN, STAGES, DIST>(p, (int)blockIdx.x, lds_a, lds_b);
 }
 
+// ---- 64x64 tiles fed by direct global -> LDS loads ---------------------------------------------
+// The mid-size path: products whose 128x128 tiling gives the chip too few workgroups (an 8192 x 100
+// output is 64 tiles of 128x128 but 256 of 64x64; a 100 x 784 weight gradient is 7 against 26).
+// Four wavefronts of 32x32 (2x2 MFMA tiles each), operand tiles of 64 x 16 doubles (8 KiB) moved by
+// global_load_lds_dwordx4 as in the 128x128 kernel, FOUR LDS stages with three tiles in flight (a
+// K step is only 16 MFMAs per wavefront, far shorter than a trip to memory, and with one or two
+// workgroups per CU nothing else covers it), one barrier per K step.
+//   contraction-contiguous operand: [64][16], 16-byte slots XOR-swizzled by row & 7 (as above);
+//   output-contiguous operand: [16][64] dense (a 1 KiB wavefront load is two k rows of 64), the
+//       16-byte slots of k rows 2g, 2g+1 XOR-ed with 8 * (g & 3): the four lane groups of a fragment
+//       read (k rows 2lk, 2lk+1 of a pair) then fall into four different 128-byte windows.
+// The contraction indices are assigned to MFMA steps as in the 128x128 kernel (pair s, lane group lk:
+// k = 8s + 2lk, then 8s + 2lk + 1).
+typedef const __attribute__((address_space(3))) v2d* lds_cv2d_t;
+typedef const __attribute__((address_space(3))) double* lds_cf64_t;
+
+constexpr int kT64 = 64;
+constexpr int kT64Stage = kT64 * BK;  // doubles per operand and stage
+constexpr int kT64Stages = 4;
+constexpr int kT64Dist = 3;
+
+template <bool KC>
+__device__ __forceinline__ void store_tile_dma64(double* __restrict__ lds, const v2d* __restrict__ reg, int tid) {
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int q = tid + u * 256;
+    if (KC) {
+      const int e = q >> 3, pr = q & 7;
+      *reinterpret_cast<v2d*>(lds + e * BK + 2 * (pr ^ (e & 7))) = reg[u];
+    } else {
+      const int kr = q >> 5, cp = q & 31;
+      *reinterpret_cast<v2d*>(lds + kr * kT64 + 2 * (cp ^ (8 * ((kr >> 1) & 3)))) = reg[u];
+    }
+  }
+}
+
+// one fragment of one pair of K steps (.x: first step, .y: second) for MFMA tile row/column `e0 + lr`
+template <bool KC>
+__device__ __forceinline__ v2d read_pair64(uint32_t stage_bytes, int e, int pr) {
+  if constexpr (KC) {
+    return *(lds_cv2d_t)(uintptr_t)(stage_bytes + 8u * (uint32_t)(e * BK + 2 * (pr ^ (e & 7))));
+  } else {
+    const uint32_t at = stage_bytes + 8u * (uint32_t)(2 * pr * kT64 + 2 * ((e >> 1) ^ (8 * (pr & 3))) + (e & 1));
+    v2d r;
+    r.x = *(lds_cf64_t)(uintptr_t)at;
+    r.y = *(lds_cf64_t)(uintptr_t)(at + 8u * kT64);
+    return r;
+  }
+}
+
+template <bool B_KC>
+__global__ __launch_bounds__(256, 2) void gemm_f64_mfma_dma64(const GemmParams p) {
+  constexpr bool A_KC = true;  // the forward and input-gradient layouts (where this kernel pays)
+  __shared__ __attribute__((aligned(1024))) double lds_a[kT64Stages * kT64Stage];
+  __shared__ __attribute__((aligned(1024))) double lds_b[kT64Stages * kT64Stage];
+  constexpr int BM = kT64, BN = kT64, NW = 4, TM = 2, TN = 2, CH = 2;
+  const int block = (int)blockIdx.x;
+  const int n_blocks = p.tiles_m * p.tiles_n;
+  const int split = block / n_blocks;
+  int logical;
+  {
+    const int pid = block - split * n_blocks;
+    const int xcd = pid & 7, local = pid >> 3;
+    const int base = n_blocks >> 3, rem = n_blocks & 7;
+    logical = xcd * base + (xcd < rem ? xcd : rem) + local;
+  }
+  int tile_m, tile_n;
+  {
+    constexpr int GROUP = 8;
+    const int group_size = GROUP * p.tiles_n;
+    const int group = logical / group_size;
+    const int first_m = group * GROUP;
+    const int gm = (p.tiles_m - first_m) < GROUP ? (p.tiles_m - first_m) : GROUP;
+    const int in_group = logical - group * group_size;
+    tile_m = first_m + in_group % gm;
+    tile_n = in_group / gm;
+  }
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int lr = lane & 15, lk = lane >> 4;
+
+  // tile DMA: uniform byte pointer per operand + constant 32-bit lane offsets, uniform LDS targets
+  const int wave_s = __builtin_amdgcn_readfirstlane(wave);
+  const char* a_ptr = reinterpret_cast<const char*>(p.A + (A_KC ? (size_t)m0 * p.lda : (size_t)m0));
+  const char* b_ptr = reinterpret_cast<const char*>(p.B + (B_KC ? (size_t)n0 * p.ldb : (size_t)n0));
+  uint32_t ao[CH], bo[CH];
+  int lchunk[CH];
+#pragma unroll
+  for (int h = 0; h < CH; ++h) {
+    const int c = wave + NW * h;  // chunk 0..7 of the tile
+    lchunk[h] = (wave_s + NW * h) * 128;
+    {
+      const int row = 8 * c + (lane >> 3);
+      const int rr = m0 + row < p.M ? row : p.M - 1 - m0;
+      ao[h] = 8u * (uint32_t)((size_t)rr * p.lda + 2 * ((lane & 7) ^ (row & 7)));
+    }
+    if (B_KC) {
+      const int row = 8 * c + (lane >> 3);
+      const int rr = n0 + row < p.N ? row : p.N - 1 - n0;
+      bo[h] = 8u * (uint32_t)((size_t)rr * p.ldb + 2 * ((lane & 7) ^ (row & 7)));
+    } else {
+      const int kr = 2 * c + (lane >> 5);
+      const int e = 2 * ((lane & 31) ^ (8 * (c & 3)));  // (kr >> 1) == c
+      const int ge = n0 + e + 1 < p.N ? e : p.N - 2 - n0;
+      bo[h] = 8u * (uint32_t)((size_t)kr * p.ldb + ge);
+    }
+  }
+  const long a_step = 8 * (A_KC ? BK : (long)BK * p.lda);
+  const long b_step = 8 * (B_KC ? BK : (long)BK * p.ldb);
+
+  v4d acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
+
+  // tiles of this workgroup: [the masked remainder of K (slice 0 only)] + the whole steps of its slice
+  const int nk_all = p.K / BK;
+  const int kt0 = split * p.steps_per_split;
+  const int nk_dma = (p.split_k > 1) ? ((nk_all - kt0 < p.steps_per_split) ? nk_all - kt0 : p.steps_per_split)
+                                     : nk_all;
+  const bool k_tail = (p.K % BK) != 0 && split == 0;
+  const int first_dma = k_tail ? 1 : 0;
+  const int nk = nk_dma + first_dma;
+  a_ptr += (long)kt0 * a_step;
+  b_ptr += (long)kt0 * b_step;
+  auto issue = [&](int stage) {
+#pragma unroll
+    for (int h = 0; h < CH; ++h) {
+      asm volatile("" : "+v"(ao[h]), "+v"(bo[h]));
+      dma16(reinterpret_cast<const double*>(a_ptr + ao[h]), lds_a + stage * kT64Stage + lchunk[h]);
+      dma16(reinterpret_cast<const double*>(b_ptr + bo[h]), lds_b + stage * kT64Stage + lchunk[h]);
+    }
+    a_ptr += a_step;
+    b_ptr += b_step;
+  };
+  if (k_tail) {
+    v2d ra[2], rb[2];
+    load_tile<BM, A_KC, true, true, 256>(ra, p.A, p.lda, m0, p.M, nk_all * BK, p.K, tid);
+    load_tile<BN, B_KC, true, true, 256>(rb, p.B, p.ldb, n0, p.N, nk_all * BK, p.K, tid);
+    store_tile_dma64<A_KC>(lds_a, ra, tid);
+    store_tile_dma64<B_KC>(lds_b, rb, tid);
+  }
+  // prologue: tiles 0 .. kT64Dist-1 on their way (the remainder tile, if any, is tile 0 and already there)
+#pragma unroll
+  for (int t = 0; t < kT64Dist; ++t)
+    if (t >= first_dma && t < nk) issue(t % kT64Stages);
+
+  const uint32_t a_base = (uint32_t)(uintptr_t)lds_a, b_base = (uint32_t)(uintptr_t)lds_b;
+  const int a_e = wm * 32 + lr, b_e = wn * 32 + lr;  // fragment 0; fragment 1 is 16 further
+
+  for (int kt = 0; kt < nk; ++kt) {
+    // tile kt has landed once at most the younger tiles in flight remain outstanding (4 loads each)
+    const int younger = nk - 1 - kt < kT64Dist - 1 ? nk - 1 - kt : kT64Dist - 1;
+    wait_vmcnt(4 * younger);
+    __syncthreads();  // everybody's share of tile kt is in LDS; everybody is done with tile kt-1
+    if (kt + kT64Dist < nk) issue((kt + kT64Dist) % kT64Stages);
+    const int stage = kt % kT64Stages;
+    const uint32_t sa = a_base + (uint32_t)stage * (kT64Stage * 8), sb = b_base + (uint32_t)stage * (kT64Stage * 8);
+    v2d fa[2][TM], fb[2][TN];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      const int pr = 4 * s2 + lk;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) fa[s2][i] = read_pair64<A_KC>(sa, a_e + 16 * i, pr);
+#pragma unroll
+      for (int j = 0; j < TN; ++j) fb[s2][j] = read_pair64<B_KC>(sb, b_e + 16 * j, pr);
+    }
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[s2][i].x, fb[s2][j].x, acc[i][j], 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[s2][i].y, fb[s2][j].y, acc[i][j], 0, 0, 0);
+    }
+  }
+  write_block<TM, TN>(p, &acc[0][0], m0 + wm * 32, n0 + wn * 32, lr, lk, split);
+}
+
 // Two independent products in one grid: workgroups [0, first_blocks) work on `first`, the others on
 // `second`.  Used for the input gradient of one layer (256 long tiles at C4's hidden width: on its
 // own one workgroup per CU) together with the weight gradient of the layer above it (many short
@@ -975,6 +1164,30 @@ int launch_dma(hipStream_t stream, GemmParams p, int want_split = 0) {
   return RST_OK;
 }
 
+// 64x64 direct-to-LDS tiles, optionally on `slices` K slices (the caller has checked the workspace)
+template <bool B_KC>
+int launch_dma64(hipStream_t stream, GemmParams p, int slices) {
+  p.tiles_m = (p.M + kT64 - 1) / kT64;
+  p.tiles_n = (p.N + kT64 - 1) / kT64;
+  const int nk = p.K / BK;
+  p.split_k = 1;
+  p.steps_per_split = nk;
+  long long blocks = (long long)p.tiles_m * p.tiles_n;
+  if (slices > 1) {
+    p.steps_per_split = (nk + slices - 1) / slices;
+    p.split_k = (nk + p.steps_per_split - 1) / p.steps_per_split;
+    if (p.split_k > 1) {
+      p.ws_colsum = p.ws + (size_t)p.split_k * p.M * p.N;
+      blocks *= p.split_k;
+    }
+  }
+  if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
+  hipLaunchKernelGGL((gemm_f64_mfma_dma64<B_KC>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
+  RST_HIP(hipGetLastError());
+  if (p.split_k > 1) RST_TRY(launch_split_reduce(stream, p));
+  return RST_OK;
+}
+
 // Few output tiles (`blocks` < split_below) but a long contraction: the number of K slices that
 // fills the chip (want_blocks workgroups, about eight per CU), 1 = none.
 long long small_tile_slices(const GemmParams& p, long long blocks, long long split_below, long long want_blocks) {
@@ -1030,9 +1243,21 @@ int launch_one(hipStream_t stream, GemmParams p, long long split_below = 256, lo
 // Which kernel a product goes to.  128x128 tiles once they fill the 256 compute units, 64x64 while
 // that still leaves about four workgroups per CU to overlap each other's load latency, else 32x32
 // (which cuts the contraction into slices when even that gives too few workgroups).
-enum class Route { kDma, kDmaSliced, kTile128, kTile64, kTile32 };
+enum class Route { kDma, kDmaSliced, kDma64, kTile128, kTile64, kTile32 };
 
-Route choose_route(const GemmParams& p, bool vec, int* dma_slices) {
+// RSTORCH_DMA64: "0" never routes to the 64x64 direct-to-LDS kernel, "1" routes every eligible
+// product there (for measurements); unset: the measured rule in choose_route.
+int dma64_mode() {
+  static const int mode = [] {
+    const char* v = std::getenv("RSTORCH_DMA64");
+    if (v && v[0] == '0') return 0;
+    if (v && v[0] == '1') return 1;
+    return -1;
+  }();
+  return mode;
+}
+
+Route choose_route(const GemmParams& p, bool vec, int* dma_slices, bool is_a_kc = false, bool is_b_kc = false) {
   auto tiles = [&](int bm, int bn) {
     return (long long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
   };
@@ -1045,13 +1270,16 @@ Route choose_route(const GemmParams& p, bool vec, int* dma_slices) {
   // slices (about two workgroups per CU, at least 32 K steps each) plus the ordered reduction
   // beats the smaller register-staged tiles by far (128 tiles, K = 4096: 87 % of the MFMA peak
   // against 62 %), as long as the slices still fill the chip.
+  int s128 = 0;       // its slices, 0 = not taken
+  bool multi_round = false;
   if (dma_ok && p.ws != nullptr) {
     const int nk = p.K / BK;
     auto fits = [&](int s) { return p.ws_capacity >= (size_t)s * ((size_t)p.M * p.N + (size_t)p.M); };
     int s = (int)((512 + t128 - 1) / t128);
     if (s > 8) s = 8;
     while (s > 1 && (nk / s < 32 || !fits(s))) --s;
-    if (!(s > 1 && t128 * s >= 256)) {
+    multi_round = s > 1 && t128 * s >= 256;
+    if (!multi_round) {
       // a shorter contraction: one round of workgroups (at most one per CU, at least three CUs in
       // four busy) on slices of 12 K steps or more still beats the register-staged small tiles
       // (8192 x 100 x 784 on 64 tiles: 39 us on four slices against 47 us); a round and a bit
@@ -1060,10 +1288,41 @@ Route choose_route(const GemmParams& p, bool vec, int* dma_slices) {
       if (s > 8) s = 8;
       if (!(s > 1 && t128 * s >= 192 && nk / s >= 12 && fits(s))) s = 1;
     }
-    if (s > 1) {
-      *dma_slices = s;
-      return Route::kDmaSliced;
+    s128 = s > 1 ? s : 0;
+  }
+  // 64x64 direct-to-LDS tiles (forward and input-gradient layouts): one workgroup per CU or more on
+  // slices that are long enough.  Measured over 260 shapes against what it replaces: 11 % faster in
+  // the geometric mean where the 128x128 kernel would run a single round of K slices or the product
+  // would fall to the register-staged 32x32 tiles (contractions of up to 1024), up to 40 % where a dimension of 64 or less made
+  // the 128-wide tiles half empty; against the 128x128 kernel on several rounds of long K slices it
+  // loses, and so it does on the weight-gradient layout (both operands output-contiguous).
+  if (dma_ok && dma64_mode() != 0 && is_a_kc) {
+    const long long t64 = tiles(64, 64);
+    const int nk = p.K / BK;
+    long long s = t64 >= 256 ? 1 : (256 + t64 - 1) / t64;
+    if (s > 32) s = 32;
+    while (s > 1 && nk / s < 8) --s;
+    const bool fits = s == 1 || (p.ws != nullptr && p.ws_capacity >= (size_t)s * ((size_t)p.M * p.N + (size_t)p.M));
+    const long long steps = nk / s;
+    const double flops = 2.0 * p.M * p.N * (double)p.K;
+    const double area128 = (double)t128 * 128.0 * 128.0, area64 = (double)t64 * 64.0 * 64.0;
+    bool take = dma64_mode() == 1 && t64 * s >= 128 && nk >= 1;
+    if (dma64_mode() != 1 && t64 * s >= 192 && flops >= 2.5e8) {
+      const bool half_empty = area128 >= 1.4 * area64 && steps >= 12;
+      // (an input gradient that would otherwise run as 32x32 tiles shares a grid with its layer's
+      // weight gradient in Linear::backward, which is worth more than the faster kernel: stay there)
+      const bool was_small_tiles = s128 <= 1;
+      const bool beats_one_round = !multi_round && nk <= 64 && (s == 1 ? steps >= 12 : steps >= 24) && (is_b_kc || !was_small_tiles);
+      take = half_empty || beats_one_round;
     }
+    if (take && fits) {
+      *dma_slices = (int)s;
+      return Route::kDma64;
+    }
+  }
+  if (s128 > 1) {
+    *dma_slices = s128;
+    return Route::kDmaSliced;
   }
   return tiles(64, 64) >= 1024 ? Route::kTile64 : Route::kTile32;
 }
@@ -1071,9 +1330,12 @@ Route choose_route(const GemmParams& p, bool vec, int* dma_slices) {
 template <bool A_KC, bool B_KC, bool VEC>
 int launch_layout(hipStream_t stream, const GemmParams& p) {
   int slices = 0;
-  switch (choose_route(p, VEC, &slices)) {
+  switch (choose_route(p, VEC, &slices, A_KC, B_KC)) {
     case Route::kDma: return launch_dma<A_KC, B_KC>(stream, p);
     case Route::kDmaSliced: return launch_dma<A_KC, B_KC>(stream, p, slices);
+    case Route::kDma64:
+      if constexpr (A_KC) return launch_dma64<B_KC>(stream, p, slices);
+      else return fail(RST_ERR_UNSUPPORTED, "no 64x64 direct-to-LDS kernel for this layout");
     case Route::kTile128: return launch_one<128, 128, 2, 4, A_KC, B_KC, VEC>(stream, p);
     case Route::kTile64: return launch_one<64, 64, 2, 2, A_KC, B_KC, VEC>(stream, p);
     default: return launch_one<32, 32, 2, 2, A_KC, B_KC, VEC>(stream, p, kSmallTileSplitBelow);
@@ -1152,7 +1414,7 @@ bool can_group_gemm(const GemmDesc& d) {
   if (d.M <= 0 || d.N <= 0 || !desc_vec_ok(d)) return false;
   const GemmParams p = make_params(d);
   int slices = 0;
-  return choose_route(p, true, &slices) == Route::kTile32;
+  return choose_route(p, true, &slices, d.a_kc, d.b_kc) == Route::kTile32;
 }
 
 size_t gemm_group_workspace(const GemmDesc& d) {

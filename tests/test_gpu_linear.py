@@ -35,6 +35,10 @@ SHAPES = [
     (512, 2048, 4096), (498, 2048, 4094), (2048, 1024, 1000),
     # the same with a K remainder (a masked extra tile in slice 0), and K below one whole step
     (512, 2056, 4096), (2048, 1000, 4096), (2048, 10, 2048),
+    # fewer than 256 tiles of 128x128 and a contraction of up to 1024: the 64x64 direct-to-LDS kernel -
+    # forward unsplit with a K remainder, forward on two K slices, input gradient of a narrow layer
+    # (128-wide tiles would be half empty) on four K slices, ragged edges
+    (2048, 1000, 512), (1024, 1024, 512), (4096, 64, 2048), (2050, 1022, 510), (16384, 512, 64),
     # small outputs with a long contraction: the split-K path (with and without a K tail)
     (8192, 784, 100), (8192, 100, 10), (32, 4099, 24), (4100, 7, 9), (16384, 33, 65),
 ]
