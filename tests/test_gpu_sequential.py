@@ -164,3 +164,59 @@ def test_layer_list_mutation_between_steps(engine, oracle):
     np.testing.assert_allclose(m.forward(x).to_numpy(), np.maximum((x @ w1.T) @ w2.T, 0), rtol=1e-13, atol=1e-13)
     g = m.backward(np.ones((5, 3)))
     assert g.shape == (5, 4)
+
+
+def _random_specs():
+    """Seeded random layer lists: Identity / ReLU anywhere (leading, doubled, trailing before the
+    loss), Linear -> Linear without an activation, odd and even widths, batches from 1 up."""
+    rng = np.random.default_rng(20261125)
+    out = []
+    for case in range(24):
+        n_linear = int(rng.integers(1, 5))
+        widths = [int(rng.choice([1, 2, 3, 7, 10, 16, 31, 33, 64, 100, 129, 200])) for _ in range(n_linear + 1)]
+        spec = []
+        for i in range(n_linear):
+            for _ in range(int(rng.integers(0, 3))):
+                spec.append(("identity",) if rng.random() < 0.5 else ("relu",))
+            spec.append(("linear", widths[i], widths[i + 1]))
+        for _ in range(int(rng.integers(0, 2))):
+            spec.append(("relu",) if rng.random() < 0.5 else ("identity",))
+        batch = int(rng.choice([1, 2, 5, 32, 67, 128, 300]))
+        out.append(("case%02d_b%d" % (case, batch), spec, batch))
+    return out
+
+
+@pytest.mark.parametrize("name,spec,batch", _random_specs(), ids=[c[0] for c in _random_specs()])
+def test_random_layer_lists_match_oracle(engine, oracle, name, spec, batch):
+    """Layer by layer through the module interface AND as the one-call device step, against the
+    oracle: logits, loss, input gradient, every dW/db and the updated parameters (1e-10), then a
+    second step."""
+    import rstorch_amd as rs
+    weights = make_weights(oracle, spec, 77)
+    model, ref = build_pair(rs, oracle, spec, weights)
+    dm = rs.DeviceModel(spec)
+    dm.load_parameters(weights)
+    n_in = next(l[1] for l in spec if l[0] == "linear")
+    n_out = [l[2] for l in spec if l[0] == "linear"][-1]
+    loss, optim = rs.CrossEntropyLoss.new(), rs.SGD.new(0.05)
+    for step in range(2):
+        x, y = batch_data(oracle, batch, n_in, n_out, 41, step, True)
+        pred = model.forward(x)
+        want_logits = ref.forward(x)
+        assert rel_err(pred.to_numpy(), want_logits) <= TOL
+        got = loss.forward(pred, y)
+        want, prob = oracle.cross_entropy_forward(want_logits, y)
+        assert abs(got - want) <= TOL * max(abs(want), 1e-300)
+        gin = model.backward(loss.backward())
+        want_gin = ref.backward(oracle.cross_entropy_backward(prob, y))
+        assert rel_err(gin.to_numpy(), want_gin) <= TOL
+        for p, (_, rg) in zip(model.parameters(), ref.parameters()):
+            assert p.grad.shape == rg.shape and rel_err(p.grad.to_numpy(), rg) <= TOL
+        optim.step(model)
+        ref.sgd_step(0.05)
+        fused = dm.train_step(x, y, 0.05)
+        assert abs(fused - want) <= TOL * max(abs(want), 1e-300)
+        for p, (q, _), (rp, _) in zip(model.parameters(), dm.parameters(), ref.parameters()):
+            assert rel_err(p.parm.to_numpy(), rp) <= TOL
+            assert rel_err(q.to_numpy(), rp) <= TOL
+    dm.close()
