@@ -820,6 +820,18 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
   dma_tile<A_KC, B_KC, WGM, WGN, STAGES, DIST>(p, (int)blockIdx.x, lds_a, lds_b);
 }
 
+// Up to kMaxGroup weight gradients with few output tiles each but a long contraction (the batch)
+// in one grid of 128x128 direct-to-LDS tiles: every problem is cut into K slices so that together
+// they give about one workgroup per CU; workgroups [first_block[i], first_block[i+1]) belong to
+// problem i and the shared reduction grid adds the slices up in order.
+__global__ __launch_bounds__(512, 4) void gemm_f64_mfma_dma_group(const GemmGroup g) {
+  __shared__ __attribute__((aligned(1024))) double lds_a[2 * kDmaStage];
+  __shared__ __attribute__((aligned(1024))) double lds_b[2 * kDmaStage];
+  int i = 0;
+  while (i + 1 < g.count && (int)blockIdx.x >= g.first_block[i + 1]) ++i;
+  dma_tile<false, false, 2, 4, 2, 1>(g.p[i], (int)blockIdx.x - g.first_block[i], lds_a, lds_b);
+}
+
 // ---- 64x64 tiles fed by direct global -> LDS loads ---------------------------------------------
 // The mid-size path: products whose 128x128 tiling gives the chip too few workgroups (an 8192 x 100
 // output is 64 tiles of 128x128 but 256 of 64x64; a 100 x 784 weight gradient is 7 against 26).
@@ -1417,23 +1429,122 @@ bool can_group_gemm(const GemmDesc& d) {
   return choose_route(p, true, &slices, d.a_kc, d.b_kc) == Route::kTile32;
 }
 
+namespace {
+// RSTORCH_DMA_GROUP: "0" keeps every group on the 32x32 kernels, "1" sends every eligible group
+// to the sliced 128x128 kernel (for measurements); unset: the rule in plan_dma_group.
+int dma_group_mode() {
+  static const int mode = [] {
+    const char* v = std::getenv("RSTORCH_DMA_GROUP");
+    if (v && v[0] == '0') return 0;
+    if (v && v[0] == '1') return 1;
+    return -1;
+  }();
+  return mode;
+}
+
+constexpr int kDmaGroupMaxSlices = 32;
+constexpr int kDmaGroupMinSteps = 8;
+
+// a weight gradient that the sliced 128x128 group kernel can take at all: at most eight output
+// tiles (more have enough workgroups of their own, and the slices of a larger output would crowd
+// the shared workspace)
+bool dma_group_member(const GemmDesc& d) {
+  return !d.a_kc && !d.b_kc && desc_vec_ok(d) && d.K / BK >= 2 * kDmaGroupMinSteps && d.M >= 2 && d.N >= 2 &&
+         (long long)((d.M + 127) / 128) * ((d.N + 127) / 128) <= 8 && d.lda < (1L << 22) && d.ldb < (1L << 22) &&
+         d.workspace != nullptr;
+}
+
+// Plans d[0..count) as one grid of sliced 128x128 tiles: every member gets the same number of
+// slices, the one that brings the grid to about one workgroup per CU (two per CU measured 4 % slower
+// on the step), shortened where a member's contraction would leave a slice fewer than
+// kDmaGroupMinSteps K steps.  False when the members do not qualify, the tiles would be mostly
+// padding, the grid would leave more than a quarter of the chip idle (batches below about 4096 for
+// a handful of tiles), or the workspace is too small.
+bool plan_dma_group(const GemmDesc* d, int count, GemmGroup* g, long long* blocks_out, long long* reduce_out) {
+  if (dma_group_mode() == 0) return false;
+  long long tiles = 0;
+  double outputs = 0.0;
+  for (int i = 0; i < count; ++i) {
+    if (!dma_group_member(d[i])) return false;
+    tiles += (long long)((d[i].M + 127) / 128) * ((d[i].N + 127) / 128);
+    outputs += (double)d[i].M * d[i].N;
+  }
+  const int cus = compute_units();
+  if (tiles > cus / 8) return false;
+  // Measured on whole training steps of small networks at batch 8192: with 61 % of the 128x128
+  // tiles' area in use (784-100-100-10) the step is 6 % shorter than on the 32x32 group (13 % at
+  // batch 32768), with 90 % (256-256-256-10) 7 %; with 41 % (1024-64-64-64-16) it is 9 % longer.
+  if (dma_group_mode() != 1 && outputs < 0.55 * 16384.0 * (double)tiles) return false;
+  long long want = cus / tiles;
+  if (want > kDmaGroupMaxSlices) want = kDmaGroupMaxSlices;
+  long long blocks = 0, reduce_blocks = 0;
+  size_t ws_used = 0;
+  g->count = count;
+  for (int i = 0; i < count; ++i) {
+    GemmParams p = make_params(d[i]);
+    p.tiles_m = (p.M + 127) / 128;
+    p.tiles_n = (p.N + 127) / 128;
+    const int nk = p.K / BK;
+    long long s = want;
+    if (s > nk / kDmaGroupMinSteps) s = nk / kDmaGroupMinSteps;
+    if (s < 2) return false;
+    p.steps_per_split = (int)((nk + s - 1) / s);
+    p.split_k = (nk + p.steps_per_split - 1) / p.steps_per_split;
+    if (p.split_k < 2) return false;
+    const size_t need = (size_t)p.split_k * ((size_t)p.M * p.N + (size_t)p.M);
+    if (ws_used + need > p.ws_capacity) return false;
+    p.ws += ws_used;
+    p.ws_colsum = p.ws + (size_t)p.split_k * p.M * p.N;
+    ws_used += need;
+    g->first_block[i] = (int)blocks;
+    g->first_reduce_block[i] = (int)reduce_blocks;
+    g->layout[i] = 0;
+    blocks += (long long)p.tiles_m * p.tiles_n * p.split_k;
+    reduce_blocks += (long long)(((size_t)p.M * p.N + 255) / 256);
+    g->p[i] = p;
+  }
+  g->first_block[count] = (int)blocks;
+  g->first_reduce_block[count] = (int)reduce_blocks;
+  if (dma_group_mode() != 1 && blocks < (3 * cus) / 4) return false;
+  *blocks_out = blocks;
+  *reduce_out = reduce_blocks;
+  return true;
+}
+}  // namespace
+
 size_t gemm_group_workspace(const GemmDesc& d) {
   GemmParams p = make_params(d);
   plan_group_member(p);
-  return p.split_k > 1 ? (size_t)p.split_k * ((size_t)p.M * p.N + (size_t)p.M) : 0;
+  size_t need = p.split_k > 1 ? (size_t)p.split_k * ((size_t)p.M * p.N + (size_t)p.M) : 0;
+  // the sliced 128x128 grid, should the whole group qualify for it, takes up to kDmaGroupMaxSlices slices
+  if (dma_group_mode() != 0 && dma_group_member(d)) {
+    const size_t dma_need = (size_t)kDmaGroupMaxSlices * ((size_t)p.M * p.N + (size_t)p.M);
+    if (dma_need > need) need = dma_need;
+  }
+  return need;
 }
 
 int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count) {
   if (count < 1 || count > kMaxGroup) return fail(RST_ERR_INVALID_ARGUMENT, "a group holds 1..%d contractions", kMaxGroup);
   GemmGroup g{};
-  g.count = count;
   long long blocks = 0, reduce_blocks = 0;
+  for (int i = 0; i < count; ++i)
+    if (d[i].workspace != d[0].workspace || d[i].workspace_count != d[0].workspace_count)
+      return fail(RST_ERR_INVALID_ARGUMENT, "the contractions of a group share one workspace");
+  if (plan_dma_group(d, count, &g, &blocks, &reduce_blocks)) {
+    hipLaunchKernelGGL(gemm_f64_mfma_dma_group, dim3((unsigned)blocks), dim3(512), 0, stream, g);
+    RST_HIP(hipGetLastError());
+    hipLaunchKernelGGL(split_reduce_group_kernel, dim3((unsigned)reduce_blocks), dim3(256), 0, stream, g);
+    RST_HIP(hipGetLastError());
+    return RST_OK;
+  }
+  g = GemmGroup{};
+  g.count = count;
+  blocks = reduce_blocks = 0;
   size_t ws_used = 0;
   bool mixed = false;  // anything but weight-gradient layouts
   for (int i = 0; i < count; ++i) {
     if (!can_group_gemm(d[i])) return fail(RST_ERR_INVALID_ARGUMENT, "contraction %d cannot join a group", i);
-    if (d[i].workspace != d[0].workspace || d[i].workspace_count != d[0].workspace_count)
-      return fail(RST_ERR_INVALID_ARGUMENT, "the contractions of a group share one workspace");
     GemmParams p = make_params(d[i]);
     plan_group_member(p);
     g.first_block[i] = (int)blocks;

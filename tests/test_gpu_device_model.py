@@ -164,37 +164,55 @@ def test_profile_records_cover_every_launch(engine, oracle):
 
 
 GROUP_CASES = [
-    ("readme_b32", README_MLP, 32),
-    # long batch: every weight gradient is cut into K slices, which share the reduction grid too
-    ("readme_b8192", README_MLP, 8192),
-    ("readme_b500", README_MLP, 500),
+    ("readme_b32", README_MLP, 32, True),
+    # Long batches: the weight gradients are cut into K slices, which share the reduction grid too.
+    # From a batch of about 4096 the shared grid runs 128x128 tiles on slices of its own choice, so
+    # the sums are taken in another order than in the per-layer launches: equal within rounding.
+    ("readme_b8192", README_MLP, 8192, False),
+    ("readme_b8200", README_MLP, 8200, False),  # batch not a multiple of the K step
+    ("three_256_wide_b4096", [("linear", 256, 256), ("relu",), ("linear", 256, 256), ("relu",),
+                              ("linear", 256, 10)], 4096, False),
+    ("readme_b2048", README_MLP, 2048, True),
+    ("readme_b500", README_MLP, 500, True),
     # more small layers than one shared grid holds (eight): two grids
     ("twelve_small_layers", [("linear", 20, 34), ("relu",)] + [("linear", 34, 34), ("relu",)] * 10 +
-     [("linear", 34, 6)], 16),
+     [("linear", 34, 6)], 16, True),
     # a layer large enough for the 128x128 kernels between small ones, and an odd width that
     # rules out 16-byte loads
     ("mixed", [("linear", 64, 2048), ("relu",), ("linear", 2048, 2048), ("relu",), ("linear", 2048, 33),
-               ("relu",), ("linear", 33, 10)], 64),
+               ("relu",), ("linear", 33, 10)], 64, True),
 ]
 
 
-@pytest.mark.parametrize("name,spec,batch", GROUP_CASES, ids=[c[0] for c in GROUP_CASES])
+@pytest.mark.parametrize("name,spec,batch,exact", GROUP_CASES, ids=[c[0] for c in GROUP_CASES])
 @pytest.mark.parametrize("fused", [True, False])
-def test_shared_grid_of_small_weight_gradients_is_bit_identical(engine, oracle, name, spec, batch, fused):
+def test_shared_grid_of_small_weight_gradients_equals_per_layer_launches(engine, oracle, name, spec, batch, exact, fused):
     """Small weight gradients share one grid at the end of backward; with profiling on every layer
-    launches on its own.  Losses, parameters and gradients must agree bit for bit."""
+    launches on its own.  Losses, parameters and gradients must agree: bit for bit where both paths
+    slice the batch alike, to 1e-13 of the tensor's largest entry where the shared grid slices it
+    differently (the first step's loss is bit-equal either way: it only depends on the forward pass)."""
     import rstorch_amd as rs
     models = [pair(rs, oracle, spec, 77)[0] for _ in range(2)]
     models[1].profile_enable(True)
     for dm in models:
         dm.fuse_sgd(fused)
+
+    def same(a, b, what):
+        if exact:
+            assert np.array_equal(a, b), what
+        else:
+            assert np.max(np.abs(a - b)) <= 1e-13 * np.max(np.abs(b)), what
+
     for step in range(3):
         x, y = batch_data(oracle, batch, models[0].in_width, models[0].out_width, 5, step, True)
         losses = [dm.train_step(x, y, 0.05) for dm in models]
-        assert losses[0] == losses[1], "step %d" % step
+        if exact or step == 0:
+            assert losses[0] == losses[1], "step %d" % step
+        else:
+            assert abs(losses[0] - losses[1]) <= 1e-13 * abs(losses[1]), "step %d" % step
         for (p, g), (q, h) in zip(models[0].parameters(), models[1].parameters()):
-            assert np.array_equal(p.to_numpy(), q.to_numpy()), "step %d" % step
-            assert np.array_equal(g.to_numpy(), h.to_numpy()), "step %d" % step
+            same(p.to_numpy(), q.to_numpy(), "step %d" % step)
+            same(g.to_numpy(), h.to_numpy(), "step %d" % step)
     kinds = [r["kernel"] for r in models[1].profile_read()]
     assert kinds.count("grad_weight") == 3 * sum(1 for l in spec if l[0] == "linear")
     models[1].profile_enable(False)
