@@ -19,6 +19,7 @@
 //
 // MFMA register layout (64 lanes): A fragment lane l holds A[l%16][l/16], B fragment lane l
 // holds B[l/16][l%16], and accumulator register r of lane l holds D[4*r + l/16][l%16].
+#include <cmath>
 #include <cstdlib>
 
 #include "common.h"
@@ -40,6 +41,7 @@ struct GemmParams {
   int epilogue;
   const double* bias;
   double divisor;
+  double divisor_reciprocal;  // exact 1 / divisor when divisor is a power of two, else 0
   const double* mask;
   long ldmask;
   double* colsum;        // weight-gradient launches only: colsum[i] = (sum_k A(i,k)) / colsum_div
@@ -238,13 +240,101 @@ __device__ __forceinline__ void store_block(const GemmParams& p, const v4d* acc,
   }
 }
 
+// The same epilogue for a block that lies wholly inside the matrix, which is nearly every block of
+// a large product.  While a workgroup is in its epilogue the other workgroup of the CU keeps the
+// matrix pipeline full, and FP64 MFMAs hold the vector ALU for all of their 64 cycles: a vector
+// instruction of the epilogue gets in only between two of them.  Measured on the 4096 x 4096 weight
+// gradient: the general epilogue above (a bounds test, a branch and 64-bit address arithmetic per
+// element, and for the weight gradient a division: some 10 to 25 vector instructions per stored
+// value) takes 27 us next to a running K loop, 47 us with the SGD update, against 2.8 us on a CU of
+// its own; the last epilogue of every CU is exposed at the end of the launch.  Here an access is a
+// wave-uniform row pointer kept in scalar registers (scalar adds from row to row), one 32-bit lane
+// offset and an immediate column offset: no vector instruction per address, no predicates, and the
+// division by a power of two (the usual batch size) is a multiplication by its exact reciprocal -
+// the same bits for every operand, gradual underflow included.
+template <int TM, int TN, int EPI, bool SGD, bool RECIP>
+__device__ __forceinline__ void store_block_interior(const GemmParams& p, const v4d* acc, double* out,
+                                                     long ld_out, int row0, int col0, int lr, int lk) {
+  constexpr bool BIAS = EPI == EPI_BIAS || EPI == EPI_BIAS_RELU;
+  uint32_t off_c = 8u * (uint32_t)(lk * ld_out + lr);
+  uint32_t off_m = EPI == EPI_MASK ? 8u * (uint32_t)(lk * p.ldmask + lr) : 0u;
+  char* c_row = reinterpret_cast<char*>(out + (size_t)row0 * ld_out + col0);
+  char* w_row = SGD ? reinterpret_cast<char*>(p.sgd_parm + (size_t)row0 * ld_out + col0) : nullptr;
+  const char* m_row = EPI == EPI_MASK ? reinterpret_cast<const char*>(p.mask + (size_t)row0 * p.ldmask + col0) : nullptr;
+  const long c_step = 32 * ld_out;      // bytes from accumulator register r to r + 1: four rows
+  const long m_step = 32 * p.ldmask;
+  double bias[TN];
+  if (BIAS) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) bias[j] = p.bias[col0 + j * 16 + lr];
+  }
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    double extra[TN][4];
+    if (EPI == EPI_MASK || SGD) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const char* src = EPI == EPI_MASK ? m_row + r * m_step : w_row + r * c_step;  // scalar
+        // hiding the offset from the optimiser before every use keeps "scalar base + 32-bit lane
+        // offset + immediate" one addressing mode instead of a 64-bit vector addition per row
+        asm volatile("" : "+v"(off_c), "+v"(off_m));
+        const uint32_t off = EPI == EPI_MASK ? off_m : off_c;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) extra[j][r] = *reinterpret_cast<const double*>(src + off + 128 * j);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      char* dst_row = c_row + r * c_step;
+      char* parm_row = SGD ? w_row + r * c_step : nullptr;
+      asm volatile("" : "+v"(off_c));
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        double v = acc[i * TN + j][r];
+        // (opaque, so that the arithmetic that two epilogue kinds have in common is not hoisted out
+        // of the switch for all 32 values at once, which spills)
+        if (EPI == EPI_DIVIDE || BIAS) asm volatile("" : "+v"(v));
+        if (EPI == EPI_BIAS) v = v + bias[j];
+        if (EPI == EPI_BIAS_RELU) v = fmax(v + bias[j], 0.0);
+        if (EPI == EPI_RELU) v = fmax(v, 0.0);
+        if (EPI == EPI_DIVIDE) v = RECIP ? v * p.divisor_reciprocal : v / p.divisor;
+        if (EPI == EPI_MASK) v = v * (extra[j][r] > 0.0 ? 1.0 : 0.0);
+        double* dst = reinterpret_cast<double*>(dst_row + off_c + 128 * j);
+        if (EPI == EPI_DIVIDE) __builtin_nontemporal_store(v, dst);
+        else *dst = v;
+        if (SGD) *reinterpret_cast<double*>(parm_row + off_c + 128 * j) = sgd_apply(extra[j][r], v, p.sgd_lr);
+      }
+    }
+    // One fragment row at a time: hoisting the arithmetic of later rows would double the live
+    // registers.  Requesting the parameters of the next row before this one is stored was measured
+    // too: the epilogue itself drops from 33 to 10 us, but the launch gets 4 % longer - every CU
+    // reaches its epilogues at about the same time, and the shorter they are, the harder their
+    // burst of loads and stores hits the tile loads of the workgroups that are still multiplying.
+    // (Stretching the epilogue with sleeps between the rows, to 41 and 50 us, costs 2 % and 5 %.)
+    __builtin_amdgcn_sched_barrier(0);
+    c_row += 4 * c_step;
+    if (SGD) w_row += 4 * c_step;
+    if (EPI == EPI_MASK) m_row += 4 * m_step;
+  }
+}
+
 // Writes the block either as raw partial products of K slice `split` (the reduction applies the
 // epilogue later) or finished, with the epilogue the launch asks for.
 template <int TM, int TN>
 __device__ __forceinline__ void write_block(const GemmParams& p, const v4d* acc, int row0, int col0,
                                             int lr, int lk, int split) {
+  // the block origin is the same for the whole wavefront: keep it in scalar registers
+  row0 = __builtin_amdgcn_readfirstlane(row0);
+  col0 = __builtin_amdgcn_readfirstlane(col0);
+  // (leading dimensions below 2^26 doubles keep the 32-bit lane offsets in range)
+  const bool interior = row0 + 16 * TM <= p.M && col0 + 16 * TN <= p.N && p.ldc < (1L << 26) &&
+                        (long)p.N < (1L << 26) && p.ldmask < (1L << 26);
   if (p.split_k > 1) {
     double* __restrict__ out = p.ws + (size_t)split * p.M * p.N;
+    if (interior) {
+      store_block_interior<TM, TN, EPI_NONE, false, false>(p, acc, out, p.N, row0, col0, lr, lk);
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -256,6 +346,22 @@ __device__ __forceinline__ void write_block(const GemmParams& p, const v4d* acc,
           if (row < p.M && col < p.N) out[(size_t)row * p.N + col] = acc[i * TN + j][r];
         }
       }
+    return;
+  }
+  // (a true division keeps to the general path: its temporaries on top of a batch of parameter
+  // loads do not fit the registers that the accumulators leave)
+  if (interior && (p.epilogue != EPI_DIVIDE || p.divisor_reciprocal != 0.0)) {
+    switch (p.epilogue) {
+      case EPI_BIAS: store_block_interior<TM, TN, EPI_BIAS, false, false>(p, acc, p.C, p.ldc, row0, col0, lr, lk); break;
+      case EPI_BIAS_RELU: store_block_interior<TM, TN, EPI_BIAS_RELU, false, false>(p, acc, p.C, p.ldc, row0, col0, lr, lk); break;
+      case EPI_RELU: store_block_interior<TM, TN, EPI_RELU, false, false>(p, acc, p.C, p.ldc, row0, col0, lr, lk); break;
+      case EPI_MASK: store_block_interior<TM, TN, EPI_MASK, false, false>(p, acc, p.C, p.ldc, row0, col0, lr, lk); break;
+      case EPI_DIVIDE:
+        if (p.sgd_parm) store_block_interior<TM, TN, EPI_DIVIDE, true, true>(p, acc, p.C, p.ldc, row0, col0, lr, lk);
+        else store_block_interior<TM, TN, EPI_DIVIDE, false, true>(p, acc, p.C, p.ldc, row0, col0, lr, lk);
+        break;
+      default: store_block_interior<TM, TN, EPI_NONE, false, false>(p, acc, p.C, p.ldc, row0, col0, lr, lk); break;
+    }
     return;
   }
   switch (p.epilogue) {
@@ -1374,6 +1480,13 @@ GemmParams make_params(const GemmDesc& d) {
   p.lda = d.lda; p.ldb = d.ldb; p.ldc = d.ldc;
   p.epilogue = d.epilogue;
   p.bias = d.bias; p.divisor = d.divisor; p.mask = d.mask; p.ldmask = d.ldmask;
+  {
+    // a power of two whose reciprocal is a normal number: x * (1 / d) and x / d are then the same
+    // correctly rounded value for every x
+    int exponent = 0;
+    const double mantissa = std::frexp(d.divisor, &exponent);
+    p.divisor_reciprocal = (std::fabs(mantissa) == 0.5 && exponent > -1000 && exponent < 1000) ? 1.0 / d.divisor : 0.0;
+  }
   p.colsum = (!d.a_kc) ? d.colsum : nullptr;
   p.colsum_div = d.colsum_div;
   p.sgd_parm = (d.epilogue == EPI_DIVIDE) ? d.sgd_parm : nullptr;
