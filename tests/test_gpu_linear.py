@@ -162,6 +162,34 @@ def test_one_hot_input_selects_weight_rows(engine):
     np.testing.assert_array_equal(lin.forward(x).to_numpy(), w[:, idx].T + b)
 
 
+# Small integers make every product and every partial sum exact, whatever the order of the
+# additions, so the three results of Linear::backward can be compared with numpy BIT FOR BIT:
+# dW = (G^T X) / batch with the division by the batch size (src/module/linear.rs:63-64; blocks
+# inside the matrix multiply by the exact reciprocal when the batch is a power of two and divide
+# otherwise, blocks on its edge always divide), db = colsum(G) / batch, dX = (G W) * [x > 0].
+# The shapes mix interior and edge blocks of the 128x128, 64x64 and 32x32 kernels.
+@pytest.mark.parametrize("batch,k,n", [(1024, 384, 300), (1000, 384, 300), (4096, 1024, 1280), (4000, 1024, 1280),
+                                       (512, 4096, 4096), (96, 130, 70), (8192, 784, 100), (8200, 784, 100)])
+def test_backward_on_integer_data_is_bit_exact(engine, batch, k, n):
+    from rstorch_amd import _ffi
+    rng = np.random.default_rng(batch + k + n)
+    hx = rng.integers(-3, 4, size=(batch, k)).astype(np.float64)
+    hw = rng.integers(-3, 4, size=(n, k)).astype(np.float64)
+    hg = rng.integers(-3, 4, size=(batch, n)).astype(np.float64)
+    x, w, g = engine.from_numpy(hx), engine.from_numpy(hw), engine.from_numpy(hg)
+    gw, gb, gx = engine.empty(n, k), engine.empty(1, n), engine.empty(batch, k)
+    _ffi.check(engine.lib.rst_linear_backward(engine.handle, g.ptr, x.ptr, w.ptr, gw.ptr, gb.ptr, gx.ptr, x.ptr,
+                                              batch, k, n))
+    np.testing.assert_array_equal(gw.to_numpy(), (hg.T @ hx) / batch)
+    np.testing.assert_array_equal(gb.to_numpy(), hg.sum(axis=0, keepdims=True) / batch)
+    np.testing.assert_array_equal(gx.to_numpy(), (hg @ hw) * (hx > 0))
+    # forward with bias and ReLU on the same data
+    hb = rng.integers(-50, 51, size=(1, n)).astype(np.float64)
+    b, out = engine.from_numpy(hb), engine.empty(batch, n)
+    _ffi.check(engine.lib.rst_linear_forward(engine.handle, x.ptr, w.ptr, b.ptr, out.ptr, batch, k, n, 1))
+    np.testing.assert_array_equal(out.to_numpy(), np.maximum(hx @ hw.T + hb, 0.0))
+
+
 def test_backward_twice_raises(engine):
     import rstorch_amd as rs
     lin = _linear(rs, np.ones((2, 3)), np.zeros((1, 2)))
