@@ -40,11 +40,11 @@ PEAK_HBM_GBPS = 8000.0
 # gradient), the reduction of the two partial results (134.3 MB); the weight gradient carries the SGD
 # update of its layer.
 C4_TRAFFIC_SOURCE = {"profile": "profiles/c4_hbm_traffic.md",
-                     "kernels_as_of_commit": "379da82 (contraction kernels unchanged since)"}
+                     "kernels_as_of_commit": "46a0b86"}
 C4_TRAFFIC_BYTES_PER_LAUNCH = {
-    "linear_forward": (8 * 436.4e6 + 3847.5e6) / 9,
-    "grad_weight": (8 * 859.2e6 + 6972.6e6) / 9,
-    "grad_input": (7 * 470.0e6 + 3357.2e6 + 134.3e6) / 8,
+    "linear_forward": (8 * 436.4e6 + 3861.9e6) / 9,
+    "grad_weight": (8 * 865.7e6 + 8083.6e6) / 9,
+    "grad_input": (7 * 470.0e6 + 3317.7e6 + 134.3e6) / 8,
 }
 
 C4_SPEC = [("linear", 4096, 4096), ("relu",)] * 8 + [("linear", 4096, 32768)]
