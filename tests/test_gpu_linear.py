@@ -221,6 +221,21 @@ def _sweep_cases():
             k = int(rng.integers(1, 60)) * 2
             n = int(rng.integers(1, 60)) * 2
         cases.append((b, k, n))
+    rng = np.random.default_rng(54321)
+    for _ in range(28):
+        kind = int(rng.integers(0, 3))
+        if kind == 0:    # the 64x64 direct-to-LDS band: a long batch, one narrow side, a contraction of a few hundred
+            b = int(rng.integers(16, 130)) * 64 + int(rng.choice([0, 2, 10]))
+            k, n = int(rng.integers(12, 70)) * 16 + int(rng.choice([0, 2, 8])), int(rng.integers(8, 130)) * 2
+            if rng.integers(0, 2):
+                k, n = n + 190, k
+        elif kind == 1:  # whole tiles only: every block takes the interior epilogue; power-of-two and other batches
+            b = int(rng.choice([256, 512, 768, 1024, 1536, 2048]))
+            k, n = int(rng.integers(1, 12)) * 128, int(rng.integers(1, 12)) * 128
+        else:            # one or two tiles of output over a very long batch (weight gradient in many K slices)
+            b = int(rng.integers(40, 140)) * 128 + int(rng.choice([0, 8]))
+            k, n = int(rng.integers(5, 130)) * 2, int(rng.integers(5, 130)) * 2
+        cases.append((b, k, n))
     return cases
 
 
