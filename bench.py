@@ -33,7 +33,7 @@ PEAK_FP64_MFMA_TFLOPS = 78.6
 PEAK_HBM_GBPS = 8000.0
 
 # HBM-side bytes per launch of the C4 contraction kernels, averaged over the launches of one step
-# (8 hidden layers + the head).  Measured with two rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE)
+# (8 hidden layers + the head).  Measured with rocprofv3 --pmc runs (FETCH_SIZE, WRITE_SIZE, with and without --no-pair)
 # of this script, scaled by the same counters on a streaming kernel of known size
 # (--calibration-copy: FETCH x 2.0, WRITE x 1.0); the summary is kept under profiles/.
 # A launch = the contraction plus, for the one that is contracted as two K slices (the head's input
@@ -42,9 +42,12 @@ PEAK_HBM_GBPS = 8000.0
 C4_TRAFFIC_SOURCE = {"profile": "profiles/c4_hbm_traffic.md",
                      "kernels_as_of_commit": "46a0b86"}
 C4_TRAFFIC_BYTES_PER_LAUNCH = {
-    "linear_forward": (8 * 436.4e6 + 3861.9e6) / 9,
-    "grad_weight": (8 * 865.7e6 + 8083.6e6) / 9,
-    "grad_input": (7 * 470.0e6 + 3317.7e6 + 134.3e6) / 8,
+    "linear_forward": (8 * 436.4e6 + 3891.6e6) / 9,
+    "grad_weight": (8 * 866.1e6 + 8700.8e6) / 9,
+    "grad_input": (7 * 470.0e6 + 3370.3e6 + 134.3e6) / 8,
+    # a layer's weight gradient + SGD and the next layer's input gradient in one grid (the default):
+    # six pairs at the hidden width and the one that carries the head's weight gradient
+    "grad_pair": (6 * 1521.3e6 + 8280.1e6) / 7,
 }
 
 C4_SPEC = [("linear", 4096, 4096), ("relu",)] * 8 + [("linear", 4096, 32768)]
@@ -386,6 +389,9 @@ def main():
                     help="run one of the small configurations alone (for profiler runs)")
     ap.add_argument("--sgd-only", action="store_true",
                     help="time only SGD::step over the configs[3] parameter set (for profiler runs)")
+    ap.add_argument("--no-pair", action="store_true",
+                    help="launch every weight gradient and input gradient of C4 on its own (profiles that "
+                         "attribute counters to one product at a time)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one streaming ReLU over 1 GiB (reads 1 GiB, writes 1 GiB): the "
                          "known-size kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE are scaled by")
@@ -430,6 +436,8 @@ def main():
     dm, x, y = make_model(rs, eng, C4_SPEC, C4_BATCH, True)
     if args.eager:
         dm.graph_enable(False)
+    if args.no_pair:
+        dm.pair_gradients(False)
     tensors, params = dm.parameter_count()
     wall, dev_ms, loss, recs = time_steps(eng, dm, x, y, args.steps, args.warmup, True)
     ms_per_step = wall * 1e3 / args.steps
@@ -443,7 +451,9 @@ def main():
     d = kernels[dominant]
     launches = [r for r in recs if r["kernel"] == dominant]
     flops_per_launch = sum(r["flops"] for r in launches) / len(launches)
-    roofline = {"kernel": "gemm_f64_mfma_dma (" + dominant + ")", "bound": "mfma",
+    kernel_names = {"grad_pair": "gemm_f64_mfma_dma_pair (a layer's weight gradient + SGD and the next layer's "
+                                 "input gradient in one grid)"}
+    roofline = {"kernel": kernel_names.get(dominant, "gemm_f64_mfma_dma (" + dominant + ")"), "bound": "mfma",
                 "achieved": d["achieved_tflops"], "peak": PEAK_FP64_MFMA_TFLOPS, "unit": "TFLOP/s",
                 "frac": d["frac"], "traffic": C4_TRAFFIC_BYTES_PER_LAUNCH.get(dominant),
                 "traffic_unit": "bytes per launch (L2 misses + write-backs, rocprofv3 FETCH_SIZE/WRITE_SIZE)",
@@ -469,6 +479,7 @@ def main():
                    "device_ms_per_step_median": per_step[len(per_step) // 2],
                    "device_ms_per_step_min": per_step[0],
                    "final_loss": loss, "per_launch_events": True,
+                   "paired_gradient_launches": not args.no_pair,
                    # the loss is computed on the device every step but the host does not read it inside
                    # the timed loop (one read after the last step); the README-shaped loop, which reads
                    # the loss and the accuracy every step, is reported as readme_loop_b32

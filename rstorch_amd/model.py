@@ -191,7 +191,8 @@ class DeviceModel:
         _ffi.check(self.engine.lib.rst_model_fuse_sgd(self.handle, 1 if on else 0))
 
     def pair_gradients(self, on=True):
-        """Launch a layer's weight gradient in one grid with the next layer's input gradient."""
+        """Launch a layer's weight gradient in one grid with the next layer's input gradient
+        when both are large (default), or one after the other."""
         _ffi.check(self.engine.lib.rst_model_pair_gradients(self.handle, 1 if on else 0))
 
     def graph_enable(self, on=True):
