@@ -40,7 +40,7 @@ PEAK_HBM_GBPS = 8000.0
 # gradient), the reduction of the two partial results (134.3 MB); the weight gradient carries the SGD
 # update of its layer.
 C4_TRAFFIC_SOURCE = {"profile": "profiles/c4_hbm_traffic.md",
-                     "kernels_as_of_commit": "46a0b86"}
+                     "kernels_as_of_commit": "d945909"}
 C4_TRAFFIC_BYTES_PER_LAUNCH = {
     "linear_forward": (8 * 436.4e6 + 3891.6e6) / 9,
     "grad_weight": (8 * 866.1e6 + 8700.8e6) / 9,
