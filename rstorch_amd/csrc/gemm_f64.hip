@@ -1409,11 +1409,18 @@ Route choose_route(const GemmParams& p, bool vec, int* dma_slices, bool is_a_kc 
     s128 = s > 1 ? s : 0;
   }
   // 64x64 direct-to-LDS tiles (forward and input-gradient layouts): one workgroup per CU or more on
-  // slices that are long enough.  Measured over 260 shapes against what it replaces: 11 % faster in
-  // the geometric mean where the 128x128 kernel would run a single round of K slices or the product
-  // would fall to the register-staged 32x32 tiles (contractions of up to 1024), up to 40 % where a dimension of 64 or less made
-  // the 128-wide tiles half empty; against the 128x128 kernel on several rounds of long K slices it
-  // loses, and so it does on the weight-gradient layout (both operands output-contiguous).
+  // slices of at least eight K steps.  The rule below is fitted to a sweep of 386 mid-size shapes
+  // (batch 128..16384, widths 64..4096), each timed with this route forced and with it off:
+  //   * never below 192 workgroups, and never against several rounds of long 128x128 slices
+  //     (contractions above 1024) - there the 128x128 kernel is 5-20 % ahead;
+  //   * always where a dimension of 64 or less leaves the 128-wide tiles half empty (up to 40 %);
+  //   * forward products otherwise whenever the slices are either not needed (four K steps are
+  //     enough), or at least four, or at least 24 steps long: 5-28 % ahead of the 32x32 tiles and
+  //     of one round of 128x128 slices (two slices of 8-16 steps lose 15-50 %); the rule picks
+  //     within 0.6 % (geometric mean) of the better of the two routes, 10 % at worst;
+  //   * input gradients only where they replace one round of 128x128 slices: an input gradient
+  //     on 32x32 tiles shares a grid with its layer's weight gradient in Linear::backward, which
+  //     is worth more than the faster kernel.
   if (dma_ok && dma64_mode() != 0 && is_a_kc) {
     const long long t64 = tiles(64, 64);
     const int nk = p.K / BK;
@@ -1425,13 +1432,15 @@ Route choose_route(const GemmParams& p, bool vec, int* dma_slices, bool is_a_kc 
     const double flops = 2.0 * p.M * p.N * (double)p.K;
     const double area128 = (double)t128 * 128.0 * 128.0, area64 = (double)t64 * 64.0 * 64.0;
     bool take = dma64_mode() == 1 && t64 * s >= 128 && nk >= 1;
-    if (dma64_mode() != 1 && t64 * s >= 192 && flops >= 2.5e8) {
+    if (dma64_mode() != 1 && t64 * s >= 192) {
       const bool half_empty = area128 >= 1.4 * area64 && steps >= 12;
-      // (an input gradient that would otherwise run as 32x32 tiles shares a grid with its layer's
-      // weight gradient in Linear::backward, which is worth more than the faster kernel: stay there)
-      const bool was_small_tiles = s128 <= 1;
-      const bool beats_one_round = !multi_round && nk <= 64 && (s == 1 ? steps >= 12 : steps >= 24) && (is_b_kc || !was_small_tiles);
-      take = half_empty || beats_one_round;
+      if (is_b_kc) {
+        const bool slices_ok = s == 1 ? steps >= 4 : (steps >= 8 && nk >= 32 && (s >= 4 || steps >= 24));
+        take = half_empty || (multi_round ? nk <= 64 : (slices_ok && (s128 <= 1 || nk <= 64)));
+      } else {
+        const bool beats_one_round = !multi_round && nk <= 64 && (s == 1 ? steps >= 12 : steps >= 24) && s128 > 1;
+        take = flops >= 2.5e8 && (half_empty || beats_one_round);
+      }
     }
     if (take && fits) {
       *dma_slices = (int)s;
