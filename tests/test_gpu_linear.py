@@ -169,7 +169,8 @@ def test_one_hot_input_selects_weight_rows(engine):
 # otherwise, blocks on its edge always divide), db = colsum(G) / batch, dX = (G W) * [x > 0].
 # The shapes mix interior and edge blocks of the 128x128, 64x64 and 32x32 kernels.
 @pytest.mark.parametrize("batch,k,n", [(1024, 384, 300), (1000, 384, 300), (4096, 1024, 1280), (4000, 1024, 1280),
-                                       (512, 4096, 4096), (96, 130, 70), (8192, 784, 100), (8200, 784, 100)])
+                                       (512, 4096, 4096), (96, 130, 70), (8192, 784, 100), (8200, 784, 100),
+                                       (64, 32, 70000), (128, 70000, 64)])  # long rows: large lane offsets in the interior epilogue
 def test_backward_on_integer_data_is_bit_exact(engine, batch, k, n):
     from rstorch_amd import _ffi
     rng = np.random.default_rng(batch + k + n)
