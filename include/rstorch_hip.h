@@ -73,6 +73,7 @@ int rst_fill(rst_engine* engine, double* dst, size_t count, double value);
 
 /* ---- timing on the engine's stream ------------------------------------------------------ */
 int rst_event_create(rst_engine* engine, rst_event** out);
+/* May be called after the event's engine has been destroyed (record and elapsed may not). */
 int rst_event_destroy(rst_event* event);
 int rst_event_record(rst_event* event);
 /* Waits for `stop` and returns the time between the two records in milliseconds. */
@@ -252,12 +253,22 @@ int rst_model_pair_gradients(rst_model* model, int enabled);
  * enabled == 0 switches to plain launches (profiling does so by itself).  Default: enabled,
  * unless the environment says RSTORCH_GRAPH=0. */
 int rst_model_graph_enable(rst_model* model, int enabled);
+/* Environment variables read once per process.  RSTORCH_GRAPH=0: new models launch plainly.
+ * The next two change which kernel a product runs on and therefore the ORDER of its summation
+ * (results stay within rounding, 1e-13 relative, of each other; every setting is deterministic and
+ * independent of the number of compute units):
+ *   RSTORCH_DMA_GROUP=0  small weight gradients never share the grid of K-sliced 128x128 tiles,
+ *                    =1  they do whenever they can (unset: the measured rule);
+ *   RSTORCH_DMA64=0      no product goes to the 64x64 direct-to-LDS kernel, =1 every eligible one. */
 /* Per-launch timing of the model's kernels: when enabled an event is recorded on the engine's
  * stream after every launch (and one before the first launch of a call); a launch's duration runs
  * from the previous event to its own, so it includes the few microseconds between the previous
  * kernel's end and its own start.  While enabled, every layer's weight gradient is a launch of
- * its own (small ones otherwise share one grid at the end of backward; the results are the same
- * bit for bit).  Records
+ * its own.  Small ones otherwise share one grid at the end of backward: bit-identical to the
+ * launches of their own as long as the shared grid runs 32x32 tiles, equal within rounding (1e-13
+ * relative) when the batch is long enough (from about 4096 rows) for the shared grid of K-sliced
+ * 128x128 tiles, which cuts the batch into other slices than a lone launch does and so adds in
+ * another order.  Records
  * accumulate over calls (up to 65536) until rst_model_profile_read, which waits for the stream,
  * copies up to `capacity` of them (host_records == NULL: only counts) and clears the list. */
 typedef struct rst_kernel_record {

@@ -80,10 +80,12 @@ bool can_pair_gemm(const GemmDesc& input_grad, const GemmDesc& weight_grad);
 int launch_gemm_pair(hipStream_t stream, const GemmDesc& input_grad, const GemmDesc& weight_grad);
 // Several small weight gradients (both operands output-contiguous, each a launch of 32x32 tiles
 // on its own, with or without K slices) in one grid, plus one shared reduction grid for the
-// sliced ones; same results as launch_gemm on each.  The descriptors share one workspace, of
-// which each sliced contraction takes gemm_group_workspace(d) doubles.
+// sliced ones; same results as launch_gemm on each, except that from a batch of about 4096 a
+// group of weight gradients runs as K-sliced 128x128 tiles whose slices differ from a lone launch's
+// (equal within rounding, 1e-13).  The descriptors share one workspace, of which the group as a
+// whole takes gemm_group_workspace(d, count) doubles.
 bool can_group_gemm(const GemmDesc& d);
-size_t gemm_group_workspace(const GemmDesc& d);
+size_t gemm_group_workspace(const GemmDesc* d, int count);
 int max_gemm_group();
 int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count);
 

@@ -259,6 +259,7 @@ int rst_fill(rst_engine* e, double* dst, size_t count, double value) {
 // ---- events -------------------------------------------------------------------------------------
 struct rst_event {
   rst_engine* engine;
+  int device;  // kept here so that destroying the event never reads an engine that is already gone
   hipEvent_t ev;
 };
 
@@ -271,6 +272,7 @@ int rst_event_create(rst_engine* e, rst_event** out) {
   rst_event* ev = new (std::nothrow) rst_event();
   if (!ev) return fail(RST_ERR_OUT_OF_MEMORY, "host allocation failed");
   ev->engine = e;
+  ev->device = e->device;
   hipError_t err = hipEventCreate(&ev->ev);
   if (err != hipSuccess) {
     delete ev;
@@ -282,7 +284,7 @@ int rst_event_create(rst_engine* e, rst_event** out) {
 
 int rst_event_destroy(rst_event* ev) {
   if (!ev) return RST_OK;
-  (void)hipSetDevice(ev->engine->device);
+  (void)hipSetDevice(ev->device);
   (void)hipEventDestroy(ev->ev);
   delete ev;
   return RST_OK;

@@ -1566,6 +1566,10 @@ int dma_group_mode() {
 
 constexpr int kDmaGroupMaxSlices = 32;
 constexpr int kDmaGroupMinSteps = 8;
+// The grid the planner aims at: one workgroup for each of the 256 compute units of the part.  A
+// constant, not the device's own count: the number of slices fixes the order in which a weight
+// gradient is summed, and results must not change with the number of CUs a device exposes.
+constexpr int kDmaGroupGrid = 256;
 
 // a weight gradient that the sliced 128x128 group kernel can take at all: at most eight output
 // tiles (more have enough workgroups of their own, and the slices of a larger output would crowd
@@ -1581,8 +1585,10 @@ bool dma_group_member(const GemmDesc& d) {
 // on the step), shortened where a member's contraction would leave a slice fewer than
 // kDmaGroupMinSteps K steps.  False when the members do not qualify, the tiles would be mostly
 // padding, the grid would leave more than a quarter of the chip idle (batches below about 4096 for
-// a handful of tiles), or the workspace is too small.
-bool plan_dma_group(const GemmDesc* d, int count, GemmGroup* g, long long* blocks_out, long long* reduce_out) {
+// a handful of tiles), or the workspace is too small.  *ws_need: doubles of the shared workspace
+// that the plan takes.
+bool plan_dma_group(const GemmDesc* d, int count, GemmGroup* g, long long* blocks_out, long long* reduce_out,
+                    size_t* ws_need = nullptr) {
   if (dma_group_mode() == 0) return false;
   long long tiles = 0;
   double outputs = 0.0;
@@ -1591,13 +1597,12 @@ bool plan_dma_group(const GemmDesc* d, int count, GemmGroup* g, long long* block
     tiles += (long long)((d[i].M + 127) / 128) * ((d[i].N + 127) / 128);
     outputs += (double)d[i].M * d[i].N;
   }
-  const int cus = compute_units();
-  if (tiles > cus / 8) return false;
+  if (tiles > kDmaGroupGrid / 8) return false;
   // Measured on whole training steps of small networks at batch 8192: with 61 % of the 128x128
   // tiles' area in use (784-100-100-10) the step is 6 % shorter than on the 32x32 group (13 % at
   // batch 32768), with 90 % (256-256-256-10) 7 %; with 41 % (1024-64-64-64-16) it is 9 % longer.
   if (dma_group_mode() != 1 && outputs < 0.55 * 16384.0 * (double)tiles) return false;
-  long long want = cus / tiles;
+  long long want = kDmaGroupGrid / tiles;
   if (want > kDmaGroupMaxSlices) want = kDmaGroupMaxSlices;
   long long blocks = 0, reduce_blocks = 0;
   size_t ws_used = 0;
@@ -1627,21 +1632,29 @@ bool plan_dma_group(const GemmDesc* d, int count, GemmGroup* g, long long* block
   }
   g->first_block[count] = (int)blocks;
   g->first_reduce_block[count] = (int)reduce_blocks;
-  if (dma_group_mode() != 1 && blocks < (3 * cus) / 4) return false;
+  if (dma_group_mode() != 1 && blocks < (3 * kDmaGroupGrid) / 4) return false;
   *blocks_out = blocks;
   *reduce_out = reduce_blocks;
+  if (ws_need) *ws_need = ws_used;
   return true;
 }
 }  // namespace
 
-size_t gemm_group_workspace(const GemmDesc& d) {
-  GemmParams p = make_params(d);
-  plan_group_member(p);
-  size_t need = p.split_k > 1 ? (size_t)p.split_k * ((size_t)p.M * p.N + (size_t)p.M) : 0;
-  // the sliced 128x128 grid, should the whole group qualify for it, takes up to kDmaGroupMaxSlices slices
-  if (dma_group_mode() != 0 && dma_group_member(d)) {
-    const size_t dma_need = (size_t)kDmaGroupMaxSlices * ((size_t)p.M * p.N + (size_t)p.M);
-    if (dma_need > need) need = dma_need;
+// What launch_gemm_group(d, count) will take from the workspace the descriptors share: the need of
+// the sliced 128x128 grid when the group as a whole qualifies for it, else the sum over the members'
+// own 32x32 slice plans.
+size_t gemm_group_workspace(const GemmDesc* d, int count) {
+  if (count >= 1 && count <= kMaxGroup) {
+    GemmGroup g{};
+    long long blocks = 0, reduce_blocks = 0;
+    size_t need = 0;
+    if (plan_dma_group(d, count, &g, &blocks, &reduce_blocks, &need)) return need;
+  }
+  size_t need = 0;
+  for (int i = 0; i < count; ++i) {
+    GemmParams p = make_params(d[i]);
+    plan_group_member(p);
+    if (p.split_k > 1) need += (size_t)p.split_k * ((size_t)p.M * p.N + (size_t)p.M);
   }
   return need;
 }

@@ -299,8 +299,14 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
   // shared grid at the end; their operands - the layer's cached input and the gradient buffer of
   // the layer above - stay untouched until then.  Not while profiling: every layer keeps its record.
   std::vector<Pending> held;
-  size_t held_ws = 0;  // doubles of the split-K workspace that the held ones will take
   const bool may_hold = !m->profiling;
+  // doubles of the split-K workspace that the held ones, plus `extra` if given, take as one group
+  auto group_need = [&](const Pending* extra) -> size_t {
+    std::vector<GemmDesc> descs;
+    for (const Pending& q : held) descs.push_back(q.d);
+    if (extra) descs.push_back(extra->d);
+    return gemm_group_workspace(descs.data(), (int)descs.size());
+  };
   auto launch_pending = [&](const Pending& q) -> int {
     Layer& pl = m->layers[q.layer];
     RST_TRY(prof_begin(m, RST_KERNEL_GRAD_WEIGHT, q.layer, q.flops, q.bytes));
@@ -322,7 +328,6 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
       RST_TRY(launch_gemm_group(e->stream, descs.data(), (int)descs.size()));
     }
     held.clear();
-    held_ws = 0;
     return RST_OK;
   };
 
@@ -330,11 +335,9 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
     if (!pend.active) return RST_OK;
     pend.active = false;
     if (may_hold && pend.fused_bias && can_group_gemm(pend.d)) {
-      const size_t need = gemm_group_workspace(pend.d);
       // a full grid (or a full workspace) goes out, and the next one starts
-      if ((int)held.size() == max_gemm_group() || held_ws + need > e->gemm_ws_count) RST_TRY(flush_held());
-      if (need <= e->gemm_ws_count) {
-        held_ws += need;
+      if ((int)held.size() == max_gemm_group() || group_need(&pend) > e->gemm_ws_count) RST_TRY(flush_held());
+      if (group_need(&pend) <= e->gemm_ws_count) {
         held.push_back(pend);
         return RST_OK;
       }

@@ -93,9 +93,9 @@ int rst_linear_backward(rst_engine* e, const double* grad, const double* x, cons
   dx.mask = relu_mask_source; dx.ldmask = (long)in_features;
   dx.workspace = e->d_gemm_ws; dx.workspace_count = e->gemm_ws_count;
   // two small products that do not depend on each other: one grid
+  const GemmDesc both[2] = {dw, dx};
   if (grad_input && can_group_gemm(dw) && can_group_gemm(dx) &&
-      gemm_group_workspace(dw) + gemm_group_workspace(dx) <= e->gemm_ws_count) {
-    const GemmDesc both[2] = {dw, dx};
+      gemm_group_workspace(both, 2) <= e->gemm_ws_count) {
     RST_TRY(launch_gemm_group(e->stream, both, 2));
   } else {
     RST_TRY(launch_gemm(e->stream, dw));

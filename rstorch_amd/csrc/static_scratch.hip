@@ -3,6 +3,9 @@
 // the NaN flags, which rst_cross_entropy keeps in buffers the engine allocates and grows, live
 // here in one fixed array that is part of the library's device image.  Each GPU holds its own
 // copy of that array at its own address for as long as the process lives.
+#include <atomic>
+#include <mutex>
+
 #include "common.h"
 
 namespace rst {
@@ -18,9 +21,12 @@ constexpr size_t kScratchDoubles = kStaticRows + 32;
 static __device__ __align__(256) double scratch[kScratchDoubles];
 
 constexpr int kMaxDevices = 64;
-double* g_scratch_ptr[kMaxDevices] = {};
+// filled in once per device, under the lock, by the first engine that opens the device; read
+// without the lock afterwards (an entry never changes once it is set)
+std::mutex g_scratch_lock;
+std::atomic<double*> g_scratch_ptr[kMaxDevices] = {};
 // a call that stopped between its two launches may have left the working NaN word set
-bool g_scratch_dirty[kMaxDevices] = {};
+std::atomic<bool> g_scratch_dirty[kMaxDevices] = {};
 
 __global__ void clear_flags_kernel(int* flags) {
   if (threadIdx.x < 4) flags[threadIdx.x] = 0;
@@ -28,21 +34,20 @@ __global__ void clear_flags_kernel(int* flags) {
 
 }  // namespace
 
-// Called by rst_engine_create with `device` current.
-int static_scratch_setup(int device, hipStream_t stream) {
+// Called by rst_engine_create with `device` current.  Only the first call for a device does
+// anything: it looks the array's address up.  The array is zero when the device image is loaded,
+// which is the state the flag words must start in, so nothing is launched here - a later engine
+// on the same GPU must not touch words that another engine's call may be using.
+int static_scratch_setup(int device, hipStream_t /*stream*/) {
   if (device < 0 || device >= kMaxDevices)
     return fail(RST_ERR_UNSUPPORTED, "device %d: the static scratch table holds %d devices", device, kMaxDevices);
-  if (!g_scratch_ptr[device]) {
-    void* ptr = nullptr;
-    RST_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
-    if (!ptr) return fail(RST_ERR_HIP, "hipGetSymbolAddress returned a null address");
-    g_scratch_ptr[device] = static_cast<double*>(ptr);
-  }
-  double* base = g_scratch_ptr[device];
-  hipLaunchKernelGGL(clear_flags_kernel, dim3(1), dim3(64), 0, stream,
-                     reinterpret_cast<int*>(base + kFlagSlot));
-  RST_HIP(hipGetLastError());
-  g_scratch_dirty[device] = false;
+  if (g_scratch_ptr[device].load(std::memory_order_acquire)) return RST_OK;
+  std::lock_guard<std::mutex> guard(g_scratch_lock);
+  if (g_scratch_ptr[device].load(std::memory_order_relaxed)) return RST_OK;
+  void* ptr = nullptr;
+  RST_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+  if (!ptr) return fail(RST_ERR_HIP, "hipGetSymbolAddress returned a null address");
+  g_scratch_ptr[device].store(static_cast<double*>(ptr), std::memory_order_release);
   return RST_OK;
 }
 
@@ -61,14 +66,14 @@ extern "C" int rst_cross_entropy_static(rst_engine* e, const double* pred, const
     return fail(RST_ERR_UNSUPPORTED,
                 "cross_entropy_static: %zu rows exceed the fixed scratch of %zu rows; use rst_cross_entropy",
                 rows, kStaticRows);
-  double* base = (e->device >= 0 && e->device < kMaxDevices) ? g_scratch_ptr[e->device] : nullptr;
+  double* base = (e->device >= 0 && e->device < kMaxDevices)
+                     ? g_scratch_ptr[e->device].load(std::memory_order_acquire) : nullptr;
   if (!base) return fail(RST_ERR_STATE, "the static scratch of device %d was never set up", e->device);
   int* flags = reinterpret_cast<int*>(base + kFlagSlot);
-  if (g_scratch_dirty[e->device]) {
+  if (g_scratch_dirty[e->device].exchange(true)) {
     hipLaunchKernelGGL(clear_flags_kernel, dim3(1), dim3(64), 0, e->stream, flags);
     RST_HIP(hipGetLastError());
   }
-  g_scratch_dirty[e->device] = true;
   LossMirror mirror;
   mirror.loss = e->hd_loss;
   mirror.flags = e->hd_flags;

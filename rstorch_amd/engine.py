@@ -30,8 +30,8 @@ class Event:
 
     def __del__(self):
         try:
-            # the native event points at its engine: once that is closed it has gone with it
-            if self.handle and self._engine.handle:
+            # destroying an event does not touch its engine, so this is safe after Engine.close()
+            if self.handle:
                 _ffi.load().rst_event_destroy(self.handle)
             self.handle = None
         except Exception:

@@ -19,6 +19,7 @@ std::set<void*> g_events, g_streams, g_graphs, g_execs;
 bool g_capturing = false;
 int g_captured_nodes = 0;
 long g_launches = 0;
+long g_malloc_calls = 0, g_free_calls = 0;  // every allocating / releasing call, device and pinned
 char g_symbol_storage[1 << 20];
 
 [[noreturn]] void die(const char* what, const void* p) {
@@ -35,6 +36,16 @@ bool known(std::set<void*>& s, void* p) { std::lock_guard<std::mutex> l(g_mu); r
 
 extern "C" long hip_stub_launch_count() { return g_launches; }
 extern "C" long hip_stub_live_device_allocations() { return (long)g_device.size(); }
+extern "C" long hip_stub_allocation_calls() { return g_malloc_calls + g_free_calls; }
+// lets the driver put the engine's stream into capture mode the way a caller's own code would
+extern "C" void hip_stub_begin_capture(void* stream) { (void)hipStreamBeginCapture((hipStream_t)stream, hipStreamCaptureModeThreadLocal); }
+extern "C" int hip_stub_end_capture(void* stream) {
+  hipGraph_t g = nullptr;
+  (void)hipStreamEndCapture((hipStream_t)stream, &g);
+  const int nodes = *(int*)g;
+  (void)hipGraphDestroy(g);
+  return nodes;
+}
 
 hipError_t hipGetDeviceCount(int* n) { *n = 1; return hipSuccess; }
 hipError_t hipSetDevice(int d) { return d == 0 ? hipSuccess : hipErrorInvalidDevice; }
@@ -53,19 +64,22 @@ hipError_t hipGetLastError() { return hipSuccess; }
 
 hipError_t hipMalloc(void** p, size_t bytes) {
   if (g_capturing) die("hipMalloc while the stream is capturing", nullptr);
+  ++g_malloc_calls;
   *p = track(g_device, std::malloc(bytes ? bytes : 1));
   return hipSuccess;
 }
 hipError_t hipFree(void* p) {
   if (!p) return hipSuccess;
   if (g_capturing) die("hipFree while the stream is capturing", p);
+  ++g_free_calls;
   untrack(g_device, p, "hipFree of a pointer that is not a live device allocation");
   std::free(p);
   return hipSuccess;
 }
-hipError_t hipHostMalloc(void** p, size_t bytes, unsigned) { *p = track(g_host, std::calloc(1, bytes ? bytes : 1)); return hipSuccess; }
+hipError_t hipHostMalloc(void** p, size_t bytes, unsigned) { ++g_malloc_calls; *p = track(g_host, std::calloc(1, bytes ? bytes : 1)); return hipSuccess; }
 hipError_t hipHostFree(void* p) {
   if (!p) return hipSuccess;
+  ++g_free_calls;
   untrack(g_host, p, "hipHostFree of a pointer that is not a live pinned allocation");
   std::free(p);
   return hipSuccess;

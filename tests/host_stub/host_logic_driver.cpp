@@ -12,6 +12,9 @@
 
 extern "C" long hip_stub_launch_count();
 extern "C" long hip_stub_live_device_allocations();
+extern "C" long hip_stub_allocation_calls();
+extern "C" void hip_stub_begin_capture(void* stream);
+extern "C" int hip_stub_end_capture(void* stream);
 
 #define OK(expr)                                                                              \
   do {                                                                                        \
@@ -136,6 +139,33 @@ int main() {
       OK(rst_cross_entropy_static(e, x, t, g, 4096, 10, nullptr));
     }
     EXPECT(rst_cross_entropy_static(e, x, t, g, RST_STATIC_CROSS_ENTROPY_MAX_ROWS + 1, 2, nullptr), RST_ERR_UNSUPPORTED);
+    {
+      // the entry point that allocates nothing: no allocating or releasing runtime call, device or
+      // pinned, on a first use at a new size, on the largest batch it takes, or under stream capture
+      // (where the stand-in aborts on an allocation or a synchronisation anyway)
+      const long before = hip_stub_allocation_calls();
+      double loss = 0.0;
+      OK(rst_cross_entropy_static(e, x, t, g, 8192, 10, &loss));
+      OK(rst_cross_entropy_static(e, x, t, g, 37, 1000, nullptr));
+      OK(rst_cross_entropy_static(e, x, t, g, 1, 40000, nullptr));
+      double* big = reinterpret_cast<double*>(x);  // 65536 x 2 doubles fit in the 8192 x 784 buffer
+      OK(rst_cross_entropy_static(e, big, big, big, RST_STATIC_CROSS_ENTROPY_MAX_ROWS, 2, nullptr));
+      hip_stub_begin_capture(rst_engine_stream(e));
+      OK(rst_cross_entropy_static(e, x, t, g, 4096, 10, nullptr));
+      const int nodes = hip_stub_end_capture(rst_engine_stream(e));
+      if (nodes < 1) { std::fprintf(stderr, "the captured call recorded no kernel\n"); return 1; }
+      if (hip_stub_allocation_calls() != before) {
+        std::fprintf(stderr, "rst_cross_entropy_static allocated or freed: %ld runtime calls\n",
+                     hip_stub_allocation_calls() - before);
+        return 1;
+      }
+      // a second engine on the same GPU does not disturb the scratch (set-up runs once per device)
+      const long launches_before = hip_stub_launch_count();
+      rst_engine* second = nullptr;
+      OK(rst_engine_create(0, &second));
+      if (hip_stub_launch_count() != launches_before) { std::fprintf(stderr, "engine creation launched a kernel\n"); return 1; }
+      OK(rst_engine_destroy(second));
+    }
     // more distinct (x, truth, batch, lr) than the graph cache holds: the oldest executables go
     for (int k = 0; k < 20; ++k) OK(rst_model_train_step(a, x + 784 * (k % 11), t, 64, 0.01 + 0.001 * (k % 3), nullptr));
     OK(rst_model_fuse_sgd(a, 0));
