@@ -23,48 +23,13 @@
 #include <cstdlib>
 
 #include "common.h"
+#include "gemm_addressing.h"
 
 namespace rst {
 namespace {
 
 typedef double v4d __attribute__((ext_vector_type(4)));
 typedef double v2d __attribute__((ext_vector_type(2)));
-
-constexpr int BK = 16;
-
-struct GemmParams {
-  const double* A;
-  const double* B;
-  double* C;
-  int M, N, K;
-  long lda, ldb, ldc;
-  int epilogue;
-  const double* bias;
-  double divisor;
-  double divisor_reciprocal;  // exact 1 / divisor when divisor is a power of two, else 0
-  const double* mask;
-  long ldmask;
-  double* colsum;        // weight-gradient launches only: colsum[i] = (sum_k A(i,k)) / colsum_div
-  double colsum_div;
-  // weight-gradient launches of the fused training step: once C = acc / divisor (and colsum) are
-  // stored, the SGD update parm -= lr * grad is applied to the parameter of the same index
-  double* sgd_parm;      // same shape and leading dimension as C, or NULL
-  double* sgd_bias;      // same shape as colsum, or NULL
-  double sgd_lr;
-  int tiles_m, tiles_n;
-  // split-K (small outputs with a long contraction): slice s of the K steps is multiplied by
-  // workgroups [s*tiles, (s+1)*tiles) and lands, without epilogue, in ws[s][M][N] (and its
-  // column sums in ws_colsum[s][M]); split_reduce_kernel adds the slices in order afterwards.
-  int split_k;           // number of slices, 1 = off
-  int steps_per_split;   // K steps (of BK) per slice
-  double* ws;
-  double* ws_colsum;
-  size_t ws_capacity;    // doubles available at ws
-  // 128x128 direct-to-LDS kernel, launches of more than one round of workgroups: the workgroups of
-  // the first round that sit in the upper wave slots of their CU start this many 10 ns ticks late
-  int dephase_ticks;
-  int first_round;       // workgroups that fit on the chip at once
-};
 
 // LDS geometry of one operand tile of EXT rows/cols by BK contraction steps.
 //   contraction-contiguous: [EXT][BK], element (e, k) at e*BK + (k ^ (e & 15)).  The XOR spreads
@@ -81,66 +46,25 @@ struct TileGeom {
   static_assert(EXT * BK / 2 % THREADS == 0, "tile must split evenly over the block");
 };
 
-// Copy one operand tile global -> registers without any divergent branch.
-//   `ext0`/`ext_n`: first row (or column) of the tile along the output dimension and its limit;
-//   rows beyond the limit are clamped onto the last valid ones - they only feed output rows or
-//   columns that are never stored.
-//   `k0`/`k_n`: first contraction index and its limit.  TAIL = false promises k0 + BK <= k_n;
-//   TAIL = true clamps the address and zeroes what lies beyond the limit (both operands do, so
-//   no stray NaN or infinity meets a zero).
-//   VEC = true promises 16-byte alignment of every pair (even leading dimension, even extent).
+// Copy one operand tile global -> registers without any divergent branch: which pair a thread slot
+// takes, with its clamps and the zeroing of the masked K tail, is staged_pair_source's business.
 template <int EXT, bool KC, bool VEC, bool TAIL, int THREADS>
 __device__ __forceinline__ void load_tile(v2d* __restrict__ reg, const double* __restrict__ base,
                                           long ld, int ext0, int ext_n, int k0, int k_n, int tid) {
   constexpr int L = TileGeom<EXT, KC, THREADS>::loads;
 #pragma unroll
   for (int u = 0; u < L; ++u) {
-    const int q = tid + u * THREADS;
-    int e, k;  // coordinates of the first of the two doubles
-    if (KC) {
-      e = ext0 + (q >> 3);  // BK/2 = 8 pairs per row
-      k = k0 + 2 * (q & 7);
-    } else {
-      k = k0 + q / (EXT / 2);
-      e = ext0 + 2 * (q % (EXT / 2));
-    }
+    const PairSource src = staged_pair_source<EXT, KC, VEC, TAIL>(tid + u * THREADS, ld, ext0, ext_n, k0, k_n);
     v2d v;
-    if (KC) {
-      const int ec = e < ext_n ? e : ext_n - 1;
-      int ka = k, kb = k + 1;
-      if (TAIL) {
-        ka = ka < k_n ? ka : k_n - 1;
-        kb = kb < k_n ? kb : k_n - 1;
-      }
-      const double* row = base + (size_t)ec * ld;
-      if (VEC && !TAIL) {
-        v = *reinterpret_cast<const v2d*>(row + ka);
-      } else {
-        v.x = row[ka];
-        v.y = row[kb];
-      }
-      if (TAIL) {
-        v.x = k < k_n ? v.x : 0.0;
-        v.y = k + 1 < k_n ? v.y : 0.0;
-      }
+    if (src.vec) {
+      v = *reinterpret_cast<const v2d*>(base + src.first);
     } else {
-      int kc = k;
-      if (TAIL) kc = kc < k_n ? kc : k_n - 1;
-      const double* row = base + (size_t)kc * ld;
-      if (VEC) {
-        const int ec = e + 1 < ext_n ? e : ext_n - 2;
-        v = *reinterpret_cast<const v2d*>(row + ec);
-      } else {
-        const int ea = e < ext_n ? e : ext_n - 1;
-        const int eb = e + 1 < ext_n ? e + 1 : ext_n - 1;
-        v.x = row[ea];
-        v.y = row[eb];
-      }
-      if (TAIL) {
-        const bool in = k < k_n;
-        v.x = in ? v.x : 0.0;
-        v.y = in ? v.y : 0.0;
-      }
+      v.x = base[src.first];
+      v.y = base[src.second];
+    }
+    if (TAIL) {
+      v.x = src.keep_first ? v.x : 0.0;
+      v.y = src.keep_second ? v.y : 0.0;
     }
     reg[u] = v;
   }
@@ -197,7 +121,7 @@ __device__ __forceinline__ void store_block(const GemmParams& p, const v4d* acc,
     double bias[TN];
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
-      const int col = col0 + j * 16 + lr;
+      const int col = acc_col(col0, j, lr);
       const int cc = col < p.N ? col : p.N - 1;
       if (EPI == EPI_BIAS || EPI == EPI_BIAS_RELU) bias[j] = p.bias[cc];
       if (EPI == EPI_MASK || SGD) {
@@ -205,7 +129,7 @@ __device__ __forceinline__ void store_block(const GemmParams& p, const v4d* acc,
         for (int ii = 0; ii < IB; ++ii)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const int row = row0 + (i0 + ii) * 16 + 4 * r + lk;
+            const int row = acc_row(row0, i0 + ii, r, lk);
             const int rc = row < p.M ? row : p.M - 1;
             extra[ii][j][r] = (EPI == EPI_MASK) ? p.mask[(size_t)rc * p.ldmask + cc]
                                                 : p.sgd_parm[(size_t)rc * p.ldc + cc];
@@ -216,10 +140,10 @@ __device__ __forceinline__ void store_block(const GemmParams& p, const v4d* acc,
     for (int ii = 0; ii < IB; ++ii)
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        const int col = col0 + j * 16 + lr;
+        const int col = acc_col(col0, j, lr);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int row = row0 + (i0 + ii) * 16 + 4 * r + lk;
+          const int row = acc_row(row0, i0 + ii, r, lk);
           double v = acc[(i0 + ii) * TN + j][r];
           if (EPI == EPI_BIAS) v = v + bias[j];
           if (EPI == EPI_BIAS_RELU) v = fmax(v + bias[j], 0.0);
@@ -256,8 +180,8 @@ template <int TM, int TN, int EPI, bool SGD, bool RECIP>
 __device__ __forceinline__ void store_block_interior(const GemmParams& p, const v4d* acc, double* out,
                                                      long ld_out, int row0, int col0, int lr, int lk) {
   constexpr bool BIAS = EPI == EPI_BIAS || EPI == EPI_BIAS_RELU;
-  uint32_t off_c = 8u * (uint32_t)(lk * ld_out + lr);
-  uint32_t off_m = EPI == EPI_MASK ? 8u * (uint32_t)(lk * p.ldmask + lr) : 0u;
+  uint32_t off_c = interior_lane_offset<uint32_t>(lk, lr, ld_out);
+  uint32_t off_m = EPI == EPI_MASK ? interior_lane_offset<uint32_t>(lk, lr, p.ldmask) : 0u;
   char* c_row = reinterpret_cast<char*>(out + (size_t)row0 * ld_out + col0);
   char* w_row = SGD ? reinterpret_cast<char*>(p.sgd_parm + (size_t)row0 * ld_out + col0) : nullptr;
   const char* m_row = EPI == EPI_MASK ? reinterpret_cast<const char*>(p.mask + (size_t)row0 * p.ldmask + col0) : nullptr;
@@ -327,10 +251,9 @@ __device__ __forceinline__ void write_block(const GemmParams& p, const v4d* acc,
   row0 = __builtin_amdgcn_readfirstlane(row0);
   col0 = __builtin_amdgcn_readfirstlane(col0);
   // (leading dimensions below 2^26 doubles keep the 32-bit lane offsets in range)
-  const bool interior = row0 + 16 * TM <= p.M && col0 + 16 * TN <= p.N && p.ldc < (1L << 26) &&
-                        (long)p.N < (1L << 26) && p.ldmask < (1L << 26);
+  const bool interior = block_is_interior(p, row0, col0, TM, TN);
   if (p.split_k > 1) {
-    double* __restrict__ out = p.ws + (size_t)split * p.M * p.N;
+    double* __restrict__ out = p.ws + ws_slice_offset(p, split);
     if (interior) {
       store_block_interior<TM, TN, EPI_NONE, false, false>(p, acc, out, p.N, row0, col0, lr, lk);
       return;
@@ -339,10 +262,10 @@ __device__ __forceinline__ void write_block(const GemmParams& p, const v4d* acc,
     for (int i = 0; i < TM; ++i)
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
-        const int col = col0 + j * 16 + lr;
+        const int col = acc_col(col0, j, lr);
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          const int row = row0 + i * 16 + 4 * r + lk;
+          const int row = acc_row(row0, i, r, lk);
           if (row < p.M && col < p.N) out[(size_t)row * p.N + col] = acc[i * TN + j][r];
         }
       }
@@ -403,7 +326,7 @@ __device__ __forceinline__ void colsum_finish(double partial, double* __restrict
 #pragma unroll
     for (int g = 0; g < G; ++g) t += scratch[g * BM + e];
     if (p.split_k > 1) {
-      p.ws_colsum[(size_t)split * p.M + m0 + e] = t;  // slice sum, reduced later
+      p.ws_colsum[ws_colsum_offset(p, split) + m0 + e] = t;  // slice sum, reduced later
     } else {
       const double g = t / p.colsum_div;
       p.colsum[m0 + e] = g;
@@ -433,29 +356,10 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block, 
   auto lds_a = [&](int stage) { return lds_a_base + stage * GA::size; };
   auto lds_b = [&](int stage) { return lds_b_base + stage * GB::size; };
 
-  // Workgroups are handed to the 8 XCDs round-robin; renumber them so that each XCD (and
-  // its private L2) works on one compact patch of the tile grid, then walk the patch in
-  // groups of 8 tile rows so that concurrently resident workgroups share operand panels.
-  const int n_blocks = p.tiles_m * p.tiles_n;
-  const int split = block / n_blocks;  // K slice of this workgroup (0 without split-K)
-  int logical;
-  {
-    const int pid = block - split * n_blocks;
-    const int xcd = pid & 7, local = pid >> 3;
-    const int base = n_blocks >> 3, rem = n_blocks & 7;
-    logical = xcd * base + (xcd < rem ? xcd : rem) + local;
-  }
-  int tile_m, tile_n;
-  {
-    constexpr int GROUP = 8;
-    const int group_size = GROUP * p.tiles_n;
-    const int group = logical / group_size;
-    const int first_m = group * GROUP;
-    const int gm = (p.tiles_m - first_m) < GROUP ? (p.tiles_m - first_m) : GROUP;
-    const int in_group = logical - group * group_size;
-    tile_m = first_m + in_group % gm;
-    tile_n = in_group / gm;
-  }
+  // (XCD-aware walk of the tile grid: tile_of_block)
+  const TileCoord tc = tile_of_block(p.tiles_m, p.tiles_n, block);
+  const int split = tc.split;  // K slice of this workgroup (0 without split-K)
+  const int tile_m = tc.tile_m, tile_n = tc.tile_n;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int tid = threadIdx.x;
@@ -469,11 +373,9 @@ __device__ __forceinline__ void gemm_tile(const GemmParams& p, const int block, 
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
 
-  const int nk_full = p.K / BK;                     // K steps that need no bounds handling
-  const int nk_all = nk_full + (p.K % BK != 0 ? 1 : 0);
-  const int kt0 = split * p.steps_per_split;        // this workgroup's K steps: [kt0, nk)
-  const int nk = (p.split_k > 1 && kt0 + p.steps_per_split < nk_all) ? kt0 + p.steps_per_split
-                                                                      : nk_all;
+  const StagedSteps ks = staged_k_steps(p.K, p.split_k, p.steps_per_split, split);
+  const int nk_full = ks.nk_full;  // K steps that need no bounds handling
+  const int kt0 = ks.kt0, nk = ks.nk;  // this workgroup's K steps: [kt0, nk)
 
   // Loads the operand tiles of K step `kt` into registers; only the last step can be partial.
   auto fetch = [&](int kt, v2d* ra, v2d* rb) {
@@ -573,22 +475,12 @@ __global__ __launch_bounds__(WGM * WGN * 64, (BURST > 0 ? 1 : WGM * WGN >= 8 ? 4
 // more than its arithmetic).  Workgroups [first_block[i], first_block[i+1]) belong to problem i;
 // problems cut into K slices are finished by one shared reduction grid, whose workgroups
 // [first_reduce_block[i], first_reduce_block[i+1]) belong to problem i.
-constexpr int kMaxGroup = 8;
-struct GemmGroup {
-  int count;
-  int first_block[kMaxGroup + 1];
-  int first_reduce_block[kMaxGroup + 1];
-  unsigned char layout[kMaxGroup];  // bit 0: A contraction-contiguous, bit 1: B (the mixed kernel reads it)
-  GemmParams p[kMaxGroup];
-};
-static_assert(sizeof(GemmGroup) <= 4096, "a group travels as one kernel argument");
 
 template <bool A_KC, bool B_KC, int BURST>
 __global__ __launch_bounds__(256, (BURST > 0 ? 1 : 2)) void gemm_f64_mfma_group(const GemmGroup g) {
   __shared__ __attribute__((aligned(16))) double lds_a[tile_lds_doubles<32, A_KC, 256, BURST>()];
   __shared__ __attribute__((aligned(16))) double lds_b[tile_lds_doubles<32, B_KC, 256, BURST>()];
-  int i = 0;
-  while (i + 1 < g.count && (int)blockIdx.x >= g.first_block[i + 1]) ++i;
+  const int i = group_member_of_block(g.first_block, g.count, (int)blockIdx.x);
   gemm_tile<32, 32, 2, 2, A_KC, B_KC, true, BURST>(g.p[i], (int)blockIdx.x - g.first_block[i], lds_a, lds_b);
 }
 
@@ -598,8 +490,7 @@ __global__ __launch_bounds__(256, (BURST > 0 ? 1 : 2)) void gemm_f64_mfma_mixed_
   // an output-contiguous tile is the larger of the two layouts
   __shared__ __attribute__((aligned(16))) double lds_a[tile_lds_doubles<32, false, 256, BURST>()];
   __shared__ __attribute__((aligned(16))) double lds_b[tile_lds_doubles<32, false, 256, BURST>()];
-  int i = 0;
-  while (i + 1 < g.count && (int)blockIdx.x >= g.first_block[i + 1]) ++i;
+  const int i = group_member_of_block(g.first_block, g.count, (int)blockIdx.x);
   const int block = (int)blockIdx.x - g.first_block[i];
   switch (g.layout[i]) {
     case 0: gemm_tile<32, 32, 2, 2, false, false, true, BURST>(g.p[i], block, lds_a, lds_b); break;
@@ -642,7 +533,7 @@ __device__ __forceinline__ void store_tile_dma(double* __restrict__ lds, const v
     const int q = tid + u * THREADS;
     if (KC) {
       const int e = q >> 3, pr = q & 7;  // row, pair k/2
-      *reinterpret_cast<v2d*>(lds + e * BK + 2 * (pr ^ (e & 7))) = reg[u];
+      *reinterpret_cast<v2d*>(lds + frag_lds_kc(e, pr)) = reg[u];
     } else {
       *reinterpret_cast<v2d*>(lds + (q / (EXT / 2)) * (EXT + 16) + 2 * (q % (EXT / 2))) = reg[u];
     }
@@ -698,26 +589,9 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
   constexpr int B_SIZE = B_KC ? BN * BK : BK * (BN + 16);
   static_assert(A_SIZE <= kDmaStage && B_SIZE <= kDmaStage, "stage size");
 
-  const int n_blocks = p.tiles_m * p.tiles_n;
-  const int split = block / n_blocks;  // K slice of this workgroup (0 without split-K)
-  int logical;
-  {
-    const int pid = block - split * n_blocks;
-    const int xcd = pid & 7, local = pid >> 3;
-    const int base = n_blocks >> 3, rem = n_blocks & 7;
-    logical = xcd * base + (xcd < rem ? xcd : rem) + local;
-  }
-  int tile_m, tile_n;
-  {
-    constexpr int GROUP = 8;
-    const int group_size = GROUP * p.tiles_n;
-    const int group = logical / group_size;
-    const int first_m = group * GROUP;
-    const int gm = (p.tiles_m - first_m) < GROUP ? (p.tiles_m - first_m) : GROUP;
-    const int in_group = logical - group * group_size;
-    tile_m = first_m + in_group % gm;
-    tile_n = in_group / gm;
-  }
+  const TileCoord tc = tile_of_block(p.tiles_m, p.tiles_n, block);
+  const int split = tc.split;  // K slice of this workgroup (0 without split-K)
+  const int tile_m = tc.tile_m, tile_n = tc.tile_n;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -737,28 +611,22 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
   for (int h = 0; h < CH; ++h) {
     const int c = wave + NW * h, cs = wave_s + NW * h;
     if (A_KC) {
-      const int row = 8 * c + (lane >> 3);
-      const int rr = m0 + row < p.M ? row : p.M - 1 - m0;
-      ao[h] = 8u * (uint32_t)((size_t)rr * p.lda + 2 * ((lane & 7) ^ (row & 7)));
-      la[h] = cs * 128;
+      ao[h] = dma_offset_kc<uint32_t>(c, lane, m0, p.M, p.lda);
+      la[h] = dma_lds_chunk_kc(cs);
     } else {
-      const int ge = m0 + 2 * lane + 1 < p.M ? 2 * lane : p.M - 2 - m0;
-      ao[h] = 8u * (uint32_t)((size_t)c * p.lda + ge);
-      la[h] = cs * (BM + 16);
+      ao[h] = dma_offset_oc128<uint32_t>(c, lane, m0, p.M, p.lda);
+      la[h] = dma_lds_chunk_oc128(cs, BM);
     }
     if (B_KC) {
-      const int row = 8 * c + (lane >> 3);
-      const int rr = n0 + row < p.N ? row : p.N - 1 - n0;
-      bo[h] = 8u * (uint32_t)((size_t)rr * p.ldb + 2 * ((lane & 7) ^ (row & 7)));
-      lb[h] = cs * 128;
+      bo[h] = dma_offset_kc<uint32_t>(c, lane, n0, p.N, p.ldb);
+      lb[h] = dma_lds_chunk_kc(cs);
     } else {
-      const int ge = n0 + 2 * lane + 1 < p.N ? 2 * lane : p.N - 2 - n0;
-      bo[h] = 8u * (uint32_t)((size_t)c * p.ldb + ge);
-      lb[h] = cs * (BN + 16);
+      bo[h] = dma_offset_oc128<uint32_t>(c, lane, n0, p.N, p.ldb);
+      lb[h] = dma_lds_chunk_oc128(cs, BN);
     }
   }
-  const long a_step = 8 * (A_KC ? BK : (long)BK * p.lda);  // bytes per K step
-  const long b_step = 8 * (B_KC ? BK : (long)BK * p.ldb);
+  const long a_step = dma_k_step_bytes(A_KC, p.lda);  // bytes per K step
+  const long b_step = dma_k_step_bytes(B_KC, p.ldb);
 
   v4d acc[TM][TN];
 #pragma unroll
@@ -769,11 +637,10 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
   // K steps of this workgroup: all whole ones, or slice `split` of a split contraction.  What is
   // left of K beyond its last whole step (K % 16 indices) is an extra first tile of slice 0, copied
   // into stage 0 by ordinary masked loads; the whole steps follow through the DMA pipeline.
+  const DmaSteps ks = dma_k_steps(p.K, p.split_k, p.steps_per_split, split);
   const int nk_all = p.K / BK;
-  const int kt0 = split * p.steps_per_split;
-  const int nk_dma = (p.split_k > 1) ? ((nk_all - kt0 < p.steps_per_split) ? nk_all - kt0 : p.steps_per_split)
-                                     : nk_all;
-  const bool k_tail = (p.K % BK) != 0 && split == 0;
+  const int kt0 = ks.kt0, nk_dma = ks.nk_dma;
+  const bool k_tail = ks.k_tail;
   const int nk = nk_dma + (k_tail ? 1 : 0);
   a_ptr += (long)kt0 * a_step;
   b_ptr += (long)kt0 * b_step;
@@ -836,10 +703,8 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
 #pragma unroll
   for (int s2 = 0; s2 < 2; ++s2) {
     const int pr = 4 * s2 + lk;  // pair index = k / 2
-    a_off[s2] = 8u * (A_KC ? (uint32_t)((wm * WM + lr) * BK + 2 * (pr ^ (lr & 7)))
-                           : (uint32_t)(2 * pr * (BM + 16) + wm * WM + lr));
-    b_off[s2] = 8u * (B_KC ? (uint32_t)((wn * WN + lr) * BK + 2 * (pr ^ (lr & 7)))
-                           : (uint32_t)(2 * pr * (BN + 16) + wn * WN + lr));
+    a_off[s2] = 8u * (uint32_t)(A_KC ? frag_lds_kc(wm * WM + lr, pr) : frag_lds_oc128(wm * WM + lr, pr, BM));
+    b_off[s2] = 8u * (uint32_t)(B_KC ? frag_lds_kc(wn * WN + lr, pr) : frag_lds_oc128(wn * WN + lr, pr, BN));
   }
   const uint32_t a_base = (uint32_t)(uintptr_t)lds_a, b_base = (uint32_t)(uintptr_t)lds_b;
   v2d fa[4], fb[2][2];  // A fragments (single set), B fragments [buffer][j]
@@ -933,8 +798,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
 __global__ __launch_bounds__(512, 4) void gemm_f64_mfma_dma_group(const GemmGroup g) {
   __shared__ __attribute__((aligned(1024))) double lds_a[2 * kDmaStage];
   __shared__ __attribute__((aligned(1024))) double lds_b[2 * kDmaStage];
-  int i = 0;
-  while (i + 1 < g.count && (int)blockIdx.x >= g.first_block[i + 1]) ++i;
+  const int i = group_member_of_block(g.first_block, g.count, (int)blockIdx.x);
   dma_tile<false, false, 2, 4, 2, 1>(g.p[i], (int)blockIdx.x - g.first_block[i], lds_a, lds_b);
 }
 
@@ -966,7 +830,7 @@ __device__ __forceinline__ void store_tile_dma64(double* __restrict__ lds, const
     const int q = tid + u * 256;
     if (KC) {
       const int e = q >> 3, pr = q & 7;
-      *reinterpret_cast<v2d*>(lds + e * BK + 2 * (pr ^ (e & 7))) = reg[u];
+      *reinterpret_cast<v2d*>(lds + frag_lds_kc(e, pr)) = reg[u];
     } else {
       const int kr = q >> 5, cp = q & 31;
       *reinterpret_cast<v2d*>(lds + kr * kT64 + 2 * (cp ^ (8 * ((kr >> 1) & 3)))) = reg[u];
@@ -978,9 +842,9 @@ __device__ __forceinline__ void store_tile_dma64(double* __restrict__ lds, const
 template <bool KC>
 __device__ __forceinline__ v2d read_pair64(uint32_t stage_bytes, int e, int pr) {
   if constexpr (KC) {
-    return *(lds_cv2d_t)(uintptr_t)(stage_bytes + 8u * (uint32_t)(e * BK + 2 * (pr ^ (e & 7))));
+    return *(lds_cv2d_t)(uintptr_t)(stage_bytes + 8u * (uint32_t)frag_lds_kc(e, pr));
   } else {
-    const uint32_t at = stage_bytes + 8u * (uint32_t)(2 * pr * kT64 + 2 * ((e >> 1) ^ (8 * (pr & 3))) + (e & 1));
+    const uint32_t at = stage_bytes + 8u * (uint32_t)frag_lds_oc64(e, pr);
     v2d r;
     r.x = *(lds_cf64_t)(uintptr_t)at;
     r.y = *(lds_cf64_t)(uintptr_t)(at + 8u * kT64);
@@ -995,26 +859,9 @@ __global__ __launch_bounds__(256, 2) void gemm_f64_mfma_dma64(const GemmParams p
   __shared__ __attribute__((aligned(1024))) double lds_b[kT64Stages * kT64Stage];
   constexpr int BM = kT64, BN = kT64, NW = 4, TM = 2, TN = 2, CH = 2;
   const int block = (int)blockIdx.x;
-  const int n_blocks = p.tiles_m * p.tiles_n;
-  const int split = block / n_blocks;
-  int logical;
-  {
-    const int pid = block - split * n_blocks;
-    const int xcd = pid & 7, local = pid >> 3;
-    const int base = n_blocks >> 3, rem = n_blocks & 7;
-    logical = xcd * base + (xcd < rem ? xcd : rem) + local;
-  }
-  int tile_m, tile_n;
-  {
-    constexpr int GROUP = 8;
-    const int group_size = GROUP * p.tiles_n;
-    const int group = logical / group_size;
-    const int first_m = group * GROUP;
-    const int gm = (p.tiles_m - first_m) < GROUP ? (p.tiles_m - first_m) : GROUP;
-    const int in_group = logical - group * group_size;
-    tile_m = first_m + in_group % gm;
-    tile_n = in_group / gm;
-  }
+  const TileCoord tc = tile_of_block(p.tiles_m, p.tiles_n, block);
+  const int split = tc.split;  // K slice of this workgroup (0 without split-K)
+  const int tile_m = tc.tile_m, tile_n = tc.tile_n;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
@@ -1030,25 +877,13 @@ __global__ __launch_bounds__(256, 2) void gemm_f64_mfma_dma64(const GemmParams p
 #pragma unroll
   for (int h = 0; h < CH; ++h) {
     const int c = wave + NW * h;  // chunk 0..7 of the tile
-    lchunk[h] = (wave_s + NW * h) * 128;
-    {
-      const int row = 8 * c + (lane >> 3);
-      const int rr = m0 + row < p.M ? row : p.M - 1 - m0;
-      ao[h] = 8u * (uint32_t)((size_t)rr * p.lda + 2 * ((lane & 7) ^ (row & 7)));
-    }
-    if (B_KC) {
-      const int row = 8 * c + (lane >> 3);
-      const int rr = n0 + row < p.N ? row : p.N - 1 - n0;
-      bo[h] = 8u * (uint32_t)((size_t)rr * p.ldb + 2 * ((lane & 7) ^ (row & 7)));
-    } else {
-      const int kr = 2 * c + (lane >> 5);
-      const int e = 2 * ((lane & 31) ^ (8 * (c & 3)));  // (kr >> 1) == c
-      const int ge = n0 + e + 1 < p.N ? e : p.N - 2 - n0;
-      bo[h] = 8u * (uint32_t)((size_t)kr * p.ldb + ge);
-    }
+    lchunk[h] = dma_lds_chunk_kc(wave_s + NW * h);  // (the same for both layouts of this tile size)
+    ao[h] = dma_offset_kc<uint32_t>(c, lane, m0, p.M, p.lda);
+    if (B_KC) bo[h] = dma_offset_kc<uint32_t>(c, lane, n0, p.N, p.ldb);
+    else bo[h] = dma_offset_oc64<uint32_t>(c, lane, n0, p.N, p.ldb);
   }
-  const long a_step = 8 * (A_KC ? BK : (long)BK * p.lda);
-  const long b_step = 8 * (B_KC ? BK : (long)BK * p.ldb);
+  const long a_step = dma_k_step_bytes(A_KC, p.lda);
+  const long b_step = dma_k_step_bytes(B_KC, p.ldb);
 
   v4d acc[TM][TN];
 #pragma unroll
@@ -1057,11 +892,10 @@ __global__ __launch_bounds__(256, 2) void gemm_f64_mfma_dma64(const GemmParams p
     for (int j = 0; j < TN; ++j) acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
 
   // tiles of this workgroup: [the masked remainder of K (slice 0 only)] + the whole steps of its slice
+  const DmaSteps ks = dma_k_steps(p.K, p.split_k, p.steps_per_split, split);
   const int nk_all = p.K / BK;
-  const int kt0 = split * p.steps_per_split;
-  const int nk_dma = (p.split_k > 1) ? ((nk_all - kt0 < p.steps_per_split) ? nk_all - kt0 : p.steps_per_split)
-                                     : nk_all;
-  const bool k_tail = (p.K % BK) != 0 && split == 0;
+  const int kt0 = ks.kt0, nk_dma = ks.nk_dma;
+  const bool k_tail = ks.k_tail;
   const int first_dma = k_tail ? 1 : 0;
   const int nk = nk_dma + first_dma;
   a_ptr += (long)kt0 * a_step;
@@ -1141,17 +975,11 @@ __global__ __launch_bounds__(512, 4) void gemm_f64_mfma_dma_pair(const GemmParam
   // their value mod 8, which the XCD-aware tile walk relies on.  The placement is still the
   // dispatcher's: a CU that ends up with two runs of short tiles (each ending in an SGD epilogue)
   // finishes about 10 % late.
-  const int b = (int)blockIdx.x;
-  if (b < 2 * first_blocks) {
-    const int g = b >> 3;
-    const int local = (g >> 1) * 8 + (b & 7);
-    if (((g + (g >> 5)) & 1) == 0)
-      dma_tile<A_KC1, B_KC1, 2, 4, 2, 1>(first, local, lds_a, lds_b);
-    else
-      dma_tile<A_KC2, B_KC2, 2, 4, 2, 1>(second, local, lds_a, lds_b);
-  } else {
-    dma_tile<A_KC2, B_KC2, 2, 4, 2, 1>(second, b - first_blocks, lds_a, lds_b);
-  }
+  const PairSlot slot = pair_slot_of_block((int)blockIdx.x, first_blocks);
+  if (slot.problem == 0)
+    dma_tile<A_KC1, B_KC1, 2, 4, 2, 1>(first, slot.block, lds_a, lds_b);
+  else
+    dma_tile<A_KC2, B_KC2, 2, 4, 2, 1>(second, slot.block, lds_a, lds_b);
 }
 
 // Sum of `count` values `stride` doubles apart, added in order; up to 32 loads are in flight at a
@@ -1219,13 +1047,13 @@ __global__ __launch_bounds__(256) void split_reduce_kernel(const GemmParams p) {
 }
 
 __global__ __launch_bounds__(256) void split_reduce_group_kernel(const GemmGroup g) {
-  int i = 0;
-  while (i + 1 < g.count && (int)blockIdx.x >= g.first_reduce_block[i + 1]) ++i;
+  const int i = group_member_of_block(g.first_reduce_block, g.count, (int)blockIdx.x);
   split_reduce_body(g.p[i], (size_t)((int)blockIdx.x - g.first_reduce_block[i]));
 }
 
 int launch_split_reduce(hipStream_t stream, const GemmParams& p) {
   const size_t mn = (size_t)p.M * p.N;
+  RST_OBSERVE_GEMM(GemmKernel::kSplitReduce, 0, 0, 0, 0, false, false, false, 0, (long long)((mn + 255) / 256), 256, &p, nullptr, 0, nullptr);
   hipLaunchKernelGGL(split_reduce_kernel, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, stream, p);
   RST_HIP(hipGetLastError());
   return RST_OK;
@@ -1275,6 +1103,7 @@ int launch_dma(hipStream_t stream, GemmParams p, int want_split = 0) {
   // more than one round of workgroups (two per CU fit): stagger the first round by 0.4 us per K step
   p.first_round = 2 * compute_units();
   p.dephase_ticks = blocks > p.first_round ? (p.steps_per_split < 250 ? 40 * p.steps_per_split : 10000) : 0;
+  RST_OBSERVE_GEMM(GemmKernel::kDma128, 128, 128, 2, 4, A_KC, B_KC, true, 0, blocks, 512, &p, nullptr, 0, nullptr);
   hipLaunchKernelGGL((gemm_f64_mfma_dma<A_KC, B_KC, 2, 4, 2, 1>), dim3((unsigned)blocks),
                      dim3(512), 0, stream, p);
   RST_HIP(hipGetLastError());
@@ -1300,6 +1129,7 @@ int launch_dma64(hipStream_t stream, GemmParams p, int slices) {
     }
   }
   if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
+  RST_OBSERVE_GEMM(GemmKernel::kDma64, 64, 64, 2, 2, true, B_KC, true, 0, blocks, 256, &p, nullptr, 0, nullptr);
   hipLaunchKernelGGL((gemm_f64_mfma_dma64<B_KC>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
   RST_HIP(hipGetLastError());
   if (p.split_k > 1) RST_TRY(launch_split_reduce(stream, p));
@@ -1347,7 +1177,9 @@ int launch_one(hipStream_t stream, GemmParams p, long long split_below = 256, lo
   plan_slices(p, blocks, split_below, want_blocks);
   blocks *= p.split_k;
   if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
-  if (BM == 32 && BN == 32 && blocks <= compute_units())
+  const bool burst = BM == 32 && BN == 32 && blocks <= compute_units();
+  RST_OBSERVE_GEMM(GemmKernel::kStaged, BM, BN, WGM, WGN, A_KC, B_KC, VEC, burst ? kBurst : 0, blocks, WGM * WGN * 64, &p, nullptr, 0, nullptr);
+  if (burst)
     hipLaunchKernelGGL((gemm_f64_mfma<BM, BN, WGM, WGN, A_KC, B_KC, VEC, (BM == 32 ? kBurst : 0)>),
                        dim3((unsigned)blocks), dim3(WGM * WGN * 64), 0, stream, p);
   else
@@ -1358,10 +1190,11 @@ int launch_one(hipStream_t stream, GemmParams p, long long split_below = 256, lo
   return RST_OK;
 }
 
-// Which kernel a product goes to.  128x128 tiles once they fill the 256 compute units, 64x64 while
-// that still leaves about four workgroups per CU to overlap each other's load latency, else 32x32
-// (which cuts the contraction into slices when even that gives too few workgroups).
-enum class Route { kDma, kDmaSliced, kDma64, kTile128, kTile64, kTile32 };
+// Which kernel a product goes to.  128x128 tiles once they fill the 256 compute units; below that
+// the direct-to-LDS kernels on K slices or 64x64 tiles where the measured rules below say so, else
+// register-staged 32x32 tiles (which cut the contraction into slices when that gives too few
+// workgroups).
+enum class Route { kDma, kDmaSliced, kDma64, kTile128, kTile32 };
 
 // RSTORCH_DMA64: "0" never routes to the 64x64 direct-to-LDS kernel, "1" routes every eligible
 // product there (for measurements); unset: the measured rule in choose_route.
@@ -1451,7 +1284,8 @@ Route choose_route(const GemmParams& p, bool vec, int* dma_slices, bool is_a_kc 
     *dma_slices = s128;
     return Route::kDmaSliced;
   }
-  return tiles(64, 64) >= 1024 ? Route::kTile64 : Route::kTile32;
+  // (register-staged 64x64 tiles have no place here: 1024 of them would mean 256 tiles of 128x128)
+  return Route::kTile32;
 }
 
 template <bool A_KC, bool B_KC, bool VEC>
@@ -1464,7 +1298,6 @@ int launch_layout(hipStream_t stream, const GemmParams& p) {
       if constexpr (A_KC) return launch_dma64<B_KC>(stream, p, slices);
       else return fail(RST_ERR_UNSUPPORTED, "no 64x64 direct-to-LDS kernel for this layout");
     case Route::kTile128: return launch_one<128, 128, 2, 4, A_KC, B_KC, VEC>(stream, p);
-    case Route::kTile64: return launch_one<64, 64, 2, 2, A_KC, B_KC, VEC>(stream, p);
     default: return launch_one<32, 32, 2, 2, A_KC, B_KC, VEC>(stream, p, kSmallTileSplitBelow);
   }
 }
@@ -1667,8 +1500,10 @@ int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count) {
     if (d[i].workspace != d[0].workspace || d[i].workspace_count != d[0].workspace_count)
       return fail(RST_ERR_INVALID_ARGUMENT, "the contractions of a group share one workspace");
   if (plan_dma_group(d, count, &g, &blocks, &reduce_blocks)) {
+    RST_OBSERVE_GEMM(GemmKernel::kDma128Group, 128, 128, 2, 4, false, false, true, 0, blocks, 512, nullptr, nullptr, 0, &g);
     hipLaunchKernelGGL(gemm_f64_mfma_dma_group, dim3((unsigned)blocks), dim3(512), 0, stream, g);
     RST_HIP(hipGetLastError());
+    RST_OBSERVE_GEMM(GemmKernel::kSplitReduceGroup, 0, 0, 0, 0, false, false, false, 0, reduce_blocks, 256, nullptr, nullptr, 0, &g);
     hipLaunchKernelGGL(split_reduce_group_kernel, dim3((unsigned)reduce_blocks), dim3(256), 0, stream, g);
     RST_HIP(hipGetLastError());
     return RST_OK;
@@ -1702,6 +1537,8 @@ int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count) {
   g.first_block[count] = (int)blocks;
   g.first_reduce_block[count] = (int)reduce_blocks;
   const bool burst = blocks <= compute_units();
+  RST_OBSERVE_GEMM(mixed ? GemmKernel::kStagedMixedGroup : GemmKernel::kStagedGroup, 32, 32, 2, 2, false, false, true,
+                   burst ? kBurst : 0, blocks, 256, nullptr, nullptr, 0, &g);
   if (mixed && burst)
     hipLaunchKernelGGL((gemm_f64_mfma_mixed_group<kBurst>), dim3((unsigned)blocks), dim3(256), 0, stream, g);
   else if (mixed)
@@ -1712,6 +1549,7 @@ int launch_gemm_group(hipStream_t stream, const GemmDesc* d, int count) {
     hipLaunchKernelGGL((gemm_f64_mfma_group<false, false, 0>), dim3((unsigned)blocks), dim3(256), 0, stream, g);
   RST_HIP(hipGetLastError());
   if (reduce_blocks > 0) {
+    RST_OBSERVE_GEMM(GemmKernel::kSplitReduceGroup, 0, 0, 0, 0, false, false, false, 0, reduce_blocks, 256, nullptr, nullptr, 0, &g);
     hipLaunchKernelGGL(split_reduce_group_kernel, dim3((unsigned)reduce_blocks), dim3(256), 0, stream, g);
     RST_HIP(hipGetLastError());
   }
@@ -1733,6 +1571,7 @@ int launch_gemm_pair(hipStream_t stream, const GemmDesc& input_grad, const GemmD
   p1.tiles_m = (p1.M + 127) / 128; p1.tiles_n = (p1.N + 127) / 128; p1.steps_per_split = p1.K / BK;
   p2.tiles_m = (p2.M + 127) / 128; p2.tiles_n = (p2.N + 127) / 128; p2.steps_per_split = p2.K / BK;
   const long long b1 = (long long)p1.tiles_m * p1.tiles_n, b2 = (long long)p2.tiles_m * p2.tiles_n;
+  RST_OBSERVE_GEMM(GemmKernel::kDma128Pair, 128, 128, 2, 4, true, false, true, 0, b1 + b2, 512, &p1, &p2, (int)b1, nullptr);
   hipLaunchKernelGGL((gemm_f64_mfma_dma_pair<true, false, false, false>), dim3((unsigned)(b1 + b2)), dim3(512),
                      0, stream, p1, p2, (int)b1);
   RST_HIP(hipGetLastError());
