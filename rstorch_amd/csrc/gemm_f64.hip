@@ -671,20 +671,27 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
         __builtin_amdgcn_s_sleep(32);
     }
   }
-  // prologue: tile 0 in stage 0
-  static_assert(DIST == 1, "the prologue puts exactly one tile in flight");
+  // prologue: tile 0 in stage 0 and, with DIST > 1, tiles 1 .. DIST-1 on their way
+  static_assert(DIST >= 1 && DIST < STAGES && (DIST - 1) * 2 * CH <= 4, "ring of STAGES stages, DIST tiles ahead");
   if (k_tail) {
     v2d ra[(BM * BK / 2) / (NW * 64)], rb[(BN * BK / 2) / (NW * 64)];
     load_tile<BM, A_KC, true, true, NW * 64>(ra, p.A, p.lda, m0, p.M, nk_all * BK, p.K, tid);
     load_tile<BN, B_KC, true, true, NW * 64>(rb, p.B, p.ldb, n0, p.N, nk_all * BK, p.K, tid);
     store_tile_dma<BM, A_KC, NW * 64>(lds_a, ra, tid);
     store_tile_dma<BN, B_KC, NW * 64>(lds_b, rb, tid);
-    __syncthreads();
-  } else {
-    if (nk > 0) issue(0);
-    wait_vmcnt(0);
-    __builtin_amdgcn_s_barrier();
+  } else if (nk > 0) {
+    issue(0);
   }
+#pragma unroll
+  for (int t = 1; t < DIST; ++t)
+    if (t < nk) issue(t % STAGES);
+  {
+    // tile 0 is there once only the younger tiles of the prologue are still outstanding
+    const int younger = nk - 1 < DIST - 1 ? (nk > 0 ? nk - 1 : 0) : DIST - 1;
+    wait_vmcnt(2 * CH * younger);
+  }
+  if (k_tail) __syncthreads();
+  else __builtin_amdgcn_s_barrier();
 
   const bool do_colsum = !A_KC && p.colsum != nullptr && tile_n == 0;
   double colsum_partial = 0.0;
@@ -795,6 +802,9 @@ __global__ __launch_bounds__(WGM * WGN * 64, 4) void gemm_f64_mfma_dma(const Gem
 // in one grid of 128x128 direct-to-LDS tiles: every problem is cut into K slices so that together
 // they give about one workgroup per CU; workgroups [first_block[i], first_block[i+1]) belong to
 // problem i and the shared reduction grid adds the slices up in order.
+// (Three LDS stages with two tiles in flight were measured here, since the grid is one workgroup per
+// CU: 46.0 us against 44.7 us with two stages on C1's weight gradients - the matrix cores, not the
+// trip to memory, set the pace of a K step.)
 __global__ __launch_bounds__(512, 4) void gemm_f64_mfma_dma_group(const GemmGroup g) {
   __shared__ __attribute__((aligned(1024))) double lds_a[2 * kDmaStage];
   __shared__ __attribute__((aligned(1024))) double lds_b[2 * kDmaStage];
