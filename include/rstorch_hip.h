@@ -229,6 +229,22 @@ int rst_model_loss(rst_model* model, const double* truth, double* host_loss);
  * Linear's input gradient, which the README loop discards; otherwise *input_grad receives it. */
 int rst_model_backward(rst_model* model, const double* grad, int need_input_grad,
                        const double** input_grad);
+/* The same two passes for a host-side Sequential that hands arrays over BY VALUE, as the reference's
+ * Module::forward / backward do (src/module/mod.rs:45-47, sequential.rs:78-90): the logits and the
+ * input gradient are written into arrays the caller owns instead of buffers the model reuses.
+ * rst_model_forward_to: logits_out[batch, out].  The model keeps x and logits_out by address until
+ * the backward pass (a trailing ReLU reads logits_out again as its mask): the caller keeps both
+ * alive and unchanged until then.
+ * rst_model_backward_to: grad[batch, out] is the gradient with respect to the logits (what
+ * loss.backward() returned); input_grad_out[batch, in] may be NULL, which skips the first Linear's
+ * input gradient (the README loop drops it).  apply_sgd != 0 also runs SGD::step(lr): inside the
+ * weight-gradient launches (see rst_model_fuse_sgd), i.e. `model.backward(g); optim.step(&mut model)`
+ * as one pass with the same bits as the two calls apart.
+ * Both record their launches into a HIP graph per distinct set of addresses and replay it
+ * afterwards, like rst_model_train_step. */
+int rst_model_forward_to(rst_model* model, const double* x, size_t batch, double* logits_out);
+int rst_model_backward_to(rst_model* model, const double* grad, double* input_grad_out, int apply_sgd,
+                          double lr);
 /* SGD::step over every parameter of the model (one launch over the arena). */
 int rst_model_sgd_step(rst_model* model, double lr);
 /* forward, loss, backward, step: the README loop body (README.md:64-74) without accuracy,
@@ -249,7 +265,8 @@ int rst_model_fuse_sgd(rst_model* model, int enabled);
  * 0.946 ms per pair against 0.477 + 0.503 ms for the two launches one after the other). */
 int rst_model_pair_gradients(rst_model* model, int enabled);
 /* rst_model_train_step records its launches into a HIP graph the first time it sees a given
- * (x, truth, batch, lr) and replays the graph afterwards; a different argument re-records.
+ * (x, truth, batch, lr) and replays the graph afterwards; a different argument re-records (the 64
+ * most recently used graphs of a model are kept).
  * enabled == 0 switches to plain launches (profiling does so by itself).  Default: enabled,
  * unless the environment says RSTORCH_GRAPH=0. */
 int rst_model_graph_enable(rst_model* model, int enabled);

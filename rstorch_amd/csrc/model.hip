@@ -67,6 +67,7 @@ struct rst_model {
   // (a buffer shared through the engine could be reallocated by another caller between two replays)
   double* row_loss = nullptr;
   const double* logits = nullptr;
+  const double* forward_x = nullptr;  // the input of the forward whose caches are live
   // state machine (mirrors the Option::take() caches of the reference)
   bool forward_valid = false;
   bool loss_grad_valid = false;
@@ -74,13 +75,25 @@ struct rst_model {
   // the captured training step (one graph launch instead of ~10 kernel launches)
   // (a few graphs are kept: a staged input pipeline alternates between its slots' buffers)
   bool graph_enabled = true;
+  // what a recorded graph was recorded for: every address its kernels were given, the batch and
+  // the learning rate.  kind: 0 the whole step (x, truth), 1 forward into a caller's array (x, out),
+  // 2 backward from a caller's gradient (grad, input-gradient destination, and the forward's x and
+  // out, which the weight gradient of the first layer and the mask of the last ReLU read)
   struct StepGraph {
     hipGraphExec_t exec;
+    int kind;
     const double* x;
     const double* truth;
+    const double* aux0;
+    const double* aux1;
     size_t batch;
     double lr;
+    int flags;
     unsigned long long last_use;
+    bool matches(int k, const double* a, const double* b, const double* c, const double* d, size_t n, double l,
+                 int f) const {
+      return kind == k && x == a && truth == b && aux0 == c && aux1 == d && batch == n && lr == l && flags == f;
+    }
   };
   std::vector<StepGraph> graphs;
   unsigned long long graph_clock = 0;
@@ -100,7 +113,9 @@ struct rst_model {
 
 namespace {
 
-constexpr size_t kMaxStepGraphs = 8;
+// recorded graphs kept per model: a loop that walks a pool of resident batches records one forward
+// and one backward graph per batch
+constexpr size_t kMaxStepGraphs = 64;
 
 // Whether a new model records its step into a HIP graph: yes, unless RSTORCH_GRAPH=0 (plain
 // launches are handy for debuggers and for comparing the two launch modes from outside).
@@ -200,24 +215,38 @@ int next_non_identity(const rst_model* m, int i) {
   return -1;
 }
 
-int do_forward(rst_model* m, const double* x, size_t batch) {
+// final_out != NULL: the last layer that computes anything writes there instead of into the model's
+// own buffer (the caller's array that Sequential::forward returns by value; backward reads it again
+// as the mask of a trailing ReLU, so it must stay as it is until then).
+// launch == false: only the bookkeeping of the pass (which tensor each layer keeps for backward) -
+// what a replayed graph leaves undone on the host.
+int do_forward(rst_model* m, const double* x, size_t batch, double* final_out = nullptr, bool launch = true) {
   rst_engine* e = m->engine;
   if (batch > (size_t)INT_MAX) return fail(RST_ERR_UNSUPPORTED, "batch too large");
-  RST_TRY(reserve_activations(m, batch));
+  if (launch) RST_TRY(reserve_activations(m, batch));
   m->batch = batch;
   const double* cur = x;
   const int n = (int)m->layers.size();
+  int last = -1;  // the last layer with a launch of its own: a Linear, or a ReLU that no Linear absorbs
+  for (int i = n - 1; i >= 0 && last < 0; --i) {
+    if (m->layers[i].kind == RST_LAYER_LINEAR) last = i;
+    if (m->layers[i].kind == RST_LAYER_RELU) {
+      const int pv = prev_non_identity(m, i);
+      last = (pv >= 0 && m->layers[pv].kind == RST_LAYER_LINEAR) ? pv : i;
+    }
+  }
   for (auto& l : m->layers) { l.absorbed = false; l.relu_fused = false; l.backward_absorbed = false; }
   for (int i = 0; i < n; ++i) {
     Layer& l = m->layers[i];
     if (l.kind == RST_LAYER_IDENTITY) continue;  // identity.rs:17-19
+    double* const dest = (final_out && i == last) ? final_out : l.out_buf;
     if (l.kind == RST_LAYER_LINEAR) {
       const int nx = next_non_identity(m, i);
       const bool fuse = nx >= 0 && m->layers[nx].kind == RST_LAYER_RELU;
       l.input = cur;  // linear.rs:56 keeps the input for backward
       l.relu_fused = fuse;
       GemmDesc d{};
-      d.A = cur; d.B = l.w; d.C = l.out_buf;
+      d.A = cur; d.B = l.w; d.C = dest;
       d.M = (int)batch; d.N = (int)l.out; d.K = (int)l.in;
       d.lda = (long)l.in; d.ldb = (long)l.in; d.ldc = (long)l.out;
       d.a_kc = true; d.b_kc = true;
@@ -225,29 +254,34 @@ int do_forward(rst_model* m, const double* x, size_t batch) {
       d.bias = l.b;
       const double flops = 2.0 * (double)batch * (double)l.in * (double)l.out;
       const double bytes = 8.0 * ((double)batch * l.in + (double)l.in * l.out + (double)batch * l.out);
-      RST_TRY(prof_begin(m, RST_KERNEL_LINEAR_FORWARD, i, flops, bytes));
       d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
-      RST_TRY(launch_gemm(e->stream, d));
-      RST_TRY(prof_end(m));
-      cur = l.out_buf;
+      if (launch) {
+        RST_TRY(prof_begin(m, RST_KERNEL_LINEAR_FORWARD, i, flops, bytes));
+        RST_TRY(launch_gemm(e->stream, d));
+        RST_TRY(prof_end(m));
+      }
+      cur = dest;
       if (fuse) {
         Layer& r = m->layers[nx];
         r.absorbed = true;
         r.input = nullptr;
-        r.mask_source = l.out_buf;  // relu(z) > 0 == z > 0
+        r.mask_source = dest;  // relu(z) > 0 == z > 0
       }
     } else {  // ReLU
       if (l.absorbed) continue;  // its output already is `cur`
       const size_t cnt = batch * l.width_in;
       l.input = cur;        // relu.rs:20 keeps the pre-activation
       l.mask_source = cur;
-      RST_TRY(prof_begin(m, RST_KERNEL_RELU_FORWARD, i, 0.0, 16.0 * (double)cnt));
-      RST_TRY(launch_relu_forward(e->stream, cur, l.out_buf, cnt));
-      RST_TRY(prof_end(m));
-      cur = l.out_buf;
+      if (launch) {
+        RST_TRY(prof_begin(m, RST_KERNEL_RELU_FORWARD, i, 0.0, 16.0 * (double)cnt));
+        RST_TRY(launch_relu_forward(e->stream, cur, dest, cnt));
+        RST_TRY(prof_end(m));
+      }
+      cur = dest;
     }
   }
   m->logits = cur;
+  m->forward_x = x;
   m->forward_valid = true;
   m->loss_grad_valid = false;
   return RST_OK;
@@ -268,8 +302,11 @@ int do_loss(rst_model* m, const double* truth, double* host_loss) {
 
 // fused_lr != NULL: every weight-gradient launch also applies the SGD update to its layer
 // (the input gradient, which needs the old weights, is launched first).
+// input_grad_dest != NULL (with need_input_grad): the gradient with respect to the model's input is
+// written there (the caller's array that Sequential::backward returns by value) instead of into the
+// model's own buffer.
 int do_backward(rst_model* m, const double* grad, int need_input_grad, const double** input_grad,
-                const double* fused_lr) {
+                const double* fused_lr, double* input_grad_dest = nullptr) {
   rst_engine* e = m->engine;
   if (!m->forward_valid)
     return fail(RST_ERR_STATE, "backward without a forward (the reference panics on a consumed cache)");
@@ -284,6 +321,18 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
   int first_linear = -1;
   for (int i = 0; i < n; ++i)
     if (m->layers[i].kind == RST_LAYER_LINEAR) { first_linear = i; break; }
+  // the layer whose launch produces the gradient with respect to the model's input: the first layer
+  // that is not an Identity, or, when that is a ReLU feeding a Linear, the Linear (whose epilogue
+  // applies the ReLU's mask)
+  int producer = -1;
+  if (need_input_grad && input_grad_dest) {
+    for (int i = 0; i < n && producer < 0; ++i)
+      if (m->layers[i].kind != RST_LAYER_IDENTITY) producer = i;
+    if (producer >= 0 && m->layers[producer].kind == RST_LAYER_RELU) {
+      const int nx = next_non_identity(m, producer);
+      if (nx >= 0 && m->layers[nx].kind == RST_LAYER_LINEAR) producer = nx;
+    }
+  }
 
   // a weight gradient that has been described but not launched yet
   struct Pending {
@@ -347,13 +396,14 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
   for (int i = n - 1; i >= 0; --i) {
     Layer& l = m->layers[i];
     if (l.kind == RST_LAYER_IDENTITY) continue;  // identity.rs:22-24
+    double* const gin = (i == producer) ? input_grad_dest : l.grad_in_buf;
     if (l.kind == RST_LAYER_RELU) {
       if (l.backward_absorbed) continue;
       const size_t cnt = batch * l.width_in;
       RST_TRY(prof_begin(m, RST_KERNEL_RELU_BACKWARD, i, 0.0, 24.0 * (double)cnt));
-      RST_TRY(launch_relu_backward(e->stream, cur, l.mask_source, l.grad_in_buf, cnt));
+      RST_TRY(launch_relu_backward(e->stream, cur, l.mask_source, gin, cnt));
       RST_TRY(prof_end(m));
-      cur = l.grad_in_buf;
+      cur = gin;
       continue;
     }
     // Linear: linear.rs:60-69.  The input gradient goes first: it reads the weights, which the
@@ -367,7 +417,7 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
     GemmDesc dx{};
     double dx_bytes = 0.0;
     if (wanted) {
-      dx.A = cur; dx.B = l.w; dx.C = l.grad_in_buf;
+      dx.A = cur; dx.B = l.w; dx.C = gin;
       dx.M = (int)batch; dx.N = (int)l.in; dx.K = (int)l.out;
       dx.lda = (long)l.out; dx.ldb = (long)l.in; dx.ldc = (long)l.in;
       dx.a_kc = true; dx.b_kc = false;
@@ -418,7 +468,7 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
       pend.active = true;
     }
     if (!wanted) { cur = nullptr; break; }
-    cur = l.grad_in_buf;
+    cur = gin;
   }
   RST_TRY(flush_pending());
   RST_TRY(flush_held());
@@ -652,15 +702,15 @@ int run_step(rst_model* m, const double* x, const double* truth, size_t batch, d
   return RST_OK;
 }
 
-// Records the launches of one step into a graph.  Everything the step allocates lazily is
-// reserved first, because allocation is not allowed while the stream is capturing.  The graph
-// holds kernel nodes only (no memset nodes).
-int capture_step(rst_model* m, const double* x, const double* truth, size_t batch, double lr,
-                 hipGraphExec_t* out) {
+// Records what `run` launches into a graph.  Everything the launches allocate lazily is reserved
+// first, because allocation is not allowed while the stream is capturing.  The graph holds kernel
+// nodes only (no memset nodes).  `key` says what the graph was recorded for.
+template <class Run>
+int capture_graph(rst_model* m, rst_model::StepGraph key, Run run, hipGraphExec_t* out) {
   rst_engine* e = m->engine;
-  RST_TRY(reserve_activations(m, batch));  // drops every graph if the buffers move
+  RST_TRY(reserve_activations(m, key.batch));  // drops every graph if the buffers move
   RST_HIP(hipStreamBeginCapture(e->stream, hipStreamCaptureModeThreadLocal));
-  const int status = run_step(m, x, truth, batch, lr);
+  const int status = run();
   hipGraph_t graph = nullptr;
   const hipError_t end = hipStreamEndCapture(e->stream, &graph);
   if (status != RST_OK) {
@@ -680,10 +730,24 @@ int capture_step(rst_model* m, const double* x, const double* truth, size_t batc
     (void)hipGraphExecDestroy(m->graphs[victim].exec);
     m->graphs.erase(m->graphs.begin() + victim);
   }
-  m->graphs.push_back(rst_model::StepGraph{exec, x, truth, batch, lr, 0});
+  key.exec = exec;
+  key.last_use = ++m->graph_clock;
+  m->graphs.push_back(key);
   *out = exec;
   return RST_OK;
 }
+
+// the recorded graph for `key`, if there is one
+hipGraphExec_t find_graph(rst_model* m, const rst_model::StepGraph& key) {
+  for (auto& g : m->graphs)
+    if (g.matches(key.kind, key.x, key.truth, key.aux0, key.aux1, key.batch, key.lr, key.flags)) {
+      g.last_use = ++m->graph_clock;
+      return g.exec;
+    }
+  return nullptr;
+}
+
+bool use_graphs(const rst_model* m) { return m->graph_enabled && !m->profiling; }
 
 }  // namespace
 
@@ -697,17 +761,10 @@ int rst_model_train_step(rst_model* m, const double* x, const double* truth, siz
   RST_TRY(engine_activate(e));
   if (!x || !truth) return fail(RST_ERR_INVALID_ARGUMENT, "x or truth is null");
   if (batch == 0) return fail(RST_ERR_SHAPE, "training step on an empty batch");
-  if (m->graph_enabled && !m->profiling) {
-    hipGraphExec_t exec = nullptr;
-    for (auto& g : m->graphs)
-      if (g.x == x && g.truth == truth && g.batch == batch && g.lr == lr) {
-        exec = g.exec;
-        g.last_use = ++m->graph_clock;
-      }
-    if (!exec) {
-      RST_TRY(capture_step(m, x, truth, batch, lr, &exec));
-      m->graphs.back().last_use = ++m->graph_clock;
-    }
+  if (use_graphs(m)) {
+    const rst_model::StepGraph key{nullptr, 0, x, truth, nullptr, nullptr, batch, lr, 0, 0};
+    hipGraphExec_t exec = find_graph(m, key);
+    if (!exec) RST_TRY(capture_graph(m, key, [&] { return run_step(m, x, truth, batch, lr); }, &exec));
     RST_HIP(hipGraphLaunch(exec, e->stream));
     // the state the eager calls leave behind
     m->batch = batch;
@@ -720,6 +777,53 @@ int rst_model_train_step(rst_model* m, const double* x, const double* truth, siz
   }
   if (host_loss) return rst_loss_value(e, host_loss);
   return RST_OK;
+}
+
+int rst_model_forward_to(rst_model* m, const double* x, size_t batch, double* logits_out) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->chain_open = false;
+  rst_engine* e = m->engine;
+  RST_TRY(engine_activate(e));
+  if (batch && (!x || !logits_out)) return fail(RST_ERR_INVALID_ARGUMENT, "x or logits_out is null");
+  if (use_graphs(m) && batch > 0) {
+    const rst_model::StepGraph key{nullptr, 1, x, logits_out, nullptr, nullptr, batch, 0.0, 0, 0};
+    hipGraphExec_t exec = find_graph(m, key);
+    if (!exec) RST_TRY(capture_graph(m, key, [&] { return do_forward(m, x, batch, logits_out); }, &exec));
+    RST_HIP(hipGraphLaunch(exec, e->stream));
+    // which tensor each layer keeps for backward: what the recorded launches cannot leave behind
+    return do_forward(m, x, batch, logits_out, false);
+  }
+  return do_forward(m, x, batch, logits_out);
+}
+
+int rst_model_backward_to(rst_model* m, const double* grad, double* input_grad_out, int apply_sgd,
+                          double lr) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->chain_open = false;
+  rst_engine* e = m->engine;
+  RST_TRY(engine_activate(e));
+  if (!grad) return fail(RST_ERR_INVALID_ARGUMENT, "grad is null");
+  if (!m->forward_valid)
+    return fail(RST_ERR_STATE, "backward without a forward (the reference panics on a consumed cache)");
+  const int need = input_grad_out != nullptr;
+  const bool fused = apply_sgd != 0 && m->fuse_sgd;
+  auto run = [&]() -> int {
+    RST_TRY(do_backward(m, grad, need, nullptr, fused ? &lr : nullptr, input_grad_out));
+    if (apply_sgd && !fused) RST_TRY(do_sgd(m, lr));
+    return RST_OK;
+  };
+  if (use_graphs(m) && m->batch > 0) {
+    const rst_model::StepGraph key{nullptr, 2, grad, input_grad_out, m->forward_x, m->logits, m->batch,
+                                   apply_sgd ? lr : 0.0, apply_sgd ? 1 : 0, 0};
+    hipGraphExec_t exec = find_graph(m, key);
+    if (!exec) RST_TRY(capture_graph(m, key, run, &exec));
+    RST_HIP(hipGraphLaunch(exec, e->stream));
+    m->forward_valid = false;  // the caches are consumed, as after the eager pass
+    m->loss_grad_valid = false;
+    m->grads_valid = true;
+    return RST_OK;
+  }
+  return run();
 }
 
 int rst_model_fuse_sgd(rst_model* m, int enabled) {

@@ -123,18 +123,44 @@ class Engine:
 
 
 class Array2:
-    """Dense row-major f64 matrix in device memory."""
+    """Dense row-major f64 matrix in device memory.
 
-    def __init__(self, engine, rows, cols, ptr=None, owner=None):
+    ``ptr`` is the device address.  Two kinds of array fill it in late: the gradient views that a
+    compiled ``Sequential`` hands out (reading ``ptr`` first runs the backward pass that
+    ``backward`` deferred, see ``rstorch_amd.module``) and the input gradient that ``backward``
+    returns (computed only if somebody looks at it).  Every access to the contents goes through
+    ``ptr``, so such an array behaves like any other."""
+
+    def __init__(self, engine, rows, cols, ptr=None, owner=None, before_access=None, resolver=None):
         self.engine = engine
         self.rows, self.cols = int(rows), int(cols)
-        if ptr is None:
-            self.ptr = engine.malloc(self.rows * self.cols)
+        self._before_access = before_access  # called before every read of ``ptr`` (or None)
+        self._resolver = resolver            # called once, to produce the contents (or None)
+        if resolver is not None:
+            self._ptr = None
+            self._owns = False
+        elif ptr is None:
+            self._ptr = engine.malloc(self.rows * self.cols)
             self._owns = True
         else:
-            self.ptr = ptr
+            self._ptr = ptr
             self._owns = False
         self._owner = owner  # keeps the owning object alive for borrowed views
+
+    @property
+    def ptr(self):
+        if self._resolver is not None:
+            resolver, self._resolver = self._resolver, None
+            resolver(self)
+        if self._before_access is not None:
+            self._before_access()
+        return self._ptr
+
+    def _materialise(self):
+        """Gives a deferred array memory of its own (called by its resolver)."""
+        self._ptr = self.engine.malloc(self.rows * self.cols)
+        self._owns = True
+        return self._ptr
 
     @property
     def shape(self):
@@ -176,9 +202,9 @@ class Array2:
 
     def __del__(self):
         try:
-            if self._owns and self.ptr and self.engine.handle:
-                self.engine.free(self.ptr)
-            self.ptr = None
+            if self._owns and self._ptr and self.engine.handle:
+                self.engine.free(self._ptr)
+            self._ptr = None
         except Exception:
             pass
 

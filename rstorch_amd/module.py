@@ -5,8 +5,26 @@ Same names, argument meaning and failure behaviour as
 ``forward`` / ``backward`` / ``parameters`` / ``train`` / ``eval``; caches are consumed by
 ``backward`` (a second ``backward`` raises, where the reference panics on ``unwrap``);
 gradients are overwritten, never accumulated.  Arrays are device-resident ``Array2``.
+
+A ``Sequential`` made only of ``Identity`` / ``Linear`` / ``ReLU`` layers is *compiled*: the first
+``forward`` builds a device model (``rst_model``) over the layer list, moves the layers' weights
+into its parameter arena (the layers keep views) and from then on
+
+* ``forward`` is one replayed graph of the layers' launches,
+* ``backward`` launches nothing: it remembers its gradient, and the pass runs when somebody needs
+  its results - ``SGD.step(model)`` runs it with the optimiser update inside the weight-gradient
+  launches (one replayed graph: the README loop's ``model.backward(loss.backward());
+  optim.step(model)`` reaches exactly the launches of ``rst_model_train_step``), while reading a
+  gradient through ``parameters()`` or touching the input gradient that ``backward`` returned runs
+  it on its own first, so every value a caller can observe is the value the reference computes at
+  that point.  The input gradient itself is only computed if the returned array is kept.
+
+Any other layer list (a ``Softmax`` module, a user-defined ``Module``) runs layer by layer.  Changing
+the layer list (``push`` / ``insert`` / ``remove``) drops the compiled form; it is rebuilt on the next
+``forward``.
 """
 import ctypes
+import weakref
 
 from . import _ffi
 from .engine import Array2, as_array2, default_engine
@@ -175,6 +193,8 @@ class Linear(Module):
         self.prev_input = None
         self.grad_weight = None
         self.grad_bias = None
+        self._home = None       # the compiled Sequential (_Plan) whose arena holds the parameters
+        self._has_grad = False  # a backward pass has been asked for since the layer was made
 
     @classmethod
     def new(cls, input_size, output_size):
@@ -210,6 +230,7 @@ class Linear(Module):
         if self.grad_weight is None:
             self.grad_weight = self.engine.empty(self.output_size, self.input_size)
             self.grad_bias = self.engine.empty(1, self.output_size)
+        self._has_grad = True
         gx = self.engine.empty(x.rows, self.input_size) if need_input_grad else None
         _ffi.check(self.engine.lib.rst_linear_backward(
             self.engine.handle, g.ptr, x.ptr, self.weight.ptr, self.grad_weight.ptr,
@@ -222,7 +243,7 @@ class Linear(Module):
         return self._backward(gradient, False)
 
     def parameters(self):
-        if self.grad_weight is None:
+        if not self._has_grad:
             raise _ffi.StateError(_ffi.RST_ERR_STATE,
                                   "Linear.parameters before any backward (no gradient yet)")
         return Parameters().add(self.weight, self.grad_weight).add(self.bias, self.grad_bias)
@@ -231,23 +252,147 @@ class Linear(Module):
         return "Linear(%d, %d)" % (self.input_size, self.output_size)
 
 
+class _Plan:
+    """The compiled form of a Sequential of Identity / Linear / ReLU layers: an ``rst_model`` whose
+    arena holds the layers' parameters and gradients, plus the backward pass that has been asked
+    for but not launched yet."""
+
+    def __init__(self, layers):
+        from .model import DeviceModel
+        self.key = tuple(id(l) for l in layers)
+        self.linears = [l for l in layers if type(l) is Linear]
+        spec = []
+        for l in layers:
+            if type(l) is Linear:
+                spec.append(("linear", l.input_size, l.output_size))
+            else:
+                spec.append(("relu",) if type(l) is ReLU else ("identity",))
+        self.engine = self.linears[0].engine
+        for l in self.linears:  # whatever another compiled Sequential still owes these layers
+            if l._home is not None:
+                l._home.flush()
+        self.device = DeviceModel(spec, self.engine)
+        eng, params = self.engine, self.device.parameters()
+        for i, l in enumerate(self.linears):
+            (w, gw), (b, gb) = params[2 * i], params[2 * i + 1]
+            _ffi.check(eng.lib.rst_copy(eng.handle, w._ptr, l.weight.ptr, w.size))
+            _ffi.check(eng.lib.rst_copy(eng.handle, b._ptr, l.bias.ptr, b.size))
+            if l._has_grad and l.grad_weight is not None:  # gradients computed before the move stay readable
+                _ffi.check(eng.lib.rst_copy(eng.handle, gw._ptr, l.grad_weight.ptr, gw.size))
+                _ffi.check(eng.lib.rst_copy(eng.handle, gb._ptr, l.grad_bias.ptr, gb.size))
+            l.weight, l.bias = w, b
+            # reading a gradient first runs the backward pass that is still owed
+            gw._before_access = gb._before_access = self.flush
+            l.grad_weight, l.grad_bias = gw, gb
+            l._home = self
+        self.in_width, self.out_width = self.device.in_width, self.device.out_width
+        self.x = self.out = None      # the forward pass whose caches are live (kept alive until backward)
+        self.pending = None           # (gradient, weak reference to the deferred input gradient)
+
+    def valid_for(self, layers):
+        return self.key == tuple(id(l) for l in layers) and all(l._home is self for l in self.linears)
+
+    def forward(self, input):
+        self.flush()  # a backward pass nobody looked at would otherwise read the new activations
+        x = as_array2(input, self.engine)
+        if x.cols != self.in_width:
+            raise _ffi.ShapeError(_ffi.RST_ERR_SHAPE, "input has %d features, layer expects %d"
+                                  % (x.cols, self.in_width))
+        out = self.engine.empty(x.rows, self.out_width)
+        _ffi.check(self.engine.lib.rst_model_forward_to(self.device.handle, x.ptr, x.rows, out.ptr))
+        self.x, self.out = x, out
+        return out
+
+    def backward(self, gradient):
+        if self.x is None or self.pending is not None:  # no forward yet, or its caches are taken
+            raise _ffi.StateError(_ffi.RST_ERR_STATE, "Sequential.backward without a forward")
+        g = as_array2(gradient, self.engine)
+        if g.shape != (self.x.rows, self.out_width):
+            raise _ffi.ShapeError(_ffi.RST_ERR_SHAPE, "gradient %r vs expected %r"
+                                  % (g.shape, (self.x.rows, self.out_width)))
+        gin = Array2(self.engine, self.x.rows, self.in_width, resolver=self._resolve_input_grad)
+        self.pending = (g, weakref.ref(gin))
+        for l in self.linears:
+            l._has_grad = True
+        return gin
+
+    def _resolve_input_grad(self, gin):
+        """Somebody looks at the array that backward() returned."""
+        if self.pending is not None and self.pending[1]() is gin:
+            self._run(False, 0.0)
+        if gin._ptr is None:
+            raise _ffi.StateError(_ffi.RST_ERR_STATE, "this input gradient was never computed")
+
+    def _run(self, apply_sgd, lr):
+        g, ref = self.pending
+        self.pending = None
+        gin = ref()  # still wanted by somebody?
+        if gin is not None:
+            gin._resolver = None
+            gin._materialise()
+        _ffi.check(self.engine.lib.rst_model_backward_to(
+            self.device.handle, g.ptr, gin._ptr if gin is not None else None, 1 if apply_sgd else 0, float(lr)))
+        self.x = self.out = None  # the caches are consumed
+
+    def flush(self):
+        """Runs the backward pass that is still owed, without an optimiser step."""
+        if self.pending is not None:
+            self._run(False, 0.0)
+
+    def step_sgd(self, lr):
+        """backward + SGD::step in one pass, if a backward is still owed; else False."""
+        if self.pending is None:
+            return False
+        self._run(True, lr)
+        return True
+
+
 class Sequential(Module):
     """src/module/sequential.rs:11-110.  The layer list may change at any time; the
     Linear/ReLU fusion is decided afresh on every call."""
 
+    # False (on the class or on one instance): always run layer by layer, one call per layer
+    compile_enabled = True
+
     def __init__(self, layers=None):
         self.layers = list(layers or [])
+        self._plan = None
+
+    def _compiled(self):
+        """The compiled form, built on demand; None when the layer list has a layer it cannot hold."""
+        if not self.compile_enabled:
+            self._drop_plan()
+            return None
+        if self._plan is not None and self._plan.valid_for(self.layers):
+            return self._plan
+        self._drop_plan()
+        linears = [l for l in self.layers if type(l) is Linear]
+        if not linears or any(type(l) not in (Linear, ReLU, Identity) for l in self.layers):
+            return None
+        if any(l.engine is not linears[0].engine for l in linears):
+            return None
+        if any(a.output_size != b.input_size for a, b in zip(linears, linears[1:])):
+            return None  # the layer-by-layer pass raises the shape error where the reference panics
+        self._plan = _Plan(self.layers)
+        return self._plan
+
+    def _drop_plan(self):
+        if self._plan is not None:
+            self._plan.flush()
+            self._plan = None
 
     @classmethod
     def new(cls, layers):
         return cls(layers)
 
     def push(self, layer):
+        self._drop_plan()
         self.layers.append(layer)
 
     push_box = push
 
     def insert(self, index, layer):
+        self._drop_plan()
         self.layers.insert(index, layer)
 
     insert_box = insert
@@ -263,6 +408,7 @@ class Sequential(Module):
     def remove(self, index):
         if index >= len(self.layers):
             return None
+        self._drop_plan()
         return self.layers.pop(index)
 
     def _next_real(self, i):
@@ -278,6 +424,9 @@ class Sequential(Module):
         return -1
 
     def forward(self, input):
+        plan = self._compiled()
+        if plan is not None:
+            return plan.forward(input)
         x = input
         skip = set()
         for i, layer in enumerate(self.layers):
@@ -294,6 +443,8 @@ class Sequential(Module):
         return x
 
     def backward(self, gradient):
+        if self._plan is not None and self._plan.valid_for(self.layers):
+            return self._plan.backward(gradient)
         g = gradient
         skip = set()
         for i in range(len(self.layers) - 1, -1, -1):

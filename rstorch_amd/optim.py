@@ -22,6 +22,11 @@ class SGD(Optimizer):
         return cls(lr)
 
     def step(self, module):
+        # a compiled Sequential that still owes its backward pass runs it with this update inside
+        # the weight-gradient launches; the bits are those of the two passes apart
+        plan = getattr(module, "_plan", None)
+        if type(self) is SGD and plan is not None and plan.valid_for(module.layers) and plan.step_sgd(self.lr):
+            return
         params = list(module.parameters())
         if not params:
             return
