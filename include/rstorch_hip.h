@@ -123,6 +123,14 @@ int rst_softmax_backward(rst_engine* engine, const double* grad, const double* o
 int rst_cross_entropy(rst_engine* engine, const double* pred, const double* truth,
                       double* grad_out, double* prob_out, size_t rows, size_t cols,
                       double* host_loss);
+/* rst_cross_entropy with host_loss, and rst_accuracy(pred, truth) (src/utils.rs:55-65) with it: what
+ * the README loop asks for back to back (README.md:66-67), answered after ONE wait.  A batch that a
+ * single workgroup handles (up to 64 rows of up to 64 logits, 16 rows of up to 512) is counted by
+ * the cross-entropy launch itself; otherwise the arg-max launch follows on the stream.  Same loss
+ * bits as rst_cross_entropy, same count as rst_accuracy. */
+int rst_cross_entropy_accuracy(rst_engine* engine, const double* pred, const double* truth,
+                               double* grad_out, size_t rows, size_t cols, double* host_loss,
+                               double* host_accuracy);
 /* The loss of the latest rst_cross_entropy on this engine; waits for it.  RST_ERR_NAN if a
  * logit was NaN. */
 int rst_loss_value(rst_engine* engine, double* host_loss);
@@ -240,8 +248,8 @@ int rst_model_backward(rst_model* model, const double* grad, int need_input_grad
  * input gradient (the README loop drops it).  apply_sgd != 0 also runs SGD::step(lr): inside the
  * weight-gradient launches (see rst_model_fuse_sgd), i.e. `model.backward(g); optim.step(&mut model)`
  * as one pass with the same bits as the two calls apart.
- * Both record their launches into a HIP graph per distinct set of addresses and replay it
- * afterwards, like rst_model_train_step. */
+ * Both launch plainly (no recorded graph): their caller reads the loss between them, so the first
+ * kernel of each pass should start as soon as the call is made. */
 int rst_model_forward_to(rst_model* model, const double* x, size_t batch, double* logits_out);
 int rst_model_backward_to(rst_model* model, const double* grad, double* input_grad_out, int apply_sgd,
                           double lr);

@@ -83,6 +83,7 @@ SIGNATURES = {
     "rst_softmax_forward": [_vp, _dp, _dp, _sz, _sz, _i32],
     "rst_softmax_backward": [_vp, _dp, _dp, _dp, _sz, _sz],
     "rst_cross_entropy": [_vp, _dp, _dp, _dp, _dp, _sz, _sz, c_double_p],
+    "rst_cross_entropy_accuracy": [_vp, _dp, _dp, _dp, _sz, _sz, c_double_p, c_double_p],
     "rst_cross_entropy_static": [_vp, _dp, _dp, _dp, _sz, _sz, c_double_p],
     "rst_loss_value": [_vp, c_double_p],
     "rst_sgd_step": [_vp, c_void_pp, c_void_pp, c_size_p, _sz, _dbl],

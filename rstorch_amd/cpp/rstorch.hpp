@@ -6,11 +6,21 @@
 // Where the reference panics (unwrap on a consumed cache, shape mismatch, NaN in softmax) this
 // header throws rstorch::Panic.  Array2 is a dense row-major f64 matrix whose storage lives in
 // HBM; moving it between layers moves a handle, not data.  Header only; link librstorch_hip.so.
+//
+// A Sequential made only of Identity / Linear / ReLU layers is compiled on its first forward: a
+// device model (rst_model) is built over the layer list, the layers' parameters move into its arena
+// (the layers keep views), forward becomes one call, and backward launches nothing until
+// its results are needed: SGD::step(model) runs it with the update inside the weight-gradient
+// launches (the README loop then issues the launches of rst_model_train_step), reading a gradient
+// through parameters() or keeping the returned input gradient runs it on its own first.  Everything a
+// caller can observe is what the layer-by-layer path computes.  push / insert / remove drop the
+// compiled form.
 #pragma once
 
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <functional>
 #include <initializer_list>
 #include <memory>
 #include <random>
@@ -53,15 +63,41 @@ class Engine {
 
 // ---- Array2 (ndarray::Array2<f64> of the reference, src/module/mod.rs:42-49) ----------------
 class Array2 {
+ public:
+  // The device memory behind one or more Array2 handles.  Two kinds fill `ptr` in late: gradient
+  // views of a compiled Sequential (before_access first runs the backward pass that is still owed)
+  // and the input gradient that Sequential::backward returns (resolver computes it when somebody
+  // looks).  Every access goes through Array2::data().
   struct Storage {
     std::shared_ptr<Engine> engine;
     double* ptr = nullptr;
+    bool owns = true;                        // false: a view into memory that `keepalive` owns
+    // true for the arrays the library rewrites in place (a layer's parameters, which SGD::step
+    // updates, and its gradients, which every backward overwrites).  Everything else is written once,
+    // by the call that produced it, and never again: such an array is a value, and clone() may hand
+    // out a second handle to the same memory instead of copying it.
+    bool rewritten_in_place = false;
+    std::shared_ptr<void> keepalive;
+    std::function<void()> before_access;
+    std::function<void(Storage&)> resolver;  // runs once
+    double* get() {
+      if (resolver) {
+        auto r = std::move(resolver);
+        resolver = nullptr;
+        r(*this);
+      }
+      if (before_access) before_access();
+      return ptr;
+    }
+    void materialise(size_t count) {
+      if (rst_malloc(engine->handle(), count, &ptr) != RST_OK) throw Panic(RST_ERR_OUT_OF_MEMORY, rst_last_error());
+      owns = true;
+    }
     ~Storage() {
-      if (ptr) rst_free(engine->handle(), ptr);
+      if (ptr && owns) rst_free(engine->handle(), ptr);
     }
   };
 
- public:
   Array2() = default;
   Array2(size_t rows, size_t cols, std::shared_ptr<Engine> e = Engine::global())
       : rows_(rows), cols_(cols), s_(std::make_shared<Storage>()) {
@@ -110,18 +146,60 @@ class Array2 {
     return a;
   }
 
+  // a view of `rows x cols` doubles at `ptr`, owned by whatever `keepalive` keeps alive
+  static Array2 view(std::shared_ptr<Engine> e, double* ptr, size_t rows, size_t cols, std::shared_ptr<void> keepalive,
+                     std::function<void()> before_access = nullptr) {
+    Array2 a;
+    a.rows_ = rows; a.cols_ = cols;
+    a.s_ = std::make_shared<Storage>();
+    a.s_->engine = std::move(e);
+    a.s_->ptr = ptr;
+    a.s_->owns = false;
+    a.s_->keepalive = std::move(keepalive);
+    a.s_->before_access = std::move(before_access);
+    a.s_->rewritten_in_place = true;  // views are how parameters and gradients of an arena are handed out
+    return a;
+  }
+  // an array whose contents `resolver` produces the first time somebody asks for them
+  static Array2 deferred(std::shared_ptr<Engine> e, size_t rows, size_t cols, std::function<void(Storage&)> resolver) {
+    Array2 a;
+    a.rows_ = rows; a.cols_ = cols;
+    a.s_ = std::make_shared<Storage>();
+    a.s_->engine = std::move(e);
+    a.s_->owns = false;
+    a.s_->resolver = std::move(resolver);
+    return a;
+  }
+
   size_t nrows() const { return rows_; }
   size_t ncols() const { return cols_; }
   size_t size() const { return rows_ * cols_; }
   bool empty_handle() const { return !s_; }
-  double* data() const { return s_ ? s_->ptr : nullptr; }
+  double* data() const { return s_ ? s_->get() : nullptr; }
   rst_engine* engine() const { return s_->engine->handle(); }
+  const std::shared_ptr<Engine>& engine_ref() const { return s_->engine; }
+  const std::shared_ptr<Storage>& storage() const { return s_; }
   bool same_shape(const Array2& o) const { return rows_ == o.rows_ && cols_ == o.cols_; }
 
+  // The reference clones arrays wherever a callee consumes its argument (README.md:66:
+  // loss.forward(pred.clone(), y.clone())).  An array that nothing rewrites is a value: its clone is
+  // a second handle to the same memory (no copy is launched, and the two stay equal because
+  // neither can change).  Parameters and gradients are copied.
   Array2 clone() const {
+    if (!s_->rewritten_in_place) {
+      (void)data();  // a deferred array is computed before it is shared
+      return *this;
+    }
+    return deep_clone();
+  }
+  Array2 deep_clone() const {
     Array2 out(rows_, cols_, s_->engine);
     check(rst_copy(engine(), out.data(), data(), size()));
     return out;
+  }
+  Array2& mark_rewritten_in_place() {
+    s_->rewritten_in_place = true;
+    return *this;
   }
   std::vector<double> to_host() const {
     std::vector<double> h(size());
@@ -302,6 +380,10 @@ class Linear : public Module {
         bias_(init.bias(input_size, output_size)) {
     if (weight_.nrows() != out_ || weight_.ncols() != in_) throw Panic(RST_ERR_SHAPE, "init.weight shape");
     if (bias_.nrows() != 1 || bias_.ncols() != out_) throw Panic(RST_ERR_SHAPE, "init.bias shape");
+    // the optimiser updates them in place: they must not share memory with what the initialiser
+    // returned (which may hand out the same array twice)
+    weight_ = weight_.deep_clone().mark_rewritten_in_place();
+    bias_ = bias_.deep_clone().mark_rewritten_in_place();
   }
   static Linear new_with_kernel(size_t i, size_t o, const InitParameters& init) { return Linear(i, o, init); }
 
@@ -323,8 +405,8 @@ class Linear : public Module {
     Array2 x = std::move(prev_input_);
     if (gradient.nrows() != x.nrows() || gradient.ncols() != out_) throw Panic(RST_ERR_SHAPE, "Linear: gradient shape");
     if (!has_grad_) {
-      grad_weight_ = Array2(out_, in_);
-      grad_bias_ = Array2(1, out_);
+      grad_weight_ = Array2(out_, in_).mark_rewritten_in_place();
+      grad_bias_ = Array2(1, out_).mark_rewritten_in_place();
       has_grad_ = true;
     }
     Array2 gx(x.nrows(), in_);
@@ -347,34 +429,194 @@ class Linear : public Module {
   Array2& bias() { return bias_; }
   Array2& grad_weight() { return grad_weight_; }
   Array2& grad_bias() { return grad_bias_; }
+  size_t input_size() const { return in_; }
+  size_t output_size() const { return out_; }
+
+  // A compiled Sequential moves the parameters into its arena: the layer keeps views, `home` names
+  // the compiled form (an opaque token that also keeps the arena alive).
+  const std::shared_ptr<void>& home() const { return home_; }
+  bool has_gradient() const { return has_grad_; }
+  void rehome(std::shared_ptr<void> home, Array2 w, Array2 b, Array2 gw, Array2 gb) {
+    weight_ = std::move(w); bias_ = std::move(b);
+    grad_weight_ = std::move(gw); grad_bias_ = std::move(gb);
+    home_ = std::move(home);
+  }
+  void mark_gradient() { has_grad_ = true; }
 
  private:
   size_t in_, out_;
   Array2 weight_, bias_, prev_input_, grad_weight_, grad_bias_;
   bool has_input_ = false, has_grad_ = false;
+  std::shared_ptr<void> home_;
 };
+
+// ---- the compiled form of a Sequential of Identity / Linear / ReLU ------------------------------
+namespace detail {
+
+class Plan : public std::enable_shared_from_this<Plan> {
+ public:
+  // which object `home` tokens of this plan point at
+  static std::shared_ptr<Plan> create(const std::vector<std::unique_ptr<Module>>& layers) {
+    std::shared_ptr<Plan> p(new Plan());
+    p->build(layers);
+    return p;
+  }
+  ~Plan() {
+    if (model_) rst_model_destroy(model_);
+  }
+  bool valid_for(const std::vector<std::unique_ptr<Module>>& layers) const {
+    if (layers.size() != key_.size()) return false;
+    for (size_t i = 0; i < layers.size(); ++i)
+      if (layers[i].get() != key_[i]) return false;
+    for (Linear* l : linears_)
+      if (l->home().get() != this) return false;
+    return true;
+  }
+
+  Array2 forward(Array2 input) {
+    flush();  // a backward pass nobody looked at would otherwise read the new activations
+    if (input.ncols() != in_width_) throw Panic(RST_ERR_SHAPE, "Linear: input width");
+    Array2 out(input.nrows(), out_width_, engine_);
+    check(rst_model_forward_to(model_, input.data(), input.nrows(), out.data()));
+    x_ = std::move(input);
+    out_ = out;
+    live_ = true;
+    return out;
+  }
+
+  Array2 backward(Array2 gradient) {
+    if (!live_ || pending_) throw Panic(RST_ERR_STATE, "Sequential::backward without a forward");
+    if (gradient.nrows() != x_.nrows() || gradient.ncols() != out_width_) throw Panic(RST_ERR_SHAPE, "Linear: gradient shape");
+    std::weak_ptr<Plan> self = shared_from_this();
+    Array2 gin = Array2::deferred(engine_, x_.nrows(), in_width_, [self](Array2::Storage& s) {
+      if (auto p = self.lock()) p->resolve_input_gradient(s);
+      if (!s.ptr) throw Panic(RST_ERR_STATE, "this input gradient was never computed");
+    });
+    grad_ = std::move(gradient);
+    gin_ = gin.storage();
+    pending_ = true;
+    for (Linear* l : linears_) l->mark_gradient();
+    return gin;
+  }
+
+  // runs the backward pass that is still owed, without an optimiser step
+  void flush() {
+    if (pending_) run(false, 0.0);
+  }
+  // backward + SGD::step in one pass, if a backward is still owed
+  bool step_sgd(double lr) {
+    if (!pending_) return false;
+    run(true, lr);
+    return true;
+  }
+
+ private:
+  Plan() = default;
+
+  void build(const std::vector<std::unique_ptr<Module>>& layers) {
+    std::vector<int> kinds;
+    std::vector<size_t> in, out;
+    for (auto& l : layers) {
+      key_.push_back(l.get());
+      kinds.push_back(l->layer_kind());
+      Linear* lin = l->layer_kind() == RST_LAYER_LINEAR ? static_cast<Linear*>(l.get()) : nullptr;
+      in.push_back(lin ? lin->input_size() : 0);
+      out.push_back(lin ? lin->output_size() : 0);
+      if (lin) linears_.push_back(lin);
+    }
+    engine_ = linears_[0]->weight().engine_ref();
+    in_width_ = linears_.front()->input_size();
+    out_width_ = linears_.back()->output_size();
+    check(rst_model_create(engine_->handle(), kinds.data(), in.data(), out.data(), kinds.size(), &model_));
+    std::shared_ptr<Plan> self = shared_from_this();
+    std::weak_ptr<Plan> weak = self;
+    auto owed = [weak] { if (auto p = weak.lock()) p->flush(); };
+    for (size_t i = 0; i < linears_.size(); ++i) {
+      Linear* l = linears_[i];
+      double *w, *gw, *b, *gb;
+      size_t r, c;
+      check(rst_model_parameter(model_, 2 * i, &w, &gw, &r, &c));
+      check(rst_model_parameter(model_, 2 * i + 1, &b, &gb, &r, &c));
+      const size_t nw = l->input_size() * l->output_size(), nb = l->output_size();
+      // (reading the old arrays first runs whatever another compiled Sequential still owes them)
+      check(rst_copy(engine_->handle(), w, l->weight().data(), nw));
+      check(rst_copy(engine_->handle(), b, l->bias().data(), nb));
+      if (l->has_gradient()) {  // gradients computed before the move stay readable
+        check(rst_copy(engine_->handle(), gw, l->grad_weight().data(), nw));
+        check(rst_copy(engine_->handle(), gb, l->grad_bias().data(), nb));
+      }
+      l->rehome(self, Array2::view(engine_, w, l->output_size(), l->input_size(), self),
+                Array2::view(engine_, b, 1, l->output_size(), self),
+                Array2::view(engine_, gw, l->output_size(), l->input_size(), self, owed),
+                Array2::view(engine_, gb, 1, l->output_size(), self, owed));
+    }
+  }
+
+  void resolve_input_gradient(Array2::Storage& s) {
+    if (pending_ && gin_.lock().get() == &s) run(false, 0.0);
+  }
+
+  void run(bool apply_sgd, double lr) {
+    pending_ = false;
+    std::shared_ptr<Array2::Storage> gin = gin_.lock();  // still wanted by somebody?
+    gin_.reset();
+    if (gin) {
+      gin->resolver = nullptr;
+      gin->materialise(x_.nrows() * in_width_);
+    }
+    Array2 g = std::move(grad_);
+    check(rst_model_backward_to(model_, g.data(), gin ? gin->ptr : nullptr, apply_sgd ? 1 : 0, lr));
+    x_ = Array2();
+    out_ = Array2();  // the caches are consumed
+    live_ = false;
+  }
+
+  rst_model* model_ = nullptr;
+  std::shared_ptr<Engine> engine_;
+  std::vector<const Module*> key_;
+  std::vector<Linear*> linears_;
+  size_t in_width_ = 0, out_width_ = 0;
+  Array2 x_, out_, grad_;  // the forward pass whose caches are live; the gradient of the owed backward
+  std::weak_ptr<Array2::Storage> gin_;  // the input gradient that backward returned, if still held
+  bool live_ = false, pending_ = false;
+};
+
+}  // namespace detail
 
 // ---- Sequential: src/module/sequential.rs -------------------------------------------------------
 class Sequential : public Module {
  public:
   Sequential() = default;
   explicit Sequential(std::vector<std::unique_ptr<Module>> layers) : layers_(std::move(layers)) {}
-  template <class M> void push(M layer) { layers_.push_back(std::make_unique<M>(std::move(layer))); }
-  template <class M> void insert(size_t index, M layer) {
-    layers_.insert(layers_.begin() + index, std::make_unique<M>(std::move(layer)));
+  template <class M> void push(M layer) { push_box(std::make_unique<M>(std::move(layer))); }
+  template <class M> void insert(size_t index, M layer) { insert_box(index, std::make_unique<M>(std::move(layer))); }
+  void push_box(std::unique_ptr<Module> l) {
+    drop_plan();
+    layers_.push_back(std::move(l));
   }
-  void push_box(std::unique_ptr<Module> l) { layers_.push_back(std::move(l)); }
-  void insert_box(size_t index, std::unique_ptr<Module> l) { layers_.insert(layers_.begin() + index, std::move(l)); }
+  void insert_box(size_t index, std::unique_ptr<Module> l) {
+    drop_plan();
+    layers_.insert(layers_.begin() + index, std::move(l));
+  }
   size_t len() const { return layers_.size(); }
   bool is_empty() const { return layers_.empty(); }
   std::unique_ptr<Module> remove(size_t index) {
     if (index >= layers_.size()) return nullptr;
+    drop_plan();
     auto l = std::move(layers_[index]);
     layers_.erase(layers_.begin() + index);
     return l;
   }
+  // false: always run layer by layer, one call per layer
+  void set_compile(bool enabled) {
+    if (!enabled) drop_plan();
+    compile_ = enabled;
+  }
+  // backward + SGD::step in one pass if this Sequential is compiled and still owes a backward pass
+  bool step_sgd(double lr) { return plan_ && plan_->valid_for(layers_) && plan_->step_sgd(lr); }
 
   Array2 forward(Array2 input) override {
+    if (detail::Plan* plan = compiled()) return plan->forward(std::move(input));
     const int n = int(layers_.size());
     for (int i = 0; i < n; ++i) {
       Module* l = layers_[i].get();
@@ -395,6 +637,7 @@ class Sequential : public Module {
   }
 
   Array2 backward(Array2 gradient) override {
+    if (plan_ && plan_->valid_for(layers_)) return plan_->backward(std::move(gradient));
     const int n = int(layers_.size());
     for (int i = n - 1; i >= 0; --i) {
       Module* l = layers_[i].get();
@@ -427,6 +670,35 @@ class Sequential : public Module {
   }
 
  private:
+  // the compiled form, built on demand; null when the layer list has a layer it cannot hold
+  detail::Plan* compiled() {
+    if (!compile_) return nullptr;
+    if (plan_ && plan_->valid_for(layers_)) return plan_.get();
+    drop_plan();
+    size_t width = 0;
+    bool any = false;
+    for (auto& l : layers_) {
+      const int kind = l->layer_kind();
+      if (kind != RST_LAYER_IDENTITY && kind != RST_LAYER_RELU && kind != RST_LAYER_LINEAR) return nullptr;
+      if (kind == RST_LAYER_LINEAR) {
+        auto* lin = static_cast<Linear*>(l.get());
+        // (a width mismatch is left to the layer-by-layer pass, which panics where the reference does)
+        if (any && lin->input_size() != width) return nullptr;
+        width = lin->output_size();
+        any = true;
+      }
+    }
+    if (!any) return nullptr;
+    plan_ = detail::Plan::create(layers_);
+    return plan_.get();
+  }
+  void drop_plan() {
+    if (plan_) plan_->flush();
+    plan_.reset();
+  }
+  std::shared_ptr<detail::Plan> plan_;
+  bool compile_ = true;
+
   int next_real(int i) const {
     for (int j = i + 1; j < int(layers_.size()); ++j)
       if (layers_[j]->layer_kind() != RST_LAYER_IDENTITY) return j;
@@ -456,14 +728,37 @@ class Loss {
   virtual Array2 backward() = 0;
 };
 
+namespace detail {
+// The README loop asks for accuracy(pred, y) right after loss.forward(pred.clone(), y.clone()).  The
+// loss computes the arg-max agreement of its two arrays along the way (one launch and one wait for
+// both numbers) and leaves it here; accuracy() takes it when it is called on the same memory.  Sound
+// because such arrays are values: a clone of an array that nothing rewrites is a second handle to the
+// same memory, and neither handle can change it.
+struct AccuracyMemo {
+  std::weak_ptr<Array2::Storage> pred, truth;
+  double value = 0.0;
+};
+inline AccuracyMemo& accuracy_memo() {
+  static thread_local AccuracyMemo memo;
+  return memo;
+}
+}  // namespace detail
+
 class CrossEntropyLoss : public Loss {
  public:
   double forward(Array2 pred, Array2 truth) override {
     if (!pred.same_shape(truth)) throw Panic(RST_ERR_SHAPE, "CrossEntropyLoss: pred/truth shapes");
     Array2 g(pred.nrows(), pred.ncols());
-    double loss = 0.0;
-    check(rst_cross_entropy(pred.engine(), pred.data(), truth.data(), g.data(), nullptr, pred.nrows(),
-                            pred.ncols(), &loss));
+    double loss = 0.0, acc = 0.0;
+    check(rst_cross_entropy_accuracy(pred.engine(), pred.data(), truth.data(), g.data(), pred.nrows(),
+                                     pred.ncols(), &loss, &acc));
+    detail::AccuracyMemo& memo = detail::accuracy_memo();
+    memo.pred.reset();
+    if (!pred.storage()->rewritten_in_place && !truth.storage()->rewritten_in_place) {
+      memo.pred = pred.storage();
+      memo.truth = truth.storage();
+      memo.value = acc;
+    }
     grad_ = std::move(g);
     has_ = true;
     return loss;
@@ -490,6 +785,10 @@ class SGD : public Optimizer {
  public:
   explicit SGD(double lr) : lr_(lr) {}
   void step(Module& module) override {
+    // a compiled Sequential that still owes its backward pass runs it with this update inside the
+    // weight-gradient launches; the bits are those of the two passes apart
+    if (auto* seq = dynamic_cast<Sequential*>(&module))
+      if (seq->step_sgd(lr_)) return;
     Parameters ps = module.parameters();
     if (ps.size() == 0) return;
     std::vector<double*> parm;
@@ -514,6 +813,9 @@ class SGD : public Optimizer {
 namespace utils {
 inline double accuracy(const Array2& pred, const Array2& truth) {
   if (!pred.same_shape(truth)) throw Panic(RST_ERR_SHAPE, "accuracy: shapes");
+  const detail::AccuracyMemo& memo = detail::accuracy_memo();
+  if (pred.storage() && memo.pred.lock() == pred.storage() && memo.truth.lock() == truth.storage())
+    return memo.value;  // the loss has already counted these two arrays
   double acc = 0.0;
   check(rst_accuracy(pred.engine(), pred.data(), truth.data(), pred.nrows(), pred.ncols(), &acc));
   return acc;

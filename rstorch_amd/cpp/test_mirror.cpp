@@ -118,6 +118,67 @@ int main() {
       Array2 bad = Array2::full(2, 3, std::nan(""));
       EXPECT(panics([&] { CrossEntropyLoss().forward(bad, Array2::zeros(2, 3)); }));
     }
+    {  // the compiled Sequential (forward graph, backward deferred to the optimiser step) against the
+       // same network run layer by layer: every observable value, bit for bit
+      struct Given : InitParameters {
+        Array2 w;
+        explicit Given(Array2 a) : w(std::move(a)) {}
+        Array2 weight(size_t, size_t) const override { return w.clone(); }
+      };
+      auto make = [&](bool compile) {
+        Sequential m = sequential(Identity(), Linear::new_with_kernel(24, 40, Given(Array2::normal(40, 24, 9, 1, 0.0, 0.2))),
+                                  ReLU(), Linear::new_with_kernel(40, 40, Given(Array2::normal(40, 40, 9, 2, 0.0, 0.15))),
+                                  ReLU(), Linear::new_with_kernel(40, 6, Given(Array2::normal(6, 40, 9, 3, 0.0, 0.15))));
+        m.set_compile(compile);
+        return m;
+      };
+      Sequential fast = make(true), slow = make(false);
+      CrossEntropyLoss lf, ls;
+      SGD of(0.1), os(0.1);
+      auto same_parameters = [&] {
+        Parameters pf = fast.parameters(), ps = slow.parameters();
+        bool ok = pf.size() == ps.size();
+        for (size_t i = 0; ok && i < pf.size(); ++i)
+          ok = pf.iter()[i].parm->to_host() == ps.iter()[i].parm->to_host() &&
+               pf.iter()[i].grad->to_host() == ps.iter()[i].grad->to_host();
+        return ok;
+      };
+      EXPECT(panics([&] { fast.backward(Array2::ones(4, 6)); }));
+      EXPECT(panics([&] { fast.parameters(); }));
+      for (int step = 0; step < 6; ++step) {
+        Array2 x = Array2::normal(48, 24, 5, 10 + step % 2, 0.0, 1.0), y = Array2::one_hot(48, 6, 5, 20 + step % 2);
+        Array2 pf = fast.forward(x), ps = slow.forward(x);
+        EXPECT(pf.to_host() == ps.to_host());
+        EXPECT(lf.forward(pf.clone(), y.clone()) == ls.forward(ps.clone(), y.clone()));
+        if (step == 1) {         // the input gradient kept and read before the step
+          Array2 gf = fast.backward(lf.backward()), gs = slow.backward(ls.backward());
+          EXPECT(gf.to_host() == gs.to_host());
+        } else if (step == 2) {  // kept, read after the step: computed with the weights of before
+          Array2 gf = fast.backward(lf.backward()), gs = slow.backward(ls.backward());
+          of.step(fast); os.step(slow);
+          EXPECT(gf.to_host() == gs.to_host());
+          EXPECT(same_parameters());
+          continue;
+        } else {
+          fast.backward(lf.backward()); slow.backward(ls.backward());
+        }
+        if (step == 3) EXPECT(same_parameters());  // gradients read between backward and step
+        if (step == 4) EXPECT(panics([&] { fast.backward(Array2::ones(48, 6)); }));  // consumed
+        of.step(fast); os.step(slow);
+        EXPECT(same_parameters());
+      }
+      // the layer list changes: the compiled form is dropped, the weights stay with their layers
+      fast.push(ReLU()); slow.push(ReLU());
+      fast.insert(1, Identity()); slow.insert(1, Identity());
+      Array2 x = Array2::normal(8, 24, 5, 30, 0.0, 1.0);
+      EXPECT(fast.forward(x).to_host() == slow.forward(x).to_host());
+      Array2 gf = fast.backward(Array2::ones(8, 6)), gs = slow.backward(Array2::ones(8, 6));
+      EXPECT(gf.to_host() == gs.to_host());
+      EXPECT(same_parameters());
+      std::unique_ptr<Module> taken = fast.remove(2);  // the first Linear leaves with its trained weights
+      std::unique_ptr<Module> taken_slow = slow.remove(2);
+      EXPECT(static_cast<Linear*>(taken.get())->weight().to_host() == static_cast<Linear*>(taken_slow.get())->weight().to_host());
+    }
   } catch (const Panic& p) {
     std::printf("unexpected panic: %s\n", p.what());
     return 2;

@@ -117,22 +117,32 @@ unsigned long long sgd_blocks_for(unsigned long long count);
 // LossMirror: device-visible addresses of pinned host words that receive the loss and flags[1]
 // as well (written by the thread that finishes the loss), so that the host can read them after a
 // stream synchronisation without a copy in between.  Null members: no mirror.
+// ticket: a third pinned word that the same thread writes last, behind a system-scope fence, with
+// ticket_value: the host can then wait for exactly this result by polling the word instead of
+// synchronising the stream.  hits: when set, a cross entropy whose whole batch sits in one workgroup
+// also counts the rows whose first arg-max agrees between logits and truth (src/utils.rs:44-65) and
+// stores the count there; launch_softmax_ce reports whether it did.
 struct LossMirror {
   double* loss = nullptr;
   int* flags = nullptr;
+  unsigned long long* ticket = nullptr;
+  unsigned long long ticket_value = 0;
+  unsigned long long* hits = nullptr;
 };
 int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* grad_out,
                       double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
-                      size_t cols, LossMirror mirror = LossMirror());
+                      size_t cols, LossMirror mirror = LossMirror(), bool* hits_done = nullptr);
 int launch_softmax_columns(hipStream_t s, const double* z, double* out, int* flags, size_t rows,
                            size_t cols);
 int launch_softmax_jacobian(hipStream_t s, double* jac, size_t cols);
 // hits[0] = number of rows whose first arg-max agrees
 // hits_mirror: device-visible address of a pinned host word; *mirrored tells whether the count
 // was also written there (small inputs, counted by one workgroup without atomics)
+// ticket / ticket_value: as in LossMirror, written after the mirrored count
 int launch_accuracy(hipStream_t s, const double* pred, const double* truth, size_t rows,
                     size_t cols, unsigned long long* hits, unsigned long long* hits_mirror = nullptr,
-                    bool* mirrored = nullptr);
+                    bool* mirrored = nullptr, unsigned long long* ticket = nullptr,
+                    unsigned long long ticket_value = 0);
 
 int launch_fill_uniform(hipStream_t s, double* dst, size_t n, uint64_t seed, uint64_t stream,
                         double lo, double hi);
@@ -159,6 +169,15 @@ struct rst_engine {
   double* hd_loss = nullptr;
   int* hd_flags = nullptr;
   unsigned long long* hd_hits = nullptr;
+  // results are announced by a ticket: kernels that finish a scalar write the number they were
+  // given into a pinned word last, and the host polls that word (a few microseconds sooner than a
+  // stream synchronisation returns).  Tickets only grow.  loss_ticket: the ticket of the latest
+  // loss, 0 when that loss was enqueued without one (recorded into a graph, whose replays would all
+  // write the same number).
+  unsigned long long* h_ticket = nullptr;   // pinned
+  unsigned long long* hd_ticket = nullptr;  // the same word as the device addresses it
+  unsigned long long tickets_issued = 0;
+  unsigned long long loss_ticket = 0;
   bool loss_valid = false;
   // split-K scratch of the contraction kernels (fixed size, allocated with the engine)
   double* d_gemm_ws = nullptr;
@@ -179,12 +198,17 @@ struct rst_engine {
 
 namespace rst {
 int engine_activate(rst_engine* e);
+// waits until the kernel that was given `ticket` has written its results to the pinned words
+// (ticket 0: until the stream has drained)
+int engine_wait_ticket(rst_engine* e, unsigned long long ticket);
 int engine_reserve_row_loss(rst_engine* e, size_t rows);
 // looks up, once per device, the address of the fixed scratch behind rst_cross_entropy_static
 int static_scratch_setup(int device, hipStream_t stream);
 // row_loss: [rows] scratch of the caller, or NULL for the engine's own (which is reallocated when
 // it grows: only for launches that are not recorded into a graph)
+// hits_done != NULL: the arg-max agreement count is wanted as well (into the engine's pinned hit
+// word); *hits_done tells whether the cross-entropy launch took it
 int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, const double* truth,
                          double* grad_out, double* prob_out, size_t rows, size_t cols,
-                         double* host_loss);
+                         double* host_loss, bool* hits_done = nullptr);
 }  // namespace rst

@@ -1,6 +1,8 @@
 // Engine: device, stream, error reporting, device memory and stream timing.
 #include "common.h"
 
+#include <immintrin.h>
+
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -41,6 +43,18 @@ void clear_error() {
 int engine_activate(rst_engine* e) {
   if (!e) return fail(RST_ERR_INVALID_ARGUMENT, "engine is null");
   RST_HIP(hipSetDevice(e->device));
+  return RST_OK;
+}
+
+int engine_wait_ticket(rst_engine* e, unsigned long long ticket) {
+  if (ticket != 0) {
+    // about 100 us of polling; a result that takes longer is waited for the ordinary way
+    for (int i = 0; i < 4000; ++i) {
+      if (__atomic_load_n(e->h_ticket, __ATOMIC_ACQUIRE) >= ticket) return RST_OK;
+      _mm_pause();
+    }
+  }
+  RST_HIP(hipStreamSynchronize(e->stream));
   return RST_OK;
 }
 
@@ -103,6 +117,10 @@ int rst_engine_create(int device, rst_engine** out) {
   if (err == hipSuccess) err = hipHostMalloc(&e->h_flags, 4 * sizeof(int), hipHostMallocDefault);
   if (err == hipSuccess)
     err = hipHostMalloc(&e->h_hits, sizeof(unsigned long long), hipHostMallocDefault);
+  if (err == hipSuccess)
+    err = hipHostMalloc(&e->h_ticket, sizeof(unsigned long long), hipHostMallocDefault);
+  if (err == hipSuccess) err = hipHostGetDevicePointer((void**)&e->hd_ticket, e->h_ticket, 0);
+  if (err == hipSuccess) *e->h_ticket = 0;
   if (err == hipSuccess) err = hipHostGetDevicePointer((void**)&e->hd_loss, e->h_loss, 0);
   if (err == hipSuccess) err = hipHostGetDevicePointer((void**)&e->hd_flags, e->h_flags, 0);
   if (err == hipSuccess) err = hipHostGetDevicePointer((void**)&e->hd_hits, e->h_hits, 0);
@@ -144,6 +162,7 @@ int rst_engine_destroy(rst_engine* e) {
   if (e->h_loss) (void)hipHostFree(e->h_loss);
   if (e->h_flags) (void)hipHostFree(e->h_flags);
   if (e->h_hits) (void)hipHostFree(e->h_hits);
+  if (e->h_ticket) (void)hipHostFree(e->h_ticket);
   if (e->stream) (void)hipStreamDestroy(e->stream);
   delete e;
   return RST_OK;

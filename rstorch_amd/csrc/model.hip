@@ -67,7 +67,6 @@ struct rst_model {
   // (a buffer shared through the engine could be reallocated by another caller between two replays)
   double* row_loss = nullptr;
   const double* logits = nullptr;
-  const double* forward_x = nullptr;  // the input of the forward whose caches are live
   // state machine (mirrors the Option::take() caches of the reference)
   bool forward_valid = false;
   bool loss_grad_valid = false;
@@ -75,24 +74,17 @@ struct rst_model {
   // the captured training step (one graph launch instead of ~10 kernel launches)
   // (a few graphs are kept: a staged input pipeline alternates between its slots' buffers)
   bool graph_enabled = true;
-  // what a recorded graph was recorded for: every address its kernels were given, the batch and
-  // the learning rate.  kind: 0 the whole step (x, truth), 1 forward into a caller's array (x, out),
-  // 2 backward from a caller's gradient (grad, input-gradient destination, and the forward's x and
-  // out, which the weight gradient of the first layer and the mask of the last ReLU read)
+  // what a recorded graph was recorded for: the addresses its kernels were given, the batch and
+  // the learning rate
   struct StepGraph {
     hipGraphExec_t exec;
-    int kind;
     const double* x;
     const double* truth;
-    const double* aux0;
-    const double* aux1;
     size_t batch;
     double lr;
-    int flags;
     unsigned long long last_use;
-    bool matches(int k, const double* a, const double* b, const double* c, const double* d, size_t n, double l,
-                 int f) const {
-      return kind == k && x == a && truth == b && aux0 == c && aux1 == d && batch == n && lr == l && flags == f;
+    bool matches(const double* a, const double* b, size_t n, double l) const {
+      return x == a && truth == b && batch == n && lr == l;
     }
   };
   std::vector<StepGraph> graphs;
@@ -218,12 +210,10 @@ int next_non_identity(const rst_model* m, int i) {
 // final_out != NULL: the last layer that computes anything writes there instead of into the model's
 // own buffer (the caller's array that Sequential::forward returns by value; backward reads it again
 // as the mask of a trailing ReLU, so it must stay as it is until then).
-// launch == false: only the bookkeeping of the pass (which tensor each layer keeps for backward) -
-// what a replayed graph leaves undone on the host.
-int do_forward(rst_model* m, const double* x, size_t batch, double* final_out = nullptr, bool launch = true) {
+int do_forward(rst_model* m, const double* x, size_t batch, double* final_out = nullptr) {
   rst_engine* e = m->engine;
   if (batch > (size_t)INT_MAX) return fail(RST_ERR_UNSUPPORTED, "batch too large");
-  if (launch) RST_TRY(reserve_activations(m, batch));
+  RST_TRY(reserve_activations(m, batch));
   m->batch = batch;
   const double* cur = x;
   const int n = (int)m->layers.size();
@@ -255,11 +245,9 @@ int do_forward(rst_model* m, const double* x, size_t batch, double* final_out = 
       const double flops = 2.0 * (double)batch * (double)l.in * (double)l.out;
       const double bytes = 8.0 * ((double)batch * l.in + (double)l.in * l.out + (double)batch * l.out);
       d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
-      if (launch) {
-        RST_TRY(prof_begin(m, RST_KERNEL_LINEAR_FORWARD, i, flops, bytes));
-        RST_TRY(launch_gemm(e->stream, d));
-        RST_TRY(prof_end(m));
-      }
+      RST_TRY(prof_begin(m, RST_KERNEL_LINEAR_FORWARD, i, flops, bytes));
+      RST_TRY(launch_gemm(e->stream, d));
+      RST_TRY(prof_end(m));
       cur = dest;
       if (fuse) {
         Layer& r = m->layers[nx];
@@ -272,16 +260,13 @@ int do_forward(rst_model* m, const double* x, size_t batch, double* final_out = 
       const size_t cnt = batch * l.width_in;
       l.input = cur;        // relu.rs:20 keeps the pre-activation
       l.mask_source = cur;
-      if (launch) {
-        RST_TRY(prof_begin(m, RST_KERNEL_RELU_FORWARD, i, 0.0, 16.0 * (double)cnt));
-        RST_TRY(launch_relu_forward(e->stream, cur, dest, cnt));
-        RST_TRY(prof_end(m));
-      }
+      RST_TRY(prof_begin(m, RST_KERNEL_RELU_FORWARD, i, 0.0, 16.0 * (double)cnt));
+      RST_TRY(launch_relu_forward(e->stream, cur, dest, cnt));
+      RST_TRY(prof_end(m));
       cur = dest;
     }
   }
   m->logits = cur;
-  m->forward_x = x;
   m->forward_valid = true;
   m->loss_grad_valid = false;
   return RST_OK;
@@ -740,7 +725,7 @@ int capture_graph(rst_model* m, rst_model::StepGraph key, Run run, hipGraphExec_
 // the recorded graph for `key`, if there is one
 hipGraphExec_t find_graph(rst_model* m, const rst_model::StepGraph& key) {
   for (auto& g : m->graphs)
-    if (g.matches(key.kind, key.x, key.truth, key.aux0, key.aux1, key.batch, key.lr, key.flags)) {
+    if (g.matches(key.x, key.truth, key.batch, key.lr)) {
       g.last_use = ++m->graph_clock;
       return g.exec;
     }
@@ -762,7 +747,7 @@ int rst_model_train_step(rst_model* m, const double* x, const double* truth, siz
   if (!x || !truth) return fail(RST_ERR_INVALID_ARGUMENT, "x or truth is null");
   if (batch == 0) return fail(RST_ERR_SHAPE, "training step on an empty batch");
   if (use_graphs(m)) {
-    const rst_model::StepGraph key{nullptr, 0, x, truth, nullptr, nullptr, batch, lr, 0, 0};
+    const rst_model::StepGraph key{nullptr, x, truth, batch, lr, 0};
     hipGraphExec_t exec = find_graph(m, key);
     if (!exec) RST_TRY(capture_graph(m, key, [&] { return run_step(m, x, truth, batch, lr); }, &exec));
     RST_HIP(hipGraphLaunch(exec, e->stream));
@@ -772,6 +757,7 @@ int rst_model_train_step(rst_model* m, const double* x, const double* truth, siz
     m->loss_grad_valid = false;
     m->grads_valid = true;
     e->loss_valid = true;
+    e->loss_ticket = 0;  // a replayed loss announces no ticket: its reader waits for the stream
   } else {
     RST_TRY(run_step(m, x, truth, batch, lr));
   }
@@ -779,20 +765,16 @@ int rst_model_train_step(rst_model* m, const double* x, const double* truth, siz
   return RST_OK;
 }
 
+// These two launch plainly, never from a recorded graph: their caller reads a scalar (the loss)
+// between them, so what counts is how soon the first kernel starts after the call, and a graph
+// launch of three or four small kernels starts later than the first of as many plain launches
+// (the README loop at batch 32 through the C++ mirror: 22.1 k steps/s with plain launches, 17.7 k
+// with one graph per pass; 6.4 k against 6.1 k at batch 8192).
 int rst_model_forward_to(rst_model* m, const double* x, size_t batch, double* logits_out) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
   m->chain_open = false;
-  rst_engine* e = m->engine;
-  RST_TRY(engine_activate(e));
+  RST_TRY(engine_activate(m->engine));
   if (batch && (!x || !logits_out)) return fail(RST_ERR_INVALID_ARGUMENT, "x or logits_out is null");
-  if (use_graphs(m) && batch > 0) {
-    const rst_model::StepGraph key{nullptr, 1, x, logits_out, nullptr, nullptr, batch, 0.0, 0, 0};
-    hipGraphExec_t exec = find_graph(m, key);
-    if (!exec) RST_TRY(capture_graph(m, key, [&] { return do_forward(m, x, batch, logits_out); }, &exec));
-    RST_HIP(hipGraphLaunch(exec, e->stream));
-    // which tensor each layer keeps for backward: what the recorded launches cannot leave behind
-    return do_forward(m, x, batch, logits_out, false);
-  }
   return do_forward(m, x, batch, logits_out);
 }
 
@@ -800,30 +782,13 @@ int rst_model_backward_to(rst_model* m, const double* grad, double* input_grad_o
                           double lr) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
   m->chain_open = false;
-  rst_engine* e = m->engine;
-  RST_TRY(engine_activate(e));
+  RST_TRY(engine_activate(m->engine));
   if (!grad) return fail(RST_ERR_INVALID_ARGUMENT, "grad is null");
-  if (!m->forward_valid)
-    return fail(RST_ERR_STATE, "backward without a forward (the reference panics on a consumed cache)");
   const int need = input_grad_out != nullptr;
   const bool fused = apply_sgd != 0 && m->fuse_sgd;
-  auto run = [&]() -> int {
-    RST_TRY(do_backward(m, grad, need, nullptr, fused ? &lr : nullptr, input_grad_out));
-    if (apply_sgd && !fused) RST_TRY(do_sgd(m, lr));
-    return RST_OK;
-  };
-  if (use_graphs(m) && m->batch > 0) {
-    const rst_model::StepGraph key{nullptr, 2, grad, input_grad_out, m->forward_x, m->logits, m->batch,
-                                   apply_sgd ? lr : 0.0, apply_sgd ? 1 : 0, 0};
-    hipGraphExec_t exec = find_graph(m, key);
-    if (!exec) RST_TRY(capture_graph(m, key, run, &exec));
-    RST_HIP(hipGraphLaunch(exec, e->stream));
-    m->forward_valid = false;  // the caches are consumed, as after the eager pass
-    m->loss_grad_valid = false;
-    m->grads_valid = true;
-    return RST_OK;
-  }
-  return run();
+  RST_TRY(do_backward(m, grad, need, nullptr, fused ? &lr : nullptr, input_grad_out));
+  if (apply_sgd && !fused) RST_TRY(do_sgd(m, lr));
+  return RST_OK;
 }
 
 int rst_model_fuse_sgd(rst_model* m, int enabled) {

@@ -12,6 +12,19 @@ namespace {
 
 __global__ void reset_softmax_flag_kernel(int* flags) { flags[2] = 0; }
 
+// enqueues the arg-max agreement count of pred / truth and waits until it is in the pinned hit word
+int engine_accuracy(rst_engine* e, const double* pred, const double* truth, size_t rows, size_t cols) {
+  bool mirrored = false;
+  const unsigned long long ticket = ++e->tickets_issued;
+  RST_TRY(launch_accuracy(e->stream, pred, truth, rows, cols, e->d_hits, e->hd_hits, &mirrored, e->hd_ticket,
+                          ticket));
+  if (mirrored) return engine_wait_ticket(e, ticket);
+  RST_HIP(hipMemcpyAsync(e->h_hits, e->d_hits, sizeof(unsigned long long), hipMemcpyDeviceToHost,
+                         e->stream));
+  RST_HIP(hipStreamSynchronize(e->stream));
+  return RST_OK;
+}
+
 int check_dim(size_t v, const char* what) {
   if (v > (size_t)INT_MAX) return fail(RST_ERR_UNSUPPORTED, "%s = %zu exceeds 2^31-1", what, v);
   return RST_OK;
@@ -21,7 +34,7 @@ int check_dim(size_t v, const char* what) {
 
 int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, const double* truth,
                          double* grad_out, double* prob_out, size_t rows, size_t cols,
-                         double* host_loss) {
+                         double* host_loss, bool* hits_done) {
   if (rows == 0 || cols == 0) return fail(RST_ERR_SHAPE, "cross entropy of an empty batch");
   if (!row_loss) {  // the engine's own scratch; it moves when it grows, so nothing may keep its address
     RST_TRY(engine_reserve_row_loss(e, rows));
@@ -30,8 +43,18 @@ int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, co
   LossMirror mirror;
   mirror.loss = e->hd_loss;
   mirror.flags = e->hd_flags;
+  // A launch that is being recorded into a graph gets no ticket: every replay would announce the
+  // number of the recording.
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  RST_HIP(hipStreamIsCapturing(e->stream, &capture));
+  e->loss_ticket = 0;
+  if (capture == hipStreamCaptureStatusNone) {
+    mirror.ticket = e->hd_ticket;
+    mirror.ticket_value = e->loss_ticket = ++e->tickets_issued;
+  }
+  if (hits_done) mirror.hits = e->hd_hits;
   RST_TRY(launch_softmax_ce(e->stream, pred, truth, grad_out, prob_out, row_loss, e->d_loss,
-                            e->d_flags, rows, cols, mirror));
+                            e->d_flags, rows, cols, mirror, hits_done));
   e->loss_valid = true;
   if (host_loss) return rst_loss_value(e, host_loss);
   return RST_OK;
@@ -201,7 +224,7 @@ int rst_loss_value(rst_engine* e, double* host_loss) {
   if (!host_loss) return fail(RST_ERR_INVALID_ARGUMENT, "host_loss is null");
   if (!e->loss_valid) return fail(RST_ERR_STATE, "no loss has been computed on this engine");
   // the kernel that finished the loss stored it, and the NaN flag, in the pinned words as well
-  RST_HIP(hipStreamSynchronize(e->stream));
+  RST_TRY(engine_wait_ticket(e, e->loss_ticket));
   *host_loss = *static_cast<volatile double*>(e->h_loss);
   if (static_cast<volatile int*>(e->h_flags)[1] & 1)
     return fail(RST_ERR_NAN, "cross entropy: NaN logits (the reference panics in softmax.rs:38)");
@@ -263,14 +286,24 @@ int rst_accuracy(rst_engine* e, const double* pred, const double* truth, size_t 
   RST_TRY(engine_activate(e));
   if (!pred || !truth || !host_accuracy)
     return fail(RST_ERR_INVALID_ARGUMENT, "accuracy: null operand");
-  bool mirrored = false;
-  RST_TRY(launch_accuracy(e->stream, pred, truth, rows, cols, e->d_hits, e->hd_hits, &mirrored));
-  if (!mirrored)
-    RST_HIP(hipMemcpyAsync(e->h_hits, e->d_hits, sizeof(unsigned long long), hipMemcpyDeviceToHost,
-                           e->stream));
-  RST_HIP(hipStreamSynchronize(e->stream));
+  RST_TRY(engine_accuracy(e, pred, truth, rows, cols));
   *host_accuracy = (double)(*static_cast<volatile unsigned long long*>(e->h_hits)) / (double)rows;
   return RST_OK;
+}
+
+int rst_cross_entropy_accuracy(rst_engine* e, const double* pred, const double* truth, double* grad_out,
+                               size_t rows, size_t cols, double* host_loss, double* host_accuracy) {
+  RST_TRY(engine_activate(e));
+  if (!pred || !truth || !grad_out || !host_loss || !host_accuracy)
+    return fail(RST_ERR_INVALID_ARGUMENT, "cross_entropy_accuracy: null operand");
+  bool hits_done = false;
+  RST_TRY(engine_cross_entropy(e, nullptr, pred, truth, grad_out, nullptr, rows, cols, nullptr, &hits_done));
+  // a batch that one workgroup handles is counted by the cross-entropy launch itself; otherwise
+  // the arg-max kernels follow on the stream, and either way the host waits once
+  if (!hits_done) RST_TRY(engine_accuracy(e, pred, truth, rows, cols));
+  const int status = rst_loss_value(e, host_loss);
+  *host_accuracy = (double)(*static_cast<volatile unsigned long long*>(e->h_hits)) / (double)rows;
+  return status;
 }
 
 int rst_fill_uniform(rst_engine* e, double* dst, size_t count, uint64_t seed, uint64_t stream,

@@ -12,6 +12,7 @@
 // backwards so that the most recently read part of the row is still in L2.
 #include <cfloat>
 
+#include "argmax.h"
 #include "common.h"
 
 namespace rst {
@@ -46,6 +47,22 @@ __device__ __forceinline__ double group_reduce(double v, double* scratch) {
   return v;
 }
 
+// The thread that finishes a loss also stores it, the NaN flag and (if counted) the arg-max hits in
+// pinned host words, and announces them with the launch's ticket, written last behind a
+// system-scope fence: a host that sees the ticket sees the results.
+__device__ __forceinline__ void publish(const LossMirror& mirror, double loss, int nan_flag, bool counted,
+                                        unsigned long long hits) {
+  if (mirror.loss) {
+    mirror.loss[0] = loss;
+    mirror.flags[1] = nan_flag;
+  }
+  if (counted) mirror.hits[0] = hits;
+  if (mirror.ticket) {
+    __threadfence_system();
+    mirror.ticket[0] = mirror.ticket_value;
+  }
+}
+
 __device__ __forceinline__ double loss_term(double truth, double p) {
   if (truth == 0.0) return p > 0.0 ? 0.0 : __builtin_nan("");
   return truth * log(p);
@@ -55,12 +72,16 @@ __device__ __forceinline__ double loss_term(double truth, double p) {
 // rows per workgroup.  SOLO: the whole batch (at most 64 rows) sits in one workgroup of 1024
 // threads, which then also finishes the loss the way loss_reduce_kernel would (same order of
 // additions, same bits), so that a small batch needs one launch instead of two.
-template <int TPR, int IPT, int VEC, bool CE, int BLOCK = 256, bool SOLO = false>
+// ACC (with SOLO): the kernel also counts the rows whose first arg-max agrees between logits and truth
+// (utils.rs:44-65), which a training loop asks for right after the loss - one launch and one
+// round trip instead of two.
+template <int TPR, int IPT, int VEC, bool CE, int BLOCK = 256, bool SOLO = false, bool ACC = false>
 __global__ __launch_bounds__(BLOCK) void softmax_rows_kernel(
     const double* __restrict__ z, const double* __restrict__ truth, double* __restrict__ grad,
     double* __restrict__ prob, double* __restrict__ row_loss, double* __restrict__ loss,
     int* __restrict__ flags, size_t rows, size_t cols, LossMirror mirror) {
-  static_assert(BLOCK % TPR == 0 && (TPR <= 64 || BLOCK == TPR) && (!SOLO || (CE && BLOCK == 1024)), "unsupported shape");
+  static_assert(BLOCK % TPR == 0 && (TPR <= 64 || BLOCK == TPR) && (!SOLO || (CE && BLOCK == 1024)) &&
+                (!ACC || (SOLO && TPR <= 64)), "unsupported shape");
   constexpr int RPB = BLOCK / TPR;
   __shared__ double red[3][TPR > 64 ? TPR / 64 : 1];
 
@@ -72,6 +93,9 @@ __global__ __launch_bounds__(BLOCK) void softmax_rows_kernel(
   double x[IPT][VEC];
   bool saw_nan = false;
   double mx = -DBL_MAX;
+  // (ACC) this thread's first maximum of the logits and of the truth row: value and column
+  double best_z = 0.0, best_t = 0.0;
+  unsigned arg_z = kNoIndex, arg_t = kNoIndex;
 #pragma unroll
   for (int i = 0; i < IPT; ++i) {
     const size_t c = (size_t)(sub + i * TPR) * VEC;
@@ -89,6 +113,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_rows_kernel(
       for (int e = 0; e < VEC; ++e) {
         saw_nan |= (x[i][e] != x[i][e]);
         mx = MaxOp::apply(mx, x[i][e]);
+        if (ACC) argmax_step(best_z, arg_z, x[i][e], c + e);
       }
     }
   }
@@ -131,6 +156,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_rows_kernel(
       for (int e = 0; e < VEC; ++e) {
         lsum += loss_term(t[e], p[e]);
         g[e] = -(t[e] - p[e]);
+        if (ACC) argmax_step(best_t, arg_t, t[e], c + e);
       }
       if (VEC == 2) {
         v2d gv = {g[0], g[VEC - 1]};
@@ -151,12 +177,22 @@ __global__ __launch_bounds__(BLOCK) void softmax_rows_kernel(
   if (CE && SOLO) {
     __shared__ double solo_sum[64];
     __shared__ int solo_nan;
+    __shared__ unsigned solo_hits;
     lsum = group_reduce<TPR, SumOp>(lsum, red[2]);
     if (threadIdx.x < 64) solo_sum[threadIdx.x] = 0.0;
-    if (threadIdx.x == 0) solo_nan = 0;
+    if (threadIdx.x == 0) { solo_nan = 0; solo_hits = 0; }
+    if (ACC) {  // the TPR threads of a row (one wavefront or part of one) agree on the two columns
+      constexpr int W = TPR < 64 ? TPR : 64;
+#pragma unroll
+      for (int off = W / 2; off > 0; off >>= 1) {
+        argmax_combine(best_z, arg_z, __shfl_xor(best_z, off), __shfl_xor(arg_z, off));
+        argmax_combine(best_t, arg_t, __shfl_xor(best_t, off), __shfl_xor(arg_t, off));
+      }
+    }
     __syncthreads();
     if (sub == 0 && row_ok) solo_sum[row] = lsum;
     if (saw_nan) atomicOr(&solo_nan, 1);
+    if (ACC && sub == 0 && row_ok && arg_z == arg_t) atomicAdd(&solo_hits, 1u);  // (an integer count: any order)
     __syncthreads();
     if (threadIdx.x < 64) {
       // loss_reduce_kernel on at most 64 rows: one value per lane of wavefront 0, the butterfly
@@ -169,10 +205,7 @@ __global__ __launch_bounds__(BLOCK) void softmax_rows_kernel(
         const double l = -v / (double)rows;
         loss[0] = l;
         flags[1] = solo_nan;
-        if (mirror.loss) {
-          mirror.loss[0] = l;
-          mirror.flags[1] = solo_nan;
-        }
+        publish(mirror, l, solo_nan, ACC, solo_hits);
       }
     }
   } else if (CE) {
@@ -364,10 +397,7 @@ __global__ __launch_bounds__(1024) void loss_reduce_kernel(const double* __restr
     loss[0] = l;
     flags[1] = nan_seen;
     flags[0] = 0;
-    if (mirror.loss) {
-      mirror.loss[0] = l;
-      mirror.flags[1] = nan_seen;
-    }
+    publish(mirror, l, nan_seen, false, 0);
   }
 }
 
@@ -409,7 +439,7 @@ __global__ __launch_bounds__(256) void softmax_jacobian_kernel(double* __restric
 template <int TPR, int IPT, int VEC>
 int launch_rows(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
                 double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce,
-                LossMirror mirror, bool* loss_done) {
+                LossMirror mirror, bool* loss_done, bool* hits_done) {
   constexpr int BLOCK = 256;
   constexpr int RPB = BLOCK / TPR;
   size_t blocks = (rows + RPB - 1) / RPB;
@@ -417,8 +447,14 @@ int launch_rows(hipStream_t s, const double* z, const double* t, double* grad, d
   // (rows that span several wavefronts reduce through per-row scratch that exists once per workgroup)
   if constexpr (TPR <= 64) {
     if (ce && rows * TPR <= 1024) {
-      hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, true, 1024, true>), dim3(1), dim3(1024), 0, s,
-                         z, t, grad, prob, row_loss, loss, flags, rows, cols, mirror);
+      if (mirror.hits) {
+        hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, true, 1024, true, true>), dim3(1), dim3(1024), 0, s,
+                           z, t, grad, prob, row_loss, loss, flags, rows, cols, mirror);
+        *hits_done = true;
+      } else {
+        hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, true, 1024, true>), dim3(1), dim3(1024), 0, s,
+                           z, t, grad, prob, row_loss, loss, flags, rows, cols, mirror);
+      }
       *loss_done = true;
       RST_HIP(hipGetLastError());
       return RST_OK;
@@ -451,11 +487,11 @@ int launch_wide(hipStream_t s, const double* z, const double* t, double* grad, d
 template <int VEC>
 int dispatch(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
              double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce,
-             LossMirror mirror, bool* loss_done) {
+             LossMirror mirror, bool* loss_done, bool* hits_done) {
   const size_t units = cols / VEC;  // vectors per row
-  if (units <= 16 * 2) return launch_rows<16, 2, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done);
-  if (units <= 64 * 4) return launch_rows<64, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done);
-  if (units <= 256 * 4) return launch_rows<256, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done);
+  if (units <= 16 * 2) return launch_rows<16, 2, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done);
+  if (units <= 64 * 4) return launch_rows<64, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done);
+  if (units <= 256 * 4) return launch_rows<256, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done);
   // measured on 32 Mi logits: 256 threads per row are ahead below about 12 Ki columns, 512 above
   if (cols < 12288) return launch_wide<256, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
   return launch_wide<512, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
@@ -466,24 +502,30 @@ inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 1
 // The row kernel of a softmax or cross entropy; *loss_done tells whether it finished the loss too.
 int launch_row_kernel(hipStream_t s, const double* z, const double* t, double* grad_out, double* prob_out,
                       double* row_loss, double* loss, int* flags, size_t rows, size_t cols,
-                      LossMirror mirror, bool* loss_done) {
+                      LossMirror mirror, bool* loss_done, bool* hits_done) {
   const bool ce = grad_out != nullptr;
   const bool vec = cols % 2 == 0 && aligned16(z) && (!ce || (aligned16(t) && aligned16(grad_out))) &&
                    (!prob_out || aligned16(prob_out));
   *loss_done = false;
-  if (vec) return dispatch<2>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, mirror, loss_done);
-  return dispatch<1>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, mirror, loss_done);
+  if (vec) return dispatch<2>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done);
+  return dispatch<1>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done);
 }
 
 }  // namespace
 
 int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* grad_out,
                       double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
-                      size_t cols, LossMirror mirror) {
+                      size_t cols, LossMirror mirror, bool* hits_done) {
+  bool no_hits = false;
+  if (!hits_done) {
+    hits_done = &no_hits;
+    mirror.hits = nullptr;
+  }
+  *hits_done = false;
   if (rows == 0 || cols == 0) return RST_OK;
   const bool ce = grad_out != nullptr;
   bool loss_done = false;
-  RST_TRY(launch_row_kernel(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, mirror, &loss_done));
+  RST_TRY(launch_row_kernel(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, mirror, &loss_done, hits_done));
   if (ce && !loss_done) {
     hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(1024), 0, s, row_loss, loss, flags, rows, mirror);
     RST_HIP(hipGetLastError());

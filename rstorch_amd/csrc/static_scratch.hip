@@ -77,6 +77,7 @@ extern "C" int rst_cross_entropy_static(rst_engine* e, const double* pred, const
   LossMirror mirror;
   mirror.loss = e->hd_loss;
   mirror.flags = e->hd_flags;
+  e->loss_ticket = 0;  // no ticket: the caller may be recording this call into a graph
   RST_TRY(launch_softmax_ce(e->stream, pred, truth, grad_out, nullptr, base, base + kLossSlot, flags,
                             rows, cols, mirror));
   g_scratch_dirty[e->device] = false;  // the reduction launch re-arms the working word

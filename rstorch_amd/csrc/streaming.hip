@@ -1,6 +1,7 @@
 // HBM-bound streaming kernels: ReLU forward/backward (unfused form), fill, the bias-gradient
 // column mean, SGD and row arg-max accuracy.  All of them move each byte exactly once with
 // 16-byte accesses where alignment allows.
+#include "argmax.h"
 #include "common.h"
 
 namespace rst {
@@ -159,26 +160,12 @@ __global__ __launch_bounds__(kSgdBlock) void sgd_multi_kernel(const SgdTensor* _
 // One wavefront per row: every lane scans a strided part keeping its first maximum, then the
 // lanes are combined preferring the larger value and, on ties, the smaller column - which is
 // the reference's "first maximum wins" (strict > replacement).  NaN never replaces.
-__device__ __forceinline__ void argmax_combine(double& v, unsigned& idx, double ov, unsigned oidx) {
-  if (oidx != 0xffffffffu && (idx == 0xffffffffu || ov > v || (ov == v && oidx < idx))) {
-    v = ov;
-    idx = oidx;
-  }
-}
-
 __device__ __forceinline__ unsigned row_argmax(const double* __restrict__ row, size_t cols,
                                                int lane) {
   // the reference starts from element 0 and replaces only when e > acc
   double v = 0.0;
-  unsigned idx = 0xffffffffu;
-  for (size_t c = lane; c < cols; c += 64) {
-    double x = row[c];
-    // a NaN never wins a strict comparison, so it only counts when it is element 0 (the
-    // reference's initial accumulator), where it also can never be replaced
-    if (x != x && c != 0) continue;
-    if (idx == 0xffffffffu) { v = x; idx = (unsigned)c; }
-    else if (x > v) { v = x; idx = (unsigned)c; }
-  }
+  unsigned idx = kNoIndex;
+  for (size_t c = lane; c < cols; c += 64) argmax_step(v, idx, row[c], c);
   for (int off = 32; off > 0; off >>= 1) {
     double ov = __shfl_xor(v, off);
     unsigned oidx = __shfl_xor(idx, off);
@@ -288,7 +275,9 @@ __global__ __launch_bounds__(1024) void accuracy_small_kernel(const double* __re
                                                              const double* __restrict__ truth,
                                                              size_t rows, size_t cols,
                                                              unsigned long long* hits,
-                                                             unsigned long long* hits_mirror) {
+                                                             unsigned long long* hits_mirror,
+                                                             unsigned long long* ticket,
+                                                             unsigned long long ticket_value) {
   __shared__ unsigned counts[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   unsigned mine = 0;
@@ -304,16 +293,20 @@ __global__ __launch_bounds__(1024) void accuracy_small_kernel(const double* __re
     for (int w = 0; w < 16; ++w) total += counts[w];
     hits[0] = total;
     if (hits_mirror) hits_mirror[0] = total;
+    if (ticket) {  // announced last: a host that sees the ticket sees the count
+      __threadfence_system();
+      ticket[0] = ticket_value;
+    }
   }
 }
 
 int launch_accuracy(hipStream_t s, const double* pred, const double* truth, size_t rows,
                     size_t cols, unsigned long long* hits, unsigned long long* hits_mirror,
-                    bool* mirrored) {
+                    bool* mirrored, unsigned long long* ticket, unsigned long long ticket_value) {
   if (mirrored) *mirrored = false;
   if (hits_mirror && mirrored && rows * cols <= (size_t)1 << 16) {
     hipLaunchKernelGGL(accuracy_small_kernel, dim3(1), dim3(1024), 0, s, pred, truth, rows, cols, hits,
-                       hits_mirror);
+                       hits_mirror, ticket, ticket_value);
     RST_HIP(hipGetLastError());
     *mirrored = true;
     return RST_OK;

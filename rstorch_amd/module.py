@@ -10,11 +10,11 @@ A ``Sequential`` made only of ``Identity`` / ``Linear`` / ``ReLU`` layers is *co
 ``forward`` builds a device model (``rst_model``) over the layer list, moves the layers' weights
 into its parameter arena (the layers keep views) and from then on
 
-* ``forward`` is one replayed graph of the layers' launches,
+* ``forward`` runs the layers' launches from one call,
 * ``backward`` launches nothing: it remembers its gradient, and the pass runs when somebody needs
   its results - ``SGD.step(model)`` runs it with the optimiser update inside the weight-gradient
-  launches (one replayed graph: the README loop's ``model.backward(loss.backward());
-  optim.step(model)`` reaches exactly the launches of ``rst_model_train_step``), while reading a
+  launches (the README loop's ``model.backward(loss.backward()); optim.step(model)`` reaches
+  exactly the launches of ``rst_model_train_step``), while reading a
   gradient through ``parameters()`` or touching the input gradient that ``backward`` returned runs
   it on its own first, so every value a caller can observe is the value the reference computes at
   that point.  The input gradient itself is only computed if the returned array is kept.

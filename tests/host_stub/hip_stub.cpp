@@ -132,6 +132,10 @@ hipError_t hipStreamBeginCapture(hipStream_t, hipStreamCaptureMode) {
   g_captured_nodes = 0;
   return hipSuccess;
 }
+hipError_t hipStreamIsCapturing(hipStream_t, hipStreamCaptureStatus* status) {
+  *status = g_capturing ? hipStreamCaptureStatusActive : hipStreamCaptureStatusNone;
+  return hipSuccess;
+}
 hipError_t hipStreamEndCapture(hipStream_t, hipGraph_t* g) {
   if (!g_capturing) die("hipStreamEndCapture without a capture", nullptr);
   g_capturing = false;

@@ -139,6 +139,13 @@ int main() {
       OK(rst_cross_entropy_static(e, x, t, g, 4096, 10, nullptr));
     }
     EXPECT(rst_cross_entropy_static(e, x, t, g, RST_STATIC_CROSS_ENTROPY_MAX_ROWS + 1, 2, nullptr), RST_ERR_UNSUPPORTED);
+    {  // loss and accuracy after one wait: a batch for one workgroup, a long one, a wide one
+      double loss = 0.0, acc = 0.0;
+      OK(rst_cross_entropy_accuracy(e, x, t, g, 32, 10, &loss, &acc));
+      OK(rst_cross_entropy_accuracy(e, x, t, g, 8192, 10, &loss, &acc));
+      OK(rst_cross_entropy_accuracy(e, x, t, g, 2, 40000, &loss, &acc));
+      EXPECT(rst_cross_entropy_accuracy(e, x, t, g, 2, 4, &loss, nullptr), RST_ERR_INVALID_ARGUMENT);
+    }
     {
       // the entry point that allocates nothing: no allocating or releasing runtime call, device or
       // pinned, on a first use at a new size, on the largest batch it takes, or under stream capture

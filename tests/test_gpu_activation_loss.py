@@ -290,3 +290,66 @@ def test_accuracy_first_maximum_wins(engine, oracle):
         truth[0, :] = 0.0
         truth[0, np.argmax(pred[0])] = 1.0
         assert rs.accuracy(pred, truth) == oracle.accuracy(pred, truth)
+
+
+# rst_cross_entropy_accuracy: the loss of rst_cross_entropy and the count of rst_accuracy after one
+# wait.  One workgroup's worth of rows is counted inside the cross-entropy launch (first shapes), the
+# others by the arg-max kernels that follow it on the stream.
+@pytest.mark.parametrize("rows,cols", [(32, 10), (1, 2), (64, 64), (16, 512), (7, 33), (65, 10), (3000, 1000),
+                                       (8192, 10), (40, 4100), (8, 32768)])
+def test_cross_entropy_with_accuracy_in_one_wait(engine, oracle, rows, cols):
+    import ctypes
+    from rstorch_amd import _ffi
+    rng = np.random.default_rng(rows * 131 + cols)
+    z = np.round(rng.standard_normal((rows, cols)) * 2.0, 1)      # coarse values: ties between columns happen
+    labels = rng.integers(0, cols, rows)
+    labels[: rows // 2] = z[: rows // 2].argmax(axis=1)           # half of the rows are hits
+    t = np.zeros((rows, cols))
+    t[np.arange(rows), labels] = 1.0
+    if rows > 3 and cols > 3:
+        t[1] = 0.0; t[1, [0, 2]] = 0.5                             # a soft-label row with a tie: column 0 wins
+        z[2, :] = 0.25                                             # a row of equal logits: column 0 wins
+    dz, dt = engine.from_numpy(z), engine.from_numpy(t)
+    g1, g2 = engine.full(rows, cols, -3.0), engine.full(rows, cols, -4.0)
+    loss1, loss2, acc1, acc2 = (ctypes.c_double(-1.0) for _ in range(4))
+    _ffi.check(engine.lib.rst_cross_entropy(engine.handle, dz.ptr, dt.ptr, g1.ptr, None, rows, cols, ctypes.byref(loss1)))
+    _ffi.check(engine.lib.rst_accuracy(engine.handle, dz.ptr, dt.ptr, rows, cols, ctypes.byref(acc1)))
+    _ffi.check(engine.lib.rst_cross_entropy_accuracy(engine.handle, dz.ptr, dt.ptr, g2.ptr, rows, cols,
+                                                     ctypes.byref(loss2), ctypes.byref(acc2)))
+    assert loss2.value == loss1.value
+    assert acc2.value == acc1.value == oracle.accuracy(z, t)
+    np.testing.assert_array_equal(g2.to_numpy(), g1.to_numpy())
+    want, _ = oracle.cross_entropy_forward(z, t)
+    assert abs(loss2.value - want) <= 1e-10 * abs(want)
+    # NaN logits: the status of rst_cross_entropy
+    z[0, 0] = np.nan
+    dz = engine.from_numpy(z)
+    assert engine.lib.rst_cross_entropy_accuracy(engine.handle, dz.ptr, dt.ptr, g2.ptr, rows, cols, ctypes.byref(loss2),
+                                                 ctypes.byref(acc2)) == _ffi.RST_ERR_NAN
+
+
+def test_scalar_reads_keep_up_with_many_small_calls(engine, oracle):
+    """The loss and the hit count are announced by a ticket that the host polls: 300 alternating
+    calls on different data must each return their own result, never an earlier one."""
+    import ctypes
+    from rstorch_amd import _ffi
+    rng = np.random.default_rng(5)
+    cases = []
+    for k in range(6):
+        rows, cols = (32, 10) if k % 2 == 0 else (700, 12)
+        z = rng.standard_normal((rows, cols)) * (1.0 + k)
+        t = np.eye(cols)[rng.integers(0, cols, rows)]
+        cases.append((rows, cols, engine.from_numpy(z), engine.from_numpy(t), oracle.cross_entropy_forward(z, t)[0],
+                      oracle.accuracy(z, t)))
+    g = engine.empty(700, 12)
+    loss, acc = ctypes.c_double(), ctypes.c_double()
+    for i in range(300):
+        rows, cols, dz, dt, want_loss, want_acc = cases[i % 6]
+        if i % 3 == 0:
+            _ffi.check(engine.lib.rst_cross_entropy_accuracy(engine.handle, dz.ptr, dt.ptr, g.ptr, rows, cols,
+                                                             ctypes.byref(loss), ctypes.byref(acc)))
+        else:
+            _ffi.check(engine.lib.rst_cross_entropy(engine.handle, dz.ptr, dt.ptr, g.ptr, None, rows, cols, ctypes.byref(loss)))
+            _ffi.check(engine.lib.rst_accuracy(engine.handle, dz.ptr, dt.ptr, rows, cols, ctypes.byref(acc)))
+        assert abs(loss.value - want_loss) <= 1e-10 * abs(want_loss), i
+        assert acc.value == want_acc, i

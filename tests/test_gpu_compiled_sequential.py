@@ -1,4 +1,4 @@
-"""The compiled Sequential (module interface over the device model): forward as one replayed graph,
+"""The compiled Sequential (module interface over the device model): forward as one call,
 backward deferred until the optimiser step or the first look at a gradient.  Whatever a caller can
 observe must be what the layer-by-layer path computes - bit for bit where the two run the same tiles,
 within rounding where a shared grid slices a long batch differently - and the reference's state
@@ -49,7 +49,7 @@ def test_readme_loop_compiled_equals_layer_by_layer(engine, oracle, name, spec, 
     opt_f, opt_s = rs.SGD.new(0.05), rs.SGD.new(0.05)
     same = np.array_equal if exact else (lambda a, b: rel_err(a, b) <= 1e-12)
     for step in range(4):
-        x, y = batch_data(oracle, batch, n_in, n_out, 7, step % 2, normal)  # two batches: both graphs replay
+        x, y = batch_data(oracle, batch, n_in, n_out, 7, step % 2, normal)  # two batches in turn
         pf, ps = fast.forward(x), slow.forward(x)
         assert same(pf.to_numpy(), ps.to_numpy()), "logits, step %d" % step
         lf, ls = loss_f.forward(pf.clone(), y), loss_s.forward(ps.clone(), y)
