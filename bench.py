@@ -13,12 +13,15 @@ Prints ONE JSON line.  `roofline` is for the FP64-MFMA contraction kernel instan
 largest share of the step; per-launch durations come from HIP events recorded on the engine's
 stream around every launch of the timed steps.  `cpu_baseline` is the CPU restatement (oracle)
 timed on this host, single thread like the reference: one whole C4 step at the full batch.
-`other_configs` holds, for configs[0..2], the graph-replay rate, a second pass with per-launch events
-(contraction TFLOP/s against the FP64 MFMA peak) and the oracle timed on the same configuration;
-`readme_loop_b32` is the reference's README loop shape (layer by layer, loss and accuracy read back
-every step) run by the C++ host mirror in a child process.
+`other_configs` holds, for configs[0..2], the graph-replay rate (C0 and C1: fresh inputs every step,
+two resident batches refilled in turn on a second stream; also with the scalar loss read every step),
+a second pass with per-launch events (contraction TFLOP/s against the FP64 MFMA peak) and the oracle
+timed on the same configuration; `readme_loop` is the reference's README loop (README.md:64-74: the
+module interface, loss and accuracy read back every step) run by the C++ host mirror in child
+processes on configs[0], [1], [2] and [4], next to the single-call step of the same configuration.
 """
 import argparse
+import hashlib
 import json
 import os
 import re
@@ -39,8 +42,24 @@ PEAK_HBM_GBPS = 8000.0
 # A launch = the contraction plus, for the one that is contracted as two K slices (the head's input
 # gradient), the reduction of the two partial results (134.3 MB); the weight gradient carries the SGD
 # update of its layer.
+# The figures hold for the kernel sources they were measured on: kernel_sources_sha16 is the first 16
+# hex digits of the SHA-256 over the files below, taken when the profile was collected.  When the
+# files have changed since, `traffic` is reported as null (and tests/test_host_logic.py fails) until
+# the profile is collected again and the digest updated.
 C4_TRAFFIC_SOURCE = {"profile": "profiles/c4_hbm_traffic.md",
-                     "kernels_as_of_commit": "d945909"}
+                     "kernel_sources": ["rstorch_amd/csrc/gemm_f64.hip", "rstorch_amd/csrc/gemm_addressing.h"],
+                     "kernel_sources_sha16": "0000000000000000"}
+
+
+def kernel_sources_digest():
+    h = hashlib.sha256()
+    for rel in C4_TRAFFIC_SOURCE["kernel_sources"]:
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+
 C4_TRAFFIC_BYTES_PER_LAUNCH = {
     "linear_forward": (8 * 436.4e6 + 3891.6e6) / 9,
     "grad_weight": (8 * 866.1e6 + 8700.8e6) / 9,
@@ -202,16 +221,71 @@ def contraction_summary(recs, steps):
         "first_layer_input_gradient": "skipped (the README loop discards it)"}
 
 
-def bench_small(rs, eng, spec, batch, normal, steps, warmup, eager, profile_steps):
+def time_fresh_steps(rs, eng, loader, dm, batch, normal, steps, warmup, read_loss):
+    """Steps on fresh inputs: two resident batches; while the training engine works on one, a second
+    engine (a second stream of the same GPU) refills the other from the counter generator, stream
+    number = step.  Events hand the buffers back and forth; the host never waits inside the loop
+    unless read_loss asks for the scalar loss of every step."""
+    from rstorch_amd import _ffi
+    n_in, n_out = dm.in_width, dm.out_width
+    bufs = [(eng.empty(batch, n_in), eng.empty(batch, n_out)) for _ in range(2)]
+    filled = [loader.event() for _ in range(2)]   # recorded by the loader when a buffer is ready
+    used = [eng.event() for _ in range(2)]        # recorded by the trainer when it is done with it
+
+    def refill(slot, step):
+        x, y = bufs[slot]
+        fill = loader.lib.rst_fill_normal if normal else loader.lib.rst_fill_uniform
+        _ffi.check(fill(loader.handle, x.ptr, x.size, SEED, 1000 + 2 * step, 0.0, 1.0))
+        _ffi.check(loader.lib.rst_fill_one_hot(loader.handle, y.ptr, batch, n_out, SEED, 1001 + 2 * step))
+        filled[slot].record()
+
+    def run(first, count):
+        refill(first % 2, first)
+        loss = None
+        for k in range(first, first + count):
+            slot = k % 2
+            if k + 1 < first + count:
+                if k >= first + 1:
+                    loader.wait_event(used[1 - slot])  # the step that last read the other buffer
+                refill(1 - slot, k + 1)
+            eng.wait_event(filled[slot])
+            loss = dm.train_step(bufs[slot][0], bufs[slot][1], LR, want_loss=read_loss)
+            used[slot].record()
+        eng.synchronize()
+        loader.synchronize()
+        return loss
+
+    run(0, warmup)
+    t0 = time.perf_counter()
+    run(warmup, steps)
+    wall = time.perf_counter() - t0
+    return wall, dm.last_loss()
+
+
+def bench_small(rs, eng, spec, batch, normal, steps, warmup, eager, profile_steps, fresh_inputs=False):
     """steps_per_s: the fused step as shipped (graph replay unless --eager).  `contractions`: a
     second pass with an event after every launch (plain launches, one weight gradient per layer)."""
     dm, x, y = make_model(rs, eng, spec, batch, normal)
     if eager:
         dm.graph_enable(False)
-    wall, dev_ms, loss, _ = time_steps(eng, dm, x, y, steps, warmup, False)
-    out = {"batch": batch, "steps": steps, "ms_per_step": wall * 1e3 / steps,
-           "steps_per_s": steps / wall, "samples_per_s": steps / wall * batch, "final_loss": loss,
-           "launch_mode": "plain launches" if eager else "graph replay"}
+    out = {"batch": batch, "steps": steps, "launch_mode": "plain launches" if eager else "graph replay"}
+    if fresh_inputs:
+        loader = rs.Engine(eng.device)
+        wall, loss = time_fresh_steps(rs, eng, loader, dm, batch, normal, steps, warmup, False)
+        out["inputs"] = ("fresh every step: two resident batches, refilled in turn on a second stream by the "
+                         "counter generator (stream number = step)")
+        wall_read, loss_read = time_fresh_steps(rs, eng, loader, dm, batch, normal, steps, warmup, True)
+        out["with_loss_read_every_step"] = {"ms_per_step": wall_read * 1e3 / steps, "steps_per_s": steps / wall_read,
+                                            "final_loss": loss_read}
+        wall_one, _, loss_one, _ = time_steps(eng, dm, x, y, steps, warmup, False)
+        out["one_resident_batch"] = {"ms_per_step": wall_one * 1e3 / steps, "steps_per_s": steps / wall_one,
+                                     "final_loss": loss_one}
+        loader.close()
+    else:
+        wall, _, loss, _ = time_steps(eng, dm, x, y, steps, warmup, False)
+        out["inputs"] = "one resident batch"
+    out.update({"ms_per_step": wall * 1e3 / steps, "steps_per_s": steps / wall,
+                "samples_per_s": steps / wall * batch, "final_loss": loss})
     _, _, _, recs = time_steps(eng, dm, x, y, profile_steps, 2, True)
     kernels, out["contractions"] = contraction_summary(recs, profile_steps)
     out["kernels"] = {k: {"avg_launch_us": v["avg_launch_ms"] * 1e3, "launches_per_step": v["launches_per_step"],
@@ -220,27 +294,44 @@ def bench_small(rs, eng, spec, batch, normal, steps, warmup, eager, profile_step
     return out
 
 
-def readme_loop_child():
-    """The README-shaped loop (README.md:64-74) through the C++ mirror of the module interface, in a
-    process of its own, started before this one touches the GPU."""
+README_LOOP_RUNS = {  # configuration -> (batch, steps per epoch, epochs)
+    "C0": (32, 1875, 3), "C1": (8192, 400, 3), "C2": (2048, 40, 3), "C4": (1024, 20, 3)}
+
+
+def readme_loop_child(config, layer_by_layer=False):
+    """The README loop (README.md:64-74) through the C++ mirror of the module interface, in a process
+    of its own, started before this one touches the GPU.  The rate is that of the last epoch."""
     exe = os.path.join(ROOT, "rstorch_amd", "cpp", "bin", "readme_loop")
     if not os.path.exists(exe):
         return {"error": "rstorch_amd/cpp/bin/readme_loop is not built (__graft_entry__.build())"}
+    batch, steps, epochs = README_LOOP_RUNS[config]
+    cmd = [exe, str(epochs), str(steps), config] + (["layers"] if layer_by_layer else [])
     try:
-        proc = subprocess.run([exe, "3", "1875"], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
-                              text=True, timeout=120)
+        proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=180)
     except subprocess.TimeoutExpired:
-        return {"error": "readme_loop did not finish in 120 s"}
-    rates = [float(m) for m in re.findall(r"\((\d+) steps/s\)", proc.stdout)]
+        return {"error": "readme_loop did not finish in 180 s"}
+    rates = [float(m) for m in re.findall(r"\(([0-9.]+) steps/s\)", proc.stdout)]
     losses = [float(m) for m in re.findall(r"Avarage loss ([0-9.]+)", proc.stdout)]
     if proc.returncode != 0 or not rates:
         return {"error": "readme_loop failed: %s" % (proc.stderr.strip() or proc.stdout.strip())[:200]}
-    return {"batch": 32, "steps_per_epoch": 1875, "epochs": len(rates), "steps_per_s": rates[-1],
-            "samples_per_s": rates[-1] * 32, "steps_per_s_per_epoch": rates,
-            "average_loss_per_epoch": losses,
-            "shape": "model.forward -> loss.forward(pred.clone(), y.clone()) -> accuracy(pred, y) -> "
-                     "model.backward(loss.backward()) -> optim.step(model), layer by layer; the loss and "
-                     "the accuracy are read back every step; the first layer's input gradient is computed"}
+    return {"batch": batch, "steps_per_epoch": steps, "epochs": len(rates), "steps_per_s": rates[-1],
+            "ms_per_step": 1e3 / rates[-1], "samples_per_s": rates[-1] * batch, "steps_per_s_per_epoch": rates,
+            "average_loss_per_epoch": losses}
+
+
+def readme_loops():
+    out = {"shape": "model.forward(x) -> loss.forward(pred.clone(), y.clone()) -> accuracy(pred, y) -> "
+                    "model.backward(loss.backward()) -> optim.step(model) through the module interface of the C++ "
+                    "mirror; the loss and the accuracy are read back every step.  compiled: the Sequential runs "
+                    "as a device model (backward deferred to the optimiser step, SGD inside the weight-gradient "
+                    "launches, the first layer's input gradient skipped because the loop drops it); "
+                    "layer_by_layer: one call per layer, SGD as a pass of its own"}
+    for config in ("C0", "C1", "C2", "C4"):
+        log("README loop, %s ..." % config)
+        out[config] = {"compiled": readme_loop_child(config)}
+        if config in ("C0", "C1"):
+            out[config]["layer_by_layer"] = readme_loop_child(config, True)
+    return out
 
 
 def bench_staged(rs, eng, spec, batch, normal, steps, warmup, in_place=False):
@@ -403,8 +494,7 @@ def main():
     # a child process that uses the GPU runs before this process opens it
     readme_loop = None
     if not (args.no_extra or args.sgd_only or args.only):
-        log("README-shaped loop (C++ mirror, child process) ...")
-        readme_loop = readme_loop_child()
+        readme_loop = readme_loops()
 
     import rstorch_amd as rs
     eng = rs.default_engine()
@@ -415,12 +505,13 @@ def main():
         print(json.dumps({"sgd_c3": bench_sgd_c3(rs, eng)}), flush=True)
         return
 
-    small = {"C0": ("C0_readme_b32", C01_SPEC, 32, False, 2000, 100, 200),
-             "C1": ("C1_readme_b8192", C01_SPEC, 8192, False, 200, 20, 50),
-             "C2": ("C2_wide_b2048", C2_SPEC, 2048, True, 20, 3, 10)}
+    # (name, layers, batch, N(0,1) inputs, timed steps, warm-up, profiled steps, fresh inputs every step)
+    small = {"C0": ("C0_readme_b32", C01_SPEC, 32, False, 2000, 100, 200, True),
+             "C1": ("C1_readme_b8192", C01_SPEC, 8192, False, 200, 20, 50, True),
+             "C2": ("C2_wide_b2048", C2_SPEC, 2048, True, 20, 3, 10, False)}
     if args.only:
-        name, spec, batch, normal, steps, warmup, psteps = small[args.only]
-        print(json.dumps({name: bench_small(rs, eng, spec, batch, normal, steps, warmup, args.eager, psteps)}),
+        name, spec, batch, normal, steps, warmup, psteps, fresh = small[args.only]
+        print(json.dumps({name: bench_small(rs, eng, spec, batch, normal, steps, warmup, args.eager, psteps, fresh)}),
               flush=True)
         return
 
@@ -449,15 +540,23 @@ def main():
     gemm_kinds = [k for k in ("linear_forward", "grad_weight", "grad_input", "grad_pair") if k in kernels]
     dominant = max(gemm_kinds, key=lambda k: kernels[k]["ms_per_step"])
     d = kernels[dominant]
+    traffic_current = kernel_sources_digest() == C4_TRAFFIC_SOURCE["kernel_sources_sha16"]
+    if not traffic_current:
+        log("WARNING: the contraction kernel sources have changed since profiles/c4_hbm_traffic.md was collected: "
+            "roofline.traffic is reported as null until the counters are collected again")
     launches = [r for r in recs if r["kernel"] == dominant]
     flops_per_launch = sum(r["flops"] for r in launches) / len(launches)
     kernel_names = {"grad_pair": "gemm_f64_mfma_dma_pair (a layer's weight gradient + SGD and the next layer's "
                                  "input gradient in one grid)"}
     roofline = {"kernel": kernel_names.get(dominant, "gemm_f64_mfma_dma (" + dominant + ")"), "bound": "mfma",
                 "achieved": d["achieved_tflops"], "peak": PEAK_FP64_MFMA_TFLOPS, "unit": "TFLOP/s",
-                "frac": d["frac"], "traffic": C4_TRAFFIC_BYTES_PER_LAUNCH.get(dominant),
+                "frac": d["frac"],
+                "traffic": C4_TRAFFIC_BYTES_PER_LAUNCH.get(dominant) if traffic_current else None,
+                # the counters need a profiler run of their own (rocprofv3 --pmc): the figure is the one
+                # of the committed profile, valid while the kernel sources are the ones it was taken on
+                "traffic_measured_in_run": False,
                 "traffic_unit": "bytes per launch (L2 misses + write-backs, rocprofv3 FETCH_SIZE/WRITE_SIZE)",
-                "traffic_source": C4_TRAFFIC_SOURCE,
+                "traffic_source": dict(C4_TRAFFIC_SOURCE, kernel_sources_sha16_now=kernel_sources_digest()),
                 "algorithmic_bytes_per_launch": sum(r["bytes"] for r in launches) / len(launches),
                 "avg_launch_ms": d["avg_launch_ms"], "flops_per_launch": flops_per_launch}
     gemm_ms = sum(kernels[k]["ms_per_step"] for k in gemm_kinds)
@@ -481,8 +580,8 @@ def main():
                    "final_loss": loss, "per_launch_events": True,
                    "paired_gradient_launches": not args.no_pair,
                    # the loss is computed on the device every step but the host does not read it inside
-                   # the timed loop (one read after the last step); the README-shaped loop, which reads
-                   # the loss and the accuracy every step, is reported as readme_loop_b32
+                   # the timed loop (one read after the last step); the README loop, which reads the
+                   # loss and the accuracy every step, is reported as readme_loop
                    "per_step_loss_read": False},
         "roofline": roofline,
         "contractions": all_gemm,
@@ -495,9 +594,17 @@ def main():
         result["relu_standalone"] = bench_relu(rs, eng)
         log("other configurations ...")
         result["other_configs"] = {
-            name: bench_small(rs, eng, spec, batch, normal, steps, warmup, args.eager, psteps)
-            for name, spec, batch, normal, steps, warmup, psteps in small.values()}
-        result["readme_loop_b32"] = readme_loop
+            name: bench_small(rs, eng, spec, batch, normal, steps, warmup, args.eager, psteps, fresh)
+            for name, spec, batch, normal, steps, warmup, psteps, fresh in small.values()}
+        result["readme_loop"] = readme_loop
+        for config, name in (("C0", "C0_readme_b32"), ("C1", "C1_readme_b8192"), ("C2", "C2_wide_b2048")):
+            single = result["other_configs"][name]["steps_per_s"]
+            loop = readme_loop.get(config, {}).get("compiled", {})
+            if "steps_per_s" in loop:
+                loop["fraction_of_single_call_step"] = loop["steps_per_s"] / single
+        if "steps_per_s" in readme_loop.get("C4", {}).get("compiled", {}):
+            readme_loop["C4"]["compiled"]["fraction_of_single_call_step"] = \
+                readme_loop["C4"]["compiled"]["steps_per_s"] / (args.steps / wall)
         log("host-fed (PCIe-inclusive) runs ...")
         result["host_fed"] = {
             "C1_readme_b8192": bench_staged(rs, eng, C01_SPEC, 8192, False, 100, 10),

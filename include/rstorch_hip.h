@@ -76,6 +76,10 @@ int rst_event_create(rst_engine* engine, rst_event** out);
 /* May be called after the event's engine has been destroyed (record and elapsed may not). */
 int rst_event_destroy(rst_event* event);
 int rst_event_record(rst_event* event);
+/* Work enqueued on `engine` after this call starts only once `event` (recorded on any engine of the
+ * same GPU) has happened; the host does not wait.  How two engines - two streams - hand buffers to
+ * each other, e.g. a loader engine that refills an input array while the training engine works. */
+int rst_event_wait(rst_engine* engine, rst_event* event);
 /* Waits for `stop` and returns the time between the two records in milliseconds. */
 int rst_event_elapsed_ms(rst_event* start, rst_event* stop, double* host_ms);
 

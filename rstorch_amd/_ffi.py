@@ -74,6 +74,7 @@ SIGNATURES = {
     "rst_event_create": [_vp, c_void_pp],
     "rst_event_destroy": [_vp],
     "rst_event_record": [_vp],
+    "rst_event_wait": [_vp, _vp],
     "rst_event_elapsed_ms": [_vp, _vp, c_double_p],
     "rst_linear_forward": [_vp, _dp, _dp, _dp, _dp, _sz, _sz, _sz, _i32],
     "rst_linear_backward": [_vp, _dp, _dp, _dp, _dp, _dp, _dp, _dp, _sz, _sz, _sz],

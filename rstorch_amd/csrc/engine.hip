@@ -316,6 +316,14 @@ int rst_event_record(rst_event* ev) {
   return RST_OK;
 }
 
+int rst_event_wait(rst_engine* e, rst_event* ev) {
+  if (!ev) return fail(RST_ERR_INVALID_ARGUMENT, "event is null");
+  RST_TRY(engine_activate(e));
+  if (ev->device != e->device) return fail(RST_ERR_INVALID_ARGUMENT, "the event belongs to another GPU");
+  RST_HIP(hipStreamWaitEvent(e->stream, ev->ev, 0));
+  return RST_OK;
+}
+
 int rst_event_elapsed_ms(rst_event* start, rst_event* stop, double* host_ms) {
   if (!start || !stop || !host_ms) return fail(RST_ERR_INVALID_ARGUMENT, "null argument");
   RST_TRY(engine_activate(stop->engine));

@@ -74,6 +74,10 @@ class Engine:
     def event(self):
         return Event(self)
 
+    def wait_event(self, event):
+        """Later work on this engine starts only after ``event`` (recorded on any engine of this GPU)."""
+        _ffi.check(self.lib.rst_event_wait(self.handle, event.handle))
+
     def malloc(self, count):
         p = ctypes.c_void_p()
         _ffi.check(self.lib.rst_malloc(self.handle, int(count), ctypes.byref(p)))

@@ -286,6 +286,8 @@ int main() {
   OK(rst_event_record(b));
   double ms = 0.0;
   OK(rst_event_elapsed_ms(a, b, &ms));
+  OK(rst_event_wait(e, a));
+  EXPECT(rst_event_wait(e, nullptr), RST_ERR_INVALID_ARGUMENT);
   OK(rst_event_destroy(a));
   OK(rst_event_destroy(b));
   const long launches = hip_stub_launch_count();
