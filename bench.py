@@ -204,6 +204,87 @@ def bench_sgd_c3(rs, eng, iters=20):
     return res
 
 
+def run_streaming_kernels(rs, eng, iters=10):
+    """The HBM-bound kernels on their own, for profiler runs (kernel trace, FETCH_SIZE / WRITE_SIZE):
+    the unfused ReLU passes and the flat SGD pass over 2^27 doubles (the SGD pass, 2 GiB read and 1 GiB
+    written per launch, is the known-size kernel the counters are scaled by), the cross entropy and the
+    accuracy count at the logit shapes of configs[2] (2048 x 1000) and configs[4] (1024 x 32768).
+    Prints event-timed rates on its own."""
+    import ctypes
+    from rstorch_amd import _ffi
+    lib, h = eng.lib, eng.handle
+    n = 1 << 27
+    a, b, c = eng.normal(1, n, SEED, 3100), eng.normal(1, n, SEED, 3101, 0.0, 1e-3), eng.empty(1, n)
+    runs = [
+        ("relu_forward", 16.0 * n, lambda: lib.rst_relu_forward(h, a.ptr, c.ptr, n)),
+        ("relu_backward", 24.0 * n, lambda: lib.rst_relu_backward(h, b.ptr, a.ptr, c.ptr, n)),
+        ("sgd_flat", 24.0 * n, lambda: lib.rst_sgd_step_flat(h, a.ptr, b.ptr, n, LR)),
+    ]
+    keep = []
+    for rows, cols in ((2048, 1000), (1024, 32768)):
+        z, t, g = eng.normal(rows, cols, SEED, 3200), eng.one_hot(rows, cols, SEED, 3201), eng.empty(rows, cols)
+        keep.append((z, t, g))
+        acc = ctypes.c_double()
+        runs.append(("cross_entropy_%dx%d" % (rows, cols), 24.0 * rows * cols + 8.0 * rows,
+                     lambda z=z, t=t, g=g, rows=rows, cols=cols: lib.rst_cross_entropy(h, z.ptr, t.ptr, g.ptr, None, rows, cols, None)))
+        runs.append(("accuracy_%dx%d" % (rows, cols), 16.0 * rows * cols,
+                     lambda z=z, t=t, rows=rows, cols=cols, acc=acc: lib.rst_accuracy(h, z.ptr, t.ptr, rows, cols, ctypes.byref(acc))))
+    out = {}
+    for name, nbytes, call in runs:
+        for _ in range(2):
+            _ffi.check(call())
+        eng.synchronize()
+        ev0, ev1 = eng.event(), eng.event()
+        ev0.record()
+        for _ in range(iters):
+            _ffi.check(call())
+        ev1.record()
+        eng.synchronize()
+        ms = ev0.elapsed_ms(ev1) / iters
+        out[name] = {"ms": ms, "algorithmic_bytes": nbytes, "achieved_gbps": nbytes / (ms * 1e-3) / 1e9,
+                     "frac_of_hbm_peak": nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS}
+    return out
+
+
+def run_route_sweep(rs, eng):
+    """Times Linear::forward, the weight gradient alone and the whole Linear::backward over a grid of
+    mid-size shapes (batch 128..16384, widths 64..4096, at least one product below 256 tiles of
+    128x128) under whatever RSTORCH_DMA64 says (unset: the planner's rule; 0: never the 64x64
+    direct-to-LDS kernel; 1: wherever it is eligible).  CSV on stdout: the table the routing rule in
+    choose_route is fitted to."""
+    import itertools
+    from rstorch_amd import _ffi
+    lib, h = eng.lib, eng.handle
+
+    def timeit(fn, reps=30):
+        for _ in range(3):
+            fn()
+        eng.synchronize()
+        a, b = eng.event(), eng.event()
+        a.record()
+        for _ in range(reps):
+            fn()
+        b.record()
+        eng.synchronize()
+        return a.elapsed_ms(b) / reps * 1e3
+
+    tiles = lambda m, n: ((m + 127) // 128) * ((n + 127) // 128)
+    print("B,K,N,forward_us,weight_gradient_us,backward_us", flush=True)
+    for B, K, N in itertools.product([128, 256, 512, 1024, 2048, 4096, 8192, 16384],
+                                     [64, 100, 128, 256, 512, 784, 1024, 2048, 4096],
+                                     [64, 100, 256, 512, 1000, 2048, 4096]):
+        flops = 2.0 * B * K * N
+        if flops < 5e7 or flops > 2e10 or min(tiles(B, N), tiles(N, K), tiles(B, K)) >= 256:
+            continue
+        x, w, b, g = eng.normal(B, K, 1, 1), eng.normal(N, K, 1, 2), eng.normal(1, N, 1, 3), eng.normal(B, N, 1, 4)
+        o, gw, gb, gx = eng.empty(B, N), eng.empty(N, K), eng.empty(1, N), eng.empty(B, K)
+        f = timeit(lambda: _ffi.check(lib.rst_linear_forward(h, x.ptr, w.ptr, b.ptr, o.ptr, B, K, N, 1)))
+        dw = timeit(lambda: _ffi.check(lib.rst_linear_backward(h, g.ptr, x.ptr, w.ptr, gw.ptr, gb.ptr, None, None, B, K, N)))
+        both = timeit(lambda: _ffi.check(lib.rst_linear_backward(h, g.ptr, x.ptr, w.ptr, gw.ptr, gb.ptr, gx.ptr, x.ptr, B, K, N)))
+        print("%d,%d,%d,%.2f,%.2f,%.2f" % (B, K, N, f, dw, both), flush=True)
+        del x, w, b, g, o, gw, gb, gx
+
+
 def contraction_summary(recs, steps):
     """Contraction launches of a profiled pass: rate against the FP64 MFMA peak, the class with the
     largest share, and the step's launch count."""
@@ -483,6 +564,12 @@ def main():
     ap.add_argument("--no-pair", action="store_true",
                     help="launch every weight gradient and input gradient of C4 on its own (profiles that "
                          "attribute counters to one product at a time)")
+    ap.add_argument("--streaming-kernels", action="store_true",
+                    help="run only the HBM-bound kernels (ReLU, SGD, cross entropy, accuracy) on their own, "
+                         "for profiler runs")
+    ap.add_argument("--route-sweep", action="store_true",
+                    help="time the three products of a Linear layer over the grid of mid-size shapes the "
+                         "routing rule is fitted to; CSV on stdout")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one streaming ReLU over 1 GiB (reads 1 GiB, writes 1 GiB): the "
                          "known-size kernel that rocprofv3 FETCH_SIZE / WRITE_SIZE are scaled by")
@@ -493,7 +580,7 @@ def main():
 
     # a child process that uses the GPU runs before this process opens it
     readme_loop = None
-    if not (args.no_extra or args.sgd_only or args.only):
+    if not (args.no_extra or args.sgd_only or args.only or args.streaming_kernels or args.route_sweep):
         readme_loop = readme_loops()
 
     import rstorch_amd as rs
@@ -503,6 +590,12 @@ def main():
 
     if args.sgd_only:
         print(json.dumps({"sgd_c3": bench_sgd_c3(rs, eng)}), flush=True)
+        return
+    if args.streaming_kernels:
+        print(json.dumps({"streaming_kernels": run_streaming_kernels(rs, eng)}), flush=True)
+        return
+    if args.route_sweep:
+        run_route_sweep(rs, eng)
         return
 
     # (name, layers, batch, N(0,1) inputs, timed steps, warm-up, profiled steps, fresh inputs every step)

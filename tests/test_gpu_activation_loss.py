@@ -284,12 +284,22 @@ def test_cross_entropy_nan_logits_is_an_error(engine):
 def test_accuracy_first_maximum_wins(engine, oracle):
     import rstorch_amd as rs
     rng = np.random.default_rng(8)
-    for rows, cols in [(32, 10), (100, 1000), (5, 70)]:
+    # (the last three shapes take the one-workgroup-per-row kernel for wide rows)
+    for rows, cols in [(32, 10), (100, 1000), (5, 70), (9, 4096), (40, 4100), (12, 32768), (3, 4097)]:
         pred = rng.integers(0, 4, size=(rows, cols)).astype(np.float64)  # many ties
         truth = np.zeros((rows, cols)); truth[np.arange(rows), rng.integers(0, cols, rows)] = 1.0
         truth[0, :] = 0.0
         truth[0, np.argmax(pred[0])] = 1.0
-        assert rs.accuracy(pred, truth) == oracle.accuracy(pred, truth)
+        if rows > 4:
+            hit = rng.integers(0, cols, rows)          # rows whose single maximum sits on the label
+            pred[np.arange(2, rows), hit[2:]] = 9.0
+            truth[2:] = 0.0
+            truth[np.arange(2, rows), hit[2:]] = 1.0
+            pred[2, 0] = np.nan                         # a NaN in element 0 is never replaced (utils.rs:47-52)
+            pred[3, cols // 2] = np.nan                 # anywhere else it never wins
+        got, want = rs.accuracy(pred, truth), oracle.accuracy(pred, truth)
+        assert got == want, (rows, cols, got, want)
+        assert rows <= 4 or 0.0 < want < 1.0
 
 
 # rst_cross_entropy_accuracy: the loss of rst_cross_entropy and the count of rst_accuracy after one
