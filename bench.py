@@ -73,6 +73,8 @@ C4_SPEC = [("linear", 4096, 4096), ("relu",)] * 8 + [("linear", 4096, 32768)]
 C4_BATCH = 1024
 C2_SPEC = [("linear", 1024, 4096), ("relu",), ("linear", 4096, 4096), ("relu",),
            ("linear", 4096, 1000)]
+# configs[2] with every extent odd: nothing is 16-byte aligned from one row to the next
+C2_ODD_SPEC = [("linear", 1023, 4095), ("relu",), ("linear", 4095, 4095), ("relu",), ("linear", 4095, 999)]
 C01_SPEC = [("identity",), ("linear", 784, 100), ("relu",), ("linear", 100, 100), ("relu",),
             ("linear", 100, 10)]
 LR = 0.01
@@ -557,7 +559,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations")
     ap.add_argument("--eager", action="store_true",
                     help="plain kernel launches instead of graph replay")
-    ap.add_argument("--only", choices=["C0", "C1", "C2"],
+    ap.add_argument("--only", choices=["C0", "C1", "C2", "C2_odd"],
                     help="run one of the small configurations alone (for profiler runs)")
     ap.add_argument("--sgd-only", action="store_true",
                     help="time only SGD::step over the configs[3] parameter set (for profiler runs)")
@@ -601,7 +603,8 @@ def main():
     # (name, layers, batch, N(0,1) inputs, timed steps, warm-up, profiled steps, fresh inputs every step)
     small = {"C0": ("C0_readme_b32", C01_SPEC, 32, False, 2000, 100, 200, True),
              "C1": ("C1_readme_b8192", C01_SPEC, 8192, False, 200, 20, 50, True),
-             "C2": ("C2_wide_b2048", C2_SPEC, 2048, True, 20, 3, 10, False)}
+             "C2": ("C2_wide_b2048", C2_SPEC, 2048, True, 20, 3, 10, False),
+             "C2_odd": ("C2_odd_b2047", C2_ODD_SPEC, 2047, True, 20, 3, 10, False)}
     if args.only:
         name, spec, batch, normal, steps, warmup, psteps, fresh = small[args.only]
         print(json.dumps({name: bench_small(rs, eng, spec, batch, normal, steps, warmup, args.eager, psteps, fresh)}),

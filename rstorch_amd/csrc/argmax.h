@@ -27,4 +27,18 @@ __device__ __forceinline__ void argmax_combine(double& v, unsigned& idx, double 
   }
 }
 
+// One result record in pinned host memory, written with a single 16-byte store so that the ticket
+// and the value it announces arrive together: {value or count (8 bytes), flags, ticket}.
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_result_slot(void* slot, double value, unsigned long long count, bool is_count,
+                                                  unsigned flags, unsigned ticket) {
+  const unsigned long long bits = is_count ? count : (unsigned long long)__double_as_longlong(value);
+  v4u record;
+  record.x = (unsigned)(bits & 0xffffffffull);
+  record.y = (unsigned)(bits >> 32);
+  record.z = flags;
+  record.w = ticket;
+  __builtin_nontemporal_store(record, reinterpret_cast<v4u*>(slot));
+}
+
 }  // namespace rst

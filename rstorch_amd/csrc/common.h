@@ -117,16 +117,27 @@ unsigned long long sgd_blocks_for(unsigned long long count);
 // LossMirror: device-visible addresses of pinned host words that receive the loss and flags[1]
 // as well (written by the thread that finishes the loss), so that the host can read them after a
 // stream synchronisation without a copy in between.  Null members: no mirror.
-// ticket: a third pinned word that the same thread writes last, behind a system-scope fence, with
-// ticket_value: the host can then wait for exactly this result by polling the word instead of
-// synchronising the stream.  hits: when set, a cross entropy whose whole batch sits in one workgroup
-// also counts the rows whose first arg-max agrees between logits and truth (src/utils.rs:44-65) and
-// stores the count there; launch_softmax_ce reports whether it did.
+// slots / ticket: the same thread also writes the result, together with the launch's ticket, into a
+// 16-byte record in pinned host memory with ONE 16-byte store (slots[0]: loss and NaN flag, slots[1]:
+// hit count): the host can then wait for exactly this result by polling the record instead of
+// synchronising the stream, and a record that shows the ticket holds the result whatever order
+// separate writes to host memory may arrive in.  hits: when set, a cross entropy whose whole batch
+// sits in one workgroup also counts the rows whose first arg-max agrees between logits and truth
+// (src/utils.rs:44-65) and stores the count there; launch_softmax_ce reports whether it did.
+struct alignas(16) ResultSlot {
+  union {
+    double value;
+    unsigned long long count;
+  };
+  unsigned flags;
+  unsigned ticket;
+};
+static_assert(sizeof(ResultSlot) == 16, "one 16-byte store");
 struct LossMirror {
   double* loss = nullptr;
   int* flags = nullptr;
-  unsigned long long* ticket = nullptr;
-  unsigned long long ticket_value = 0;
+  ResultSlot* slots = nullptr;
+  unsigned ticket = 0;
   unsigned long long* hits = nullptr;
 };
 int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* grad_out,
@@ -138,11 +149,10 @@ int launch_softmax_jacobian(hipStream_t s, double* jac, size_t cols);
 // hits[0] = number of rows whose first arg-max agrees
 // hits_mirror: device-visible address of a pinned host word; *mirrored tells whether the count
 // was also written there (small inputs, counted by one workgroup without atomics)
-// ticket / ticket_value: as in LossMirror, written after the mirrored count
+// slots / ticket: as in LossMirror; the mirrored count also goes to slots[1]
 int launch_accuracy(hipStream_t s, const double* pred, const double* truth, size_t rows,
                     size_t cols, unsigned long long* hits, unsigned long long* hits_mirror = nullptr,
-                    bool* mirrored = nullptr, unsigned long long* ticket = nullptr,
-                    unsigned long long ticket_value = 0);
+                    bool* mirrored = nullptr, ResultSlot* slots = nullptr, unsigned ticket = 0);
 
 int launch_fill_uniform(hipStream_t s, double* dst, size_t n, uint64_t seed, uint64_t stream,
                         double lo, double hi);
@@ -169,15 +179,16 @@ struct rst_engine {
   double* hd_loss = nullptr;
   int* hd_flags = nullptr;
   unsigned long long* hd_hits = nullptr;
-  // results are announced by a ticket: kernels that finish a scalar write the number they were
-  // given into a pinned word last, and the host polls that word (a few microseconds sooner than a
-  // stream synchronisation returns).  Tickets only grow.  loss_ticket: the ticket of the latest
-  // loss, 0 when that loss was enqueued without one (recorded into a graph, whose replays would all
-  // write the same number).
-  unsigned long long* h_ticket = nullptr;   // pinned
-  unsigned long long* hd_ticket = nullptr;  // the same word as the device addresses it
-  unsigned long long tickets_issued = 0;
-  unsigned long long loss_ticket = 0;
+  // results are announced by a ticket: a kernel that finishes a scalar writes it, with the number
+  // the launch was given, into a pinned 16-byte record, and the host polls that record (a few
+  // microseconds sooner than a stream synchronisation returns).  Tickets are never 0.  loss_ticket:
+  // the ticket of the latest loss, 0 when that loss was enqueued without one (recorded into a graph,
+  // whose replays would all write the same number); loss_with_hits: that launch also counted hits.
+  rst::ResultSlot* h_slots = nullptr;   // pinned: [0] loss, [1] hit count
+  rst::ResultSlot* hd_slots = nullptr;  // the same records as the device addresses them
+  unsigned tickets_issued = 0;
+  unsigned loss_ticket = 0;
+  bool loss_with_hits = false;
   bool loss_valid = false;
   // split-K scratch of the contraction kernels (fixed size, allocated with the engine)
   double* d_gemm_ws = nullptr;
@@ -198,9 +209,11 @@ struct rst_engine {
 
 namespace rst {
 int engine_activate(rst_engine* e);
-// waits until the kernel that was given `ticket` has written its results to the pinned words
-// (ticket 0: until the stream has drained)
-int engine_wait_ticket(rst_engine* e, unsigned long long ticket);
+// a fresh ticket (never 0)
+unsigned engine_next_ticket(rst_engine* e);
+// waits until the kernel that was given `ticket` has written the records named by `slots` (bit 0:
+// loss, bit 1: hit count); ticket 0: until the stream has drained
+int engine_wait_ticket(rst_engine* e, unsigned ticket, int slots);
 int engine_reserve_row_loss(rst_engine* e, size_t rows);
 // looks up, once per device, the address of the fixed scratch behind rst_cross_entropy_static
 int static_scratch_setup(int device, hipStream_t stream);

@@ -46,11 +46,18 @@ int engine_activate(rst_engine* e) {
   return RST_OK;
 }
 
-int engine_wait_ticket(rst_engine* e, unsigned long long ticket) {
+unsigned engine_next_ticket(rst_engine* e) {
+  if (++e->tickets_issued == 0) ++e->tickets_issued;
+  return e->tickets_issued;
+}
+
+int engine_wait_ticket(rst_engine* e, unsigned ticket, int slots) {
   if (ticket != 0) {
     // about 100 us of polling; a result that takes longer is waited for the ordinary way
     for (int i = 0; i < 4000; ++i) {
-      if (__atomic_load_n(e->h_ticket, __ATOMIC_ACQUIRE) >= ticket) return RST_OK;
+      const bool loss_there = !(slots & 1) || __atomic_load_n(&e->h_slots[0].ticket, __ATOMIC_ACQUIRE) == ticket;
+      const bool hits_there = !(slots & 2) || __atomic_load_n(&e->h_slots[1].ticket, __ATOMIC_ACQUIRE) == ticket;
+      if (loss_there && hits_there) return RST_OK;
       _mm_pause();
     }
   }
@@ -117,10 +124,9 @@ int rst_engine_create(int device, rst_engine** out) {
   if (err == hipSuccess) err = hipHostMalloc(&e->h_flags, 4 * sizeof(int), hipHostMallocDefault);
   if (err == hipSuccess)
     err = hipHostMalloc(&e->h_hits, sizeof(unsigned long long), hipHostMallocDefault);
-  if (err == hipSuccess)
-    err = hipHostMalloc(&e->h_ticket, sizeof(unsigned long long), hipHostMallocDefault);
-  if (err == hipSuccess) err = hipHostGetDevicePointer((void**)&e->hd_ticket, e->h_ticket, 0);
-  if (err == hipSuccess) *e->h_ticket = 0;
+  if (err == hipSuccess) err = hipHostMalloc(&e->h_slots, 2 * sizeof(ResultSlot), hipHostMallocDefault);
+  if (err == hipSuccess) err = hipHostGetDevicePointer((void**)&e->hd_slots, e->h_slots, 0);
+  if (err == hipSuccess) std::memset(e->h_slots, 0, 2 * sizeof(ResultSlot));
   if (err == hipSuccess) err = hipHostGetDevicePointer((void**)&e->hd_loss, e->h_loss, 0);
   if (err == hipSuccess) err = hipHostGetDevicePointer((void**)&e->hd_flags, e->h_flags, 0);
   if (err == hipSuccess) err = hipHostGetDevicePointer((void**)&e->hd_hits, e->h_hits, 0);
@@ -162,7 +168,7 @@ int rst_engine_destroy(rst_engine* e) {
   if (e->h_loss) (void)hipHostFree(e->h_loss);
   if (e->h_flags) (void)hipHostFree(e->h_flags);
   if (e->h_hits) (void)hipHostFree(e->h_hits);
-  if (e->h_ticket) (void)hipHostFree(e->h_ticket);
+  if (e->h_slots) (void)hipHostFree(e->h_slots);
   if (e->stream) (void)hipStreamDestroy(e->stream);
   delete e;
   return RST_OK;

@@ -237,6 +237,20 @@ RST_HD PairSource staged_pair_source(int q, long ld, int ext0, int ext_n, int k0
 // row row0 + 16*i + 4*r + lk, column col0 + 16*j + lr (lr = lane % 16, lk = lane / 16).
 RST_HD int acc_row(int row0, int i, int r, int lk) { return row0 + i * 16 + 4 * r + lk; }
 RST_HD int acc_col(int col0, int j, int lr) { return col0 + j * 16 + lr; }
+// How many of the tm x tn fragments (16 x 16) of a wavefront block at (row0, col0) reach into an
+// M x N output: rows of fragments and columns of fragments (0 x 0 when the block is wholly outside).
+struct LiveFragments {
+  int rows, cols;
+};
+RST_HD LiveFragments live_fragments(int M, int N, int row0, int col0, int tm, int tn) {
+  LiveFragments l;
+  l.rows = row0 < M ? (M - row0 + 15) / 16 : 0;
+  l.cols = col0 < N ? (N - col0 + 15) / 16 : 0;
+  if (l.rows > tm) l.rows = tm;
+  if (l.cols > tn) l.cols = tn;
+  if (l.rows == 0 || l.cols == 0) l.rows = l.cols = 0;
+  return l;
+}
 // A block of TM x TN fragments that lies wholly inside the output takes the unpredicated epilogue,
 // whose lane offsets are 32-bit: every leading dimension involved must stay below 2^26 doubles.
 RST_HD bool block_is_interior(const GemmParams& p, int row0, int col0, int tm, int tn) {

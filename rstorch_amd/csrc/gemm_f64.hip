@@ -578,7 +578,11 @@ __device__ __forceinline__ void read_quad(v2d& q, uint32_t addr) {
 // are the workgroup's STAGES operand stages (A_SIZE / B_SIZE doubles each, at most kDmaStage).
 constexpr int kDmaStage = BK * (128 + 16);  // the larger of the two tile layouts
 
-template <bool A_KC, bool B_KC, int WGM, int WGN, int STAGES, int DIST>
+// RAGGED: a wavefront multiplies only the 16x16 fragments of its 64x32 block that reach into the
+// output (wave-uniform tests around the MFMAs).  For grids of few tiles around narrow outputs - a
+// 100 x 784 weight gradient - where the fragments beyond the edge are a fifth of the work; the
+// large products leave it off and keep their instruction stream free of branches.
+template <bool A_KC, bool B_KC, int WGM, int WGN, int STAGES, int DIST, bool RAGGED = false>
 __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double* __restrict__ lds_a,
                                          double* __restrict__ lds_b) {
   constexpr int BM = 128, BN = 128, NW = WGM * WGN;
@@ -717,9 +721,18 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
   v2d fa[4], fb[2][2];  // A fragments (single set), B fragments [buffer][j]
   auto a_addr = [&](int stage, int s2) { return a_base + (uint32_t)stage * (A_SIZE * 8) + a_off[s2]; };
   auto b_addr = [&](int stage, int s2) { return b_base + (uint32_t)stage * (B_SIZE * 8) + b_off[s2]; };
+  // fragments of this wavefront's block that reach into the output: rows of 16 and columns of 16
+  int tm_live = TM, tn_live = TN;
+  if (RAGGED) {
+    const LiveFragments live = live_fragments(p.M, p.N, m0 + wm * WM, n0 + wn * WN, TM, TN);
+    tm_live = __builtin_amdgcn_readfirstlane(live.rows);
+    tn_live = __builtin_amdgcn_readfirstlane(live.cols);
+  }
   auto mfma_row = [&](int i, double a, double b0, double b1) {
-    acc[i][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b0, acc[i][0], 0, 0, 0);
-    acc[i][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b1, acc[i][1], 0, 0, 0);
+    if (!RAGGED || i < tm_live) {
+      acc[i][0] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b0, acc[i][0], 0, 0, 0);
+      if (!RAGGED || tn_live > 1) acc[i][1] = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b1, acc[i][1], 0, 0, 0);
+    }
   };
   // first step of a pair: the six reads B0 B1 A0 A1 A2 A3 are outstanding in that order
   auto first_step = [&](int bb) {
@@ -809,7 +822,7 @@ __global__ __launch_bounds__(512, 4) void gemm_f64_mfma_dma_group(const GemmGrou
   __shared__ __attribute__((aligned(1024))) double lds_a[2 * kDmaStage];
   __shared__ __attribute__((aligned(1024))) double lds_b[2 * kDmaStage];
   const int i = group_member_of_block(g.first_block, g.count, (int)blockIdx.x);
-  dma_tile<false, false, 2, 4, 2, 1>(g.p[i], (int)blockIdx.x - g.first_block[i], lds_a, lds_b);
+  dma_tile<false, false, 2, 4, 2, 1, true>(g.p[i], (int)blockIdx.x - g.first_block[i], lds_a, lds_b);
 }
 
 // ---- 64x64 tiles fed by direct global -> LDS loads ---------------------------------------------
@@ -1423,13 +1436,30 @@ bool dma_group_member(const GemmDesc& d) {
          d.workspace != nullptr;
 }
 
-// Plans d[0..count) as one grid of sliced 128x128 tiles: every member gets the same number of
-// slices, the one that brings the grid to about one workgroup per CU (two per CU measured 4 % slower
-// on the step), shortened where a member's contraction would leave a slice fewer than
-// kDmaGroupMinSteps K steps.  False when the members do not qualify, the tiles would be mostly
-// padding, the grid would leave more than a quarter of the chip idle (batches below about 4096 for
-// a handful of tiles), or the workspace is too small.  *ws_need: doubles of the shared workspace
-// that the plan takes.
+// MFMAs per K step of 4 that the busiest SIMD of a 128x128 workgroup issues when only me x ne of its
+// outputs exist (the kernel skips fragments beyond the edge): wavefronts w and w + 4 share a SIMD.
+// 16 for a full tile.
+int ragged_tile_cost(int me, int ne) {
+  int worst = 0;
+  for (int simd = 0; simd < 4; ++simd) {
+    int c = 0;
+    for (int w = simd; w < 8; w += 4) {
+      const LiveFragments live = live_fragments(me, ne, (w / 4) * 64, (w % 4) * 32, 4, 2);
+      c += live.rows * live.cols;
+    }
+    if (c > worst) worst = c;
+  }
+  return worst;
+}
+
+// Plans d[0..count) as one grid of K-sliced 128x128 tiles of about one workgroup per CU (two per CU
+// measured 4 % slower on the step).  The kernel skips the MFMA fragments beyond a tile's edge, so a
+// tile costs what its busiest SIMD issues (ragged_tile_cost); a member is cut into as many slices as
+// its cost says, so that all workgroups of the grid take about equally long, and the narrow last tile
+// column of a member (784 = 6 x 128 + 16) becomes a piece of its own with fewer, longer slices.
+// False when the members do not qualify, the tiles would be mostly padding, the grid would leave more
+// than a quarter of the chip idle (batches below about 4096 for a handful of tiles), or the
+// workspace is too small.  *ws_need: doubles of the shared workspace that the plan takes.
 bool plan_dma_group(const GemmDesc* d, int count, GemmGroup* g, long long* blocks_out, long long* reduce_out,
                     size_t* ws_need = nullptr) {
   if (dma_group_mode() == 0) return false;
@@ -1445,19 +1475,56 @@ bool plan_dma_group(const GemmDesc* d, int count, GemmGroup* g, long long* block
   // tiles' area in use (784-100-100-10) the step is 6 % shorter than on the 32x32 group (13 % at
   // batch 32768), with 90 % (256-256-256-10) 7 %; with 41 % (1024-64-64-64-16) it is 9 % longer.
   if (dma_group_mode() != 1 && outputs < 0.55 * 16384.0 * (double)tiles) return false;
-  long long want = kDmaGroupGrid / tiles;
-  if (want > kDmaGroupMaxSlices) want = kDmaGroupMaxSlices;
+  // the pieces: every member, minus a cheap last tile column that goes on its own
+  GemmDesc piece[kMaxGroup];
+  int cost[kMaxGroup];
+  int pieces = 0;
+  for (int i = 0; i < count; ++i) {
+    const GemmDesc& m = d[i];
+    const int me = m.M < 128 ? m.M : 128;
+    const int rem = m.N % 128;
+    const int spare = kMaxGroup - pieces - (count - i);  // slots left once every later member has one
+    if (m.N > 128 && rem != 0 && spare >= 1 && 2 * ragged_tile_cost(me, rem) <= ragged_tile_cost(me, 128)) {
+      GemmDesc head = m, tail = m;
+      head.N = m.N - rem;
+      tail.N = rem;
+      tail.B = m.B + head.N;  // both operands of a weight gradient are output-contiguous: a column offset
+      tail.C = m.C + head.N;
+      if (m.sgd_parm) tail.sgd_parm = m.sgd_parm + head.N;
+      tail.colsum = nullptr;  // the column sums of A belong to the piece that holds tile column 0
+      tail.sgd_bias = nullptr;
+      cost[pieces] = ragged_tile_cost(me, 128);
+      piece[pieces++] = head;
+      cost[pieces] = ragged_tile_cost(me, rem);
+      piece[pieces++] = tail;
+    } else {
+      cost[pieces] = ragged_tile_cost(me, m.N < 128 ? m.N : 128);
+      piece[pieces++] = m;
+    }
+  }
+  int cost_max = 1;
+  double weight = 0.0;
+  for (int i = 0; i < pieces; ++i) {
+    // a K step costs a workgroup at least its barrier and the wait for the next tile, about what
+    // six MFMAs per SIMD take (measured: 0.8 us against 2.2 us for a full tile's sixteen)
+    if (cost[i] < 6) cost[i] = 6;
+    if (cost[i] > cost_max) cost_max = cost[i];
+    weight += (double)cost[i] * (double)(((piece[i].M + 127) / 128) * ((piece[i].N + 127) / 128));
+  }
+  const double full_slices = (double)kDmaGroupGrid * (double)cost_max / weight;  // of a piece of the highest cost
   long long blocks = 0, reduce_blocks = 0;
   size_t ws_used = 0;
-  g->count = count;
-  for (int i = 0; i < count; ++i) {
-    GemmParams p = make_params(d[i]);
+  g->count = pieces;
+  for (int i = 0; i < pieces; ++i) {
+    GemmParams p = make_params(piece[i]);
     p.tiles_m = (p.M + 127) / 128;
     p.tiles_n = (p.N + 127) / 128;
     const int nk = p.K / BK;
-    long long s = want;
+    long long s = (long long)(full_slices * (double)cost[i] / (double)cost_max + 0.5);
+    if (s > kDmaGroupMaxSlices) s = kDmaGroupMaxSlices;
     if (s > nk / kDmaGroupMinSteps) s = nk / kDmaGroupMinSteps;
-    if (s < 2) return false;
+    if (s < 2) s = 2;
+    if (nk / s < 1) return false;
     p.steps_per_split = (int)((nk + s - 1) / s);
     p.split_k = (nk + p.steps_per_split - 1) / p.steps_per_split;
     if (p.split_k < 2) return false;
@@ -1473,8 +1540,8 @@ bool plan_dma_group(const GemmDesc* d, int count, GemmGroup* g, long long* block
     reduce_blocks += (long long)(((size_t)p.M * p.N + 255) / 256);
     g->p[i] = p;
   }
-  g->first_block[count] = (int)blocks;
-  g->first_reduce_block[count] = (int)reduce_blocks;
+  g->first_block[pieces] = (int)blocks;
+  g->first_reduce_block[pieces] = (int)reduce_blocks;
   if (dma_group_mode() != 1 && blocks < (3 * kDmaGroupGrid) / 4) return false;
   *blocks_out = blocks;
   *reduce_out = reduce_blocks;

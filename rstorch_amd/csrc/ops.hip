@@ -15,10 +15,14 @@ __global__ void reset_softmax_flag_kernel(int* flags) { flags[2] = 0; }
 // enqueues the arg-max agreement count of pred / truth and waits until it is in the pinned hit word
 int engine_accuracy(rst_engine* e, const double* pred, const double* truth, size_t rows, size_t cols) {
   bool mirrored = false;
-  const unsigned long long ticket = ++e->tickets_issued;
-  RST_TRY(launch_accuracy(e->stream, pred, truth, rows, cols, e->d_hits, e->hd_hits, &mirrored, e->hd_ticket,
+  const unsigned ticket = engine_next_ticket(e);
+  RST_TRY(launch_accuracy(e->stream, pred, truth, rows, cols, e->d_hits, e->hd_hits, &mirrored, e->hd_slots,
                           ticket));
-  if (mirrored) return engine_wait_ticket(e, ticket);
+  if (mirrored) {
+    RST_TRY(engine_wait_ticket(e, ticket, 2));
+    *e->h_hits = e->h_slots[1].count;  // (the record and the plain word hold the same count; only the record is certain to be there)
+    return RST_OK;
+  }
   RST_HIP(hipMemcpyAsync(e->h_hits, e->d_hits, sizeof(unsigned long long), hipMemcpyDeviceToHost,
                          e->stream));
   RST_HIP(hipStreamSynchronize(e->stream));
@@ -48,13 +52,15 @@ int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, co
   hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
   RST_HIP(hipStreamIsCapturing(e->stream, &capture));
   e->loss_ticket = 0;
+  e->loss_with_hits = false;
   if (capture == hipStreamCaptureStatusNone) {
-    mirror.ticket = e->hd_ticket;
-    mirror.ticket_value = e->loss_ticket = ++e->tickets_issued;
+    mirror.slots = e->hd_slots;
+    mirror.ticket = e->loss_ticket = engine_next_ticket(e);
   }
   if (hits_done) mirror.hits = e->hd_hits;
   RST_TRY(launch_softmax_ce(e->stream, pred, truth, grad_out, prob_out, row_loss, e->d_loss,
                             e->d_flags, rows, cols, mirror, hits_done));
+  e->loss_with_hits = hits_done && *hits_done;
   e->loss_valid = true;
   if (host_loss) return rst_loss_value(e, host_loss);
   return RST_OK;
@@ -224,9 +230,17 @@ int rst_loss_value(rst_engine* e, double* host_loss) {
   if (!host_loss) return fail(RST_ERR_INVALID_ARGUMENT, "host_loss is null");
   if (!e->loss_valid) return fail(RST_ERR_STATE, "no loss has been computed on this engine");
   // the kernel that finished the loss stored it, and the NaN flag, in the pinned words as well
-  RST_TRY(engine_wait_ticket(e, e->loss_ticket));
-  *host_loss = *static_cast<volatile double*>(e->h_loss);
-  if (static_cast<volatile int*>(e->h_flags)[1] & 1)
+  RST_TRY(engine_wait_ticket(e, e->loss_ticket, e->loss_with_hits ? 3 : 1));
+  int nan_flag;
+  if (e->loss_ticket != 0) {  // announced by ticket: the record is certain to be there
+    *host_loss = static_cast<volatile ResultSlot*>(e->h_slots)[0].value;
+    nan_flag = (int)static_cast<volatile ResultSlot*>(e->h_slots)[0].flags;
+    if (e->loss_with_hits) *e->h_hits = static_cast<volatile ResultSlot*>(e->h_slots)[1].count;
+  } else {                    // the stream has drained: the plain words are there
+    *host_loss = *static_cast<volatile double*>(e->h_loss);
+    nan_flag = static_cast<volatile int*>(e->h_flags)[1];
+  }
+  if (nan_flag & 1)
     return fail(RST_ERR_NAN, "cross entropy: NaN logits (the reference panics in softmax.rs:38)");
   return RST_OK;
 }

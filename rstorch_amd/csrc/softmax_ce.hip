@@ -48,8 +48,8 @@ __device__ __forceinline__ double group_reduce(double v, double* scratch) {
 }
 
 // The thread that finishes a loss also stores it, the NaN flag and (if counted) the arg-max hits in
-// pinned host words, and announces them with the launch's ticket, written last behind a
-// system-scope fence: a host that sees the ticket sees the results.
+// pinned host memory: in plain words (read after a stream synchronisation) and, when the launch has
+// a ticket, in the 16-byte records that the host polls (see store_result_slot).
 __device__ __forceinline__ void publish(const LossMirror& mirror, double loss, int nan_flag, bool counted,
                                         unsigned long long hits) {
   if (mirror.loss) {
@@ -57,9 +57,9 @@ __device__ __forceinline__ void publish(const LossMirror& mirror, double loss, i
     mirror.flags[1] = nan_flag;
   }
   if (counted) mirror.hits[0] = hits;
-  if (mirror.ticket) {
-    __threadfence_system();
-    mirror.ticket[0] = mirror.ticket_value;
+  if (mirror.slots) {
+    if (counted) store_result_slot(mirror.slots + 1, (double)0, hits, true, 0u, mirror.ticket);
+    store_result_slot(mirror.slots, loss, 0ull, false, (unsigned)nan_flag, mirror.ticket);
   }
 }
 

@@ -327,8 +327,7 @@ __global__ __launch_bounds__(1024) void accuracy_small_kernel(const double* __re
                                                              size_t rows, size_t cols,
                                                              unsigned long long* hits,
                                                              unsigned long long* hits_mirror,
-                                                             unsigned long long* ticket,
-                                                             unsigned long long ticket_value) {
+                                                             ResultSlot* slots, unsigned ticket) {
   __shared__ unsigned counts[16];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   unsigned mine = 0;
@@ -344,20 +343,17 @@ __global__ __launch_bounds__(1024) void accuracy_small_kernel(const double* __re
     for (int w = 0; w < 16; ++w) total += counts[w];
     hits[0] = total;
     if (hits_mirror) hits_mirror[0] = total;
-    if (ticket) {  // announced last: a host that sees the ticket sees the count
-      __threadfence_system();
-      ticket[0] = ticket_value;
-    }
+    if (slots) store_result_slot(slots + 1, 0.0, total, true, 0u, ticket);
   }
 }
 
 int launch_accuracy(hipStream_t s, const double* pred, const double* truth, size_t rows,
                     size_t cols, unsigned long long* hits, unsigned long long* hits_mirror,
-                    bool* mirrored, unsigned long long* ticket, unsigned long long ticket_value) {
+                    bool* mirrored, ResultSlot* slots, unsigned ticket) {
   if (mirrored) *mirrored = false;
   if (hits_mirror && mirrored && rows * cols <= (size_t)1 << 16) {
     hipLaunchKernelGGL(accuracy_small_kernel, dim3(1), dim3(1024), 0, s, pred, truth, rows, cols, hits,
-                       hits_mirror, ticket, ticket_value);
+                       hits_mirror, slots, ticket);
     RST_HIP(hipGetLastError());
     *mirrored = true;
     return RST_OK;

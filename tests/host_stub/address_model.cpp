@@ -162,7 +162,10 @@ void check_staged_k_cover(const GemmParams& p) {
 }
 
 // ---- epilogue of one wavefront block (write_block<TM, TN>) ------------------------------------------------
-void check_write_block(const GemmParams& p, int tm, int tn, int row0, int col0, int split, Coverage& cov) {
+// live != NULL: the kernel skips the MFMAs of fragments beyond live->rows x live->cols, so nothing that
+// is stored may sit in one of those
+void check_write_block(const GemmParams& p, int tm, int tn, int row0, int col0, int split, Coverage& cov,
+                       const LiveFragments* live = nullptr) {
   const size_t c_limit = (size_t)(p.M - 1) * (size_t)p.ldc + (size_t)p.N;
   const size_t mask_limit = (size_t)(p.M - 1) * (size_t)p.ldmask + (size_t)p.N;
   const bool interior = block_is_interior(p, row0, col0, tm, tn);
@@ -193,6 +196,7 @@ void check_write_block(const GemmParams& p, int tm, int tn, int row0, int col0, 
                                 interior_lane_offset<uint64_t>(lk, lr, ld_out) / 8 + (size_t)16 * j;
             if (elem != (size_t)row * (size_t)ld_out + (size_t)col) bad("interior store address does not name (row, col)");
             in_range("interior store", elem, 1, out_limit);
+            if (live && (i >= live->rows || j >= live->cols)) bad("a stored element sits in a fragment whose MFMAs are skipped");
             cov.mark(split, row, col);
             if (!sliced && p.epilogue == 4) {
               const size_t me = (size_t)acc_row(row0, i, r, 0) * (size_t)p.ldmask + (size_t)col0 +
@@ -208,6 +212,7 @@ void check_write_block(const GemmParams& p, int tm, int tn, int row0, int col0, 
             if (!sliced && (p.epilogue == 1 || p.epilogue == 2)) in_range("bias read", (size_t)cc, 1, (size_t)p.N);
             if (row < p.M && col < p.N) {
               in_range("store", (size_t)row * (size_t)ld_out + (size_t)col, 1, out_limit);
+              if (live && (i >= live->rows || j >= live->cols)) bad("a stored element sits in a fragment whose MFMAs are skipped");
               cov.mark(split, row, col);
             }
           }
@@ -322,7 +327,7 @@ void check_tail_tile(const char* name, const double* base, int threads, long ld,
 }
 
 // all workgroups of one problem on 128x128 direct-to-LDS tiles (8 wavefronts of 64x32)
-void check_dma128_problem(const GemmParams& p, bool a_kc, bool b_kc, long long blocks) {
+void check_dma128_problem(const GemmParams& p, bool a_kc, bool b_kc, long long blocks, bool ragged = false) {
   g_context = std::string("dma128 ") + describe(p, a_kc, b_kc);
   check_params(p, a_kc, b_kc);
   if (p.tiles_m != (p.M + 127) / 128 || p.tiles_n != (p.N + 127) / 128) bad("tile counts do not match 128x128 tiles");
@@ -356,7 +361,8 @@ void check_dma128_problem(const GemmParams& p, bool a_kc, bool b_kc, long long b
     }
     for (int wave = 0; wave < 8; ++wave) {
       const int wm = wave / 4, wn = wave % 4;
-      check_write_block(p, 4, 2, m0 + wm * 64, n0 + wn * 32, tc.split, cov);
+      const LiveFragments live = live_fragments(p.M, p.N, m0 + wm * 64, n0 + wn * 32, 4, 2);
+      check_write_block(p, 4, 2, m0 + wm * 64, n0 + wn * 32, tc.split, cov, ragged ? &live : nullptr);
     }
     check_colsum(p, a_kc, 128, 512, m0, tc.tile_n, tc.split, want_colsum ? &colsums : nullptr);
   }
@@ -601,7 +607,7 @@ void observe_gemm_launch(const GemmLaunch& l) {
       check_group_blocks(*l.group, l.group->first_block, l.blocks);
       check_group_workspace(*l.group);
       for (int i = 0; i < l.group->count; ++i)
-        check_dma128_problem(l.group->p[i], false, false, l.group->first_block[i + 1] - l.group->first_block[i]);
+        check_dma128_problem(l.group->p[i], false, false, l.group->first_block[i + 1] - l.group->first_block[i], true);
       break;
     }
     case GemmKernel::kStagedGroup:
