@@ -53,3 +53,12 @@ def test_hip_flags_disable_packed_fp32_and_contraction():
     from rstorch_amd import _build
     flags = " ".join(_build.HIP_FLAGS)
     assert "-packed-fp32-ops" in flags and "-ffp-contract=off" in flags and "gfx950" in flags
+
+
+def test_traffic_figure_belongs_to_the_current_kernel_sources():
+    """bench.py reports roofline.traffic from a committed counter profile (profiles/c4_hbm_traffic.md);
+    the figure is only valid for the kernel sources it was measured on.  When this fails, collect the
+    profile again and update C4_TRAFFIC_BYTES_PER_LAUNCH and the digest in bench.py."""
+    sys.path.insert(0, ROOT)
+    import bench
+    assert bench.kernel_sources_digest() == bench.C4_TRAFFIC_SOURCE["kernel_sources_sha16"]
