@@ -345,6 +345,27 @@ def time_fresh_steps(rs, eng, loader, dm, batch, normal, steps, warmup, read_los
     return wall, dm.last_loss()
 
 
+def time_generated_in_stream(eng, dm, batch, normal, steps, warmup):
+    """Steps on fresh inputs without a second stream: the counter generator refills the one batch on
+    the training stream ahead of every step, so its time is inside the step and no event is needed."""
+    from rstorch_amd import _ffi
+    x, y = eng.empty(batch, dm.in_width), eng.empty(batch, dm.out_width)
+    fill = eng.lib.rst_fill_normal if normal else eng.lib.rst_fill_uniform
+
+    def run(first, count):
+        for k in range(first, first + count):
+            _ffi.check(fill(eng.handle, x.ptr, x.size, SEED, 1000 + 2 * k, 0.0, 1.0))
+            _ffi.check(eng.lib.rst_fill_one_hot(eng.handle, y.ptr, batch, dm.out_width, SEED, 1001 + 2 * k))
+            dm.train_step(x, y, LR, want_loss=False)
+        eng.synchronize()
+
+    run(0, warmup)
+    t0 = time.perf_counter()
+    run(warmup, steps)
+    wall = time.perf_counter() - t0
+    return wall, dm.last_loss()
+
+
 def bench_small(rs, eng, spec, batch, normal, steps, warmup, eager, profile_steps, fresh_inputs=False):
     """steps_per_s: the fused step as shipped (graph replay unless --eager).  `contractions`: a
     second pass with an event after every launch (plain launches, one weight gradient per layer)."""
@@ -360,6 +381,12 @@ def bench_small(rs, eng, spec, batch, normal, steps, warmup, eager, profile_step
         wall_read, loss_read = time_fresh_steps(rs, eng, loader, dm, batch, normal, steps, warmup, True)
         out["with_loss_read_every_step"] = {"ms_per_step": wall_read * 1e3 / steps, "steps_per_s": steps / wall_read,
                                             "final_loss": loss_read}
+        wall_gen, loss_gen = time_generated_in_stream(eng, dm, batch, normal, steps, warmup)
+        out["generator_on_the_training_stream"] = {
+            "ms_per_step": wall_gen * 1e3 / steps, "steps_per_s": steps / wall_gen, "final_loss": loss_gen,
+            "note": "no second stream and no events: the generator's launches run ahead of every step on the "
+                    "training stream, their time inside the step; at these sizes the two event hand-overs of the "
+                    "two-stream protocol cost more than the generator takes"}
         wall_one, _, loss_one, _ = time_steps(eng, dm, x, y, steps, warmup, False)
         out["one_resident_batch"] = {"ms_per_step": wall_one * 1e3 / steps, "steps_per_s": steps / wall_one,
                                      "final_loss": loss_one}
