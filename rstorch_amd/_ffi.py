@@ -117,6 +117,7 @@ SIGNATURES = {
     "rst_model_profile_enable": [_vp, _i32],
     "rst_model_graph_enable": [_vp, _i32],
     "rst_model_fuse_sgd": [_vp, _i32],
+    "rst_model_fuse_head": [_vp, _i32],
     "rst_model_pair_gradients": [_vp, _i32],
     "rst_model_profile_read": [_vp, ctypes.POINTER(KernelRecord), _sz, c_size_p],
 }

@@ -143,6 +143,17 @@ struct LossMirror {
 int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* grad_out,
                       double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,
                       size_t cols, LossMirror mirror = LossMirror(), bool* hits_done = nullptr);
+// The classifier head of a training step in one launch: logits = h.w^T + bias ([rows, cols], h is
+// [rows, in_features] with contiguous rows), cross entropy against truth with grad = -(truth - p),
+// dx = grad.w (NULL: not wanted; mask: zeroed where h <= 0, the backward of a ReLU that produced h)
+// and the loss, finished by the workgroup that arrives last (flags[4..5], one 64-bit word, counts
+// arrivals and is left at zero; flags[1], loss and the mirror as for launch_softmax_ce; row_loss is
+// [rows] scratch).  Only for shapes
+// head_ce_supported accepts: few classes on few inputs, where the weight matrix sits in LDS.
+bool head_ce_supported(size_t cols, size_t in_features);
+int launch_head_ce(hipStream_t s, const double* h, const double* w, const double* bias, const double* truth,
+                   double* logits, double* grad, double* dx, bool mask, double* row_loss, double* loss,
+                   int* flags, size_t rows, size_t cols, size_t in_features, LossMirror mirror = LossMirror());
 int launch_softmax_columns(hipStream_t s, const double* z, double* out, int* flags, size_t rows,
                            size_t cols);
 int launch_softmax_jacobian(hipStream_t s, double* jac, size_t cols);
@@ -224,4 +235,8 @@ int static_scratch_setup(int device, hipStream_t stream);
 int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, const double* truth,
                          double* grad_out, double* prob_out, size_t rows, size_t cols,
                          double* host_loss, bool* hits_done = nullptr);
+// the fused classifier head (launch_head_ce) with the engine's loss words, mirror and ticket
+int engine_head_cross_entropy(rst_engine* e, double* row_loss, const double* h, const double* w,
+                              const double* bias, const double* truth, double* logits, double* grad,
+                              double* dx, bool mask, size_t rows, size_t cols, size_t in_features);
 }  // namespace rst

@@ -116,7 +116,7 @@ int rst_engine_create(int device, rst_engine** out) {
   hipError_t err = hipGetDeviceProperties(&e->props, device);
   if (err == hipSuccess) err = hipStreamCreateWithFlags(&e->stream, hipStreamNonBlocking);
   if (err == hipSuccess) err = hipMalloc(&e->d_loss, sizeof(double));
-  if (err == hipSuccess) err = hipMalloc(&e->d_flags, 4 * sizeof(int));
+  if (err == hipSuccess) err = hipMalloc(&e->d_flags, 8 * sizeof(int));
   if (err == hipSuccess) err = hipMalloc(&e->d_hits, sizeof(unsigned long long));
   e->gemm_ws_count = (size_t)16 << 20;  // 16 Mi doubles = 128 MiB
   if (err == hipSuccess) err = hipMalloc(&e->d_gemm_ws, e->gemm_ws_count * sizeof(double));
@@ -135,7 +135,7 @@ int rst_engine_create(int device, rst_engine** out) {
     e->h_flags[0] = e->h_flags[1] = e->h_flags[2] = e->h_flags[3] = 0;
     *e->h_hits = 0;
   }
-  if (err == hipSuccess) err = hipMemsetAsync(e->d_flags, 0, 4 * sizeof(int), e->stream);
+  if (err == hipSuccess) err = hipMemsetAsync(e->d_flags, 0, 8 * sizeof(int), e->stream);
   if (err != hipSuccess) {
     int status = fail_hip(err, "engine set-up", __FILE__, __LINE__);
     rst_engine_destroy(e);

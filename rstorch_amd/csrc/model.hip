@@ -94,6 +94,9 @@ struct rst_model {
   // backward launches a layer's weight gradient together with the next layer's input gradient when
   // both are large (C4: a pair takes 0.946 ms against 0.477 + 0.503 ms for the two launches apart)
   bool pair_gradients = true;
+  // train_step runs a small classifier head (last Linear, cross entropy, that Linear's input
+  // gradient) as one launch when the shape allows it
+  bool fuse_head = true;
   // profiling
   bool profiling = false;
   bool slot_open = false;
@@ -113,6 +116,12 @@ constexpr size_t kMaxStepGraphs = 64;
 // launches are handy for debuggers and for comparing the two launch modes from outside).
 bool default_graph_enabled() {
   const char* v = std::getenv("RSTORCH_GRAPH");
+  return !(v && v[0] == '0');
+}
+
+// Whether train_step hands a small classifier head to the fused launch: yes, unless RSTORCH_HEAD=0.
+bool default_head_enabled() {
+  const char* v = std::getenv("RSTORCH_HEAD");
   return !(v && v[0] == '0');
 }
 
@@ -210,7 +219,9 @@ int next_non_identity(const rst_model* m, int i) {
 // final_out != NULL: the last layer that computes anything writes there instead of into the model's
 // own buffer (the caller's array that Sequential::forward returns by value; backward reads it again
 // as the mask of a trailing ReLU, so it must stay as it is until then).
-int do_forward(rst_model* m, const double* x, size_t batch, double* final_out = nullptr) {
+// head >= 0: that layer, the last Linear, is left to the fused head launch (do_head), which also
+// computes the loss: its input is noted, nothing is launched for it.
+int do_forward(rst_model* m, const double* x, size_t batch, double* final_out = nullptr, int head = -1) {
   rst_engine* e = m->engine;
   if (batch > (size_t)INT_MAX) return fail(RST_ERR_UNSUPPORTED, "batch too large");
   RST_TRY(reserve_activations(m, batch));
@@ -235,6 +246,10 @@ int do_forward(rst_model* m, const double* x, size_t batch, double* final_out = 
       const bool fuse = nx >= 0 && m->layers[nx].kind == RST_LAYER_RELU;
       l.input = cur;  // linear.rs:56 keeps the input for backward
       l.relu_fused = fuse;
+      if (i == head) {
+        cur = dest;
+        continue;
+      }
       GemmDesc d{};
       d.A = cur; d.B = l.w; d.C = dest;
       d.M = (int)batch; d.N = (int)l.out; d.K = (int)l.in;
@@ -285,13 +300,44 @@ int do_loss(rst_model* m, const double* truth, double* host_loss) {
   return RST_OK;
 }
 
+// The layer that train_step can hand to the fused head launch, or -1: the last layer that is not an
+// Identity, if it is a Linear whose shape the head kernel takes.
+int head_layer(const rst_model* m) {
+  if (!m->fuse_head) return -1;
+  const int i = prev_non_identity(m, (int)m->layers.size());
+  if (i < 0 || m->layers[i].kind != RST_LAYER_LINEAR) return -1;
+  return head_ce_supported(m->layers[i].out, m->layers[i].in) ? i : -1;
+}
+
+// Forward of the head Linear, the loss with its gradient and, unless the head is the first Linear
+// (whose input gradient train_step does not need), the head's input gradient: one launch.
+int do_head(rst_model* m, int head, const double* truth) {
+  rst_engine* e = m->engine;
+  if (!truth) return fail(RST_ERR_INVALID_ARGUMENT, "truth is null");
+  Layer& l = m->layers[head];
+  const size_t rows = m->batch;
+  bool wanted = false;
+  for (int i = 0; i < head; ++i) wanted |= m->layers[i].kind == RST_LAYER_LINEAR;
+  const int pv = prev_non_identity(m, head);
+  const bool mask = pv >= 0 && m->layers[pv].kind == RST_LAYER_RELU;
+  const double work = (double)rows * (double)l.in * (double)l.out;
+  RST_TRY(prof_begin(m, RST_KERNEL_CROSS_ENTROPY, head, (wanted ? 4.0 : 2.0) * work,
+                     8.0 * ((double)rows * l.in * (wanted ? 2.0 : 1.0) + 3.0 * (double)rows * l.out)));
+  RST_TRY(engine_head_cross_entropy(e, m->row_loss, l.input, l.w, l.b, truth, l.out_buf, m->loss_grad,
+                                    wanted ? l.grad_in_buf : nullptr, mask, rows, l.out, l.in));
+  RST_TRY(prof_end(m));
+  m->loss_grad_valid = true;
+  return RST_OK;
+}
+
 // fused_lr != NULL: every weight-gradient launch also applies the SGD update to its layer
 // (the input gradient, which needs the old weights, is launched first).
 // input_grad_dest != NULL (with need_input_grad): the gradient with respect to the model's input is
 // written there (the caller's array that Sequential::backward returns by value) instead of into the
 // model's own buffer.
+// head >= 0: the input gradient of that Linear (the last one) has been written by do_head already.
 int do_backward(rst_model* m, const double* grad, int need_input_grad, const double** input_grad,
-                const double* fused_lr, double* input_grad_dest = nullptr) {
+                const double* fused_lr, double* input_grad_dest = nullptr, int head = -1) {
   rst_engine* e = m->engine;
   if (!m->forward_valid)
     return fail(RST_ERR_STATE, "backward without a forward (the reference panics on a consumed cache)");
@@ -413,7 +459,9 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
       dx_bytes = 8.0 * ((double)batch * l.out + (double)l.in * l.out +
                         (double)batch * l.in * (mask ? 2.0 : 1.0));
     }
-    if (pend.active && wanted && m->pair_gradients && can_pair_gemm(dx, pend.d)) {
+    if (i == head) {
+      // (nothing is pending: the head is the first layer this loop meets)
+    } else if (pend.active && wanted && m->pair_gradients && can_pair_gemm(dx, pend.d)) {
       RST_TRY(prof_begin(m, RST_KERNEL_GRAD_PAIR, i, 2.0 * mnk + pend.flops, dx_bytes + pend.bytes));
       RST_TRY(launch_gemm_pair(e->stream, dx, pend.d));
       RST_TRY(prof_end(m));
@@ -489,6 +537,7 @@ int rst_model_create(rst_engine* e, const int* kinds, const size_t* in_features,
   if (!m) return fail(RST_ERR_OUT_OF_MEMORY, "host allocation failed");
   m->engine = e;
   m->graph_enabled = default_graph_enabled();
+  m->fuse_head = default_head_enabled();
   m->layers.resize(layer_count);
   size_t offset = 0;
   size_t width = 0;
@@ -676,12 +725,17 @@ int rst_model_sgd_step(rst_model* m, double lr) {
 namespace {
 
 int run_step(rst_model* m, const double* x, const double* truth, size_t batch, double lr) {
-  RST_TRY(do_forward(m, x, batch));
-  RST_TRY(do_loss(m, truth, nullptr));
-  if (m->fuse_sgd) {  // SGD::step rides in the epilogues of the weight-gradient launches
-    RST_TRY(do_backward(m, nullptr, 0, nullptr, &lr));
+  const int head = head_layer(m);
+  RST_TRY(do_forward(m, x, batch, nullptr, head));
+  if (head >= 0) {
+    RST_TRY(do_head(m, head, truth));
   } else {
-    RST_TRY(do_backward(m, nullptr, 0, nullptr, nullptr));
+    RST_TRY(do_loss(m, truth, nullptr));
+  }
+  if (m->fuse_sgd) {  // SGD::step rides in the epilogues of the weight-gradient launches
+    RST_TRY(do_backward(m, nullptr, 0, nullptr, &lr, nullptr, head));
+  } else {
+    RST_TRY(do_backward(m, nullptr, 0, nullptr, nullptr, nullptr, head));
     RST_TRY(do_sgd(m, lr));
   }
   return RST_OK;
@@ -794,6 +848,13 @@ int rst_model_backward_to(rst_model* m, const double* grad, double* input_grad_o
 int rst_model_fuse_sgd(rst_model* m, int enabled) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
   m->fuse_sgd = enabled != 0;
+  drop_graph(m);
+  return RST_OK;
+}
+
+int rst_model_fuse_head(rst_model* m, int enabled) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->fuse_head = enabled != 0;
   drop_graph(m);
   return RST_OK;
 }

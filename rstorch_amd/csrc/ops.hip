@@ -36,6 +36,37 @@ int check_dim(size_t v, const char* what) {
 
 }  // namespace
 
+namespace {
+// where the launch that finishes a loss stores it for the host, and the launch's ticket
+int loss_mirror(rst_engine* e, LossMirror* mirror) {
+  mirror->loss = e->hd_loss;
+  mirror->flags = e->hd_flags;
+  // A launch that is being recorded into a graph gets no ticket: every replay would announce the
+  // number of the recording.
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  RST_HIP(hipStreamIsCapturing(e->stream, &capture));
+  e->loss_ticket = 0;
+  e->loss_with_hits = false;
+  if (capture == hipStreamCaptureStatusNone) {
+    mirror->slots = e->hd_slots;
+    mirror->ticket = e->loss_ticket = engine_next_ticket(e);
+  }
+  return RST_OK;
+}
+}  // namespace
+
+int engine_head_cross_entropy(rst_engine* e, double* row_loss, const double* h, const double* w,
+                              const double* bias, const double* truth, double* logits, double* grad,
+                              double* dx, bool mask, size_t rows, size_t cols, size_t in_features) {
+  if (rows == 0 || cols == 0) return fail(RST_ERR_SHAPE, "cross entropy of an empty batch");
+  LossMirror mirror;
+  RST_TRY(loss_mirror(e, &mirror));
+  RST_TRY(launch_head_ce(e->stream, h, w, bias, truth, logits, grad, dx, mask, row_loss, e->d_loss, e->d_flags,
+                         rows, cols, in_features, mirror));
+  e->loss_valid = true;
+  return RST_OK;
+}
+
 int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, const double* truth,
                          double* grad_out, double* prob_out, size_t rows, size_t cols,
                          double* host_loss, bool* hits_done) {
@@ -45,18 +76,7 @@ int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, co
     row_loss = e->d_row_loss;
   }
   LossMirror mirror;
-  mirror.loss = e->hd_loss;
-  mirror.flags = e->hd_flags;
-  // A launch that is being recorded into a graph gets no ticket: every replay would announce the
-  // number of the recording.
-  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-  RST_HIP(hipStreamIsCapturing(e->stream, &capture));
-  e->loss_ticket = 0;
-  e->loss_with_hits = false;
-  if (capture == hipStreamCaptureStatusNone) {
-    mirror.slots = e->hd_slots;
-    mirror.ticket = e->loss_ticket = engine_next_ticket(e);
-  }
+  RST_TRY(loss_mirror(e, &mirror));
   if (hits_done) mirror.hits = e->hd_hits;
   RST_TRY(launch_softmax_ce(e->stream, pred, truth, grad_out, prob_out, row_loss, e->d_loss,
                             e->d_flags, rows, cols, mirror, hits_done));

@@ -20,6 +20,9 @@ namespace {
 
 typedef double v2d __attribute__((ext_vector_type(2)));
 
+// the fused classifier head: the most classes it takes
+constexpr int kHeadCols = 16;
+
 struct MaxOp {
   __device__ static double apply(double a, double b) { return a < b ? b : a; }
 };
@@ -401,6 +404,228 @@ __global__ __launch_bounds__(1024) void loss_reduce_kernel(const double* __restr
   }
 }
 
+// The classifier head of a training step in one launch: the last Linear's forward
+// (src/module/linear.rs:44-58), the cross entropy on its logits with the gradient
+// (src/loss/cross_entropy.rs:34-47), that Linear's input gradient (linear.rs:68) with the mask of a
+// preceding ReLU (src/module/activation/relu.rs:25-28), and the loss itself, finished by the
+// workgroup that arrives last.  For heads of at most kHeadCols classes on a few hundred inputs,
+// where the four launches this replaces are each over before the next one has started.
+//
+// A workgroup of BLOCK threads takes BLOCK / 16 rows, 16 lanes to a row.  Lane j of a row keeps inputs j, j + 16, ...
+// of that row in registers (KI of them at most) and the whole weight matrix sits in LDS.  Logits: the
+// lane adds up its share of every class's dot product in ascending k, a butterfly over the 16 lanes
+// completes the sums (every lane then holds all of them), and lane c goes on with class c through
+// the softmax with the arithmetic of softmax_rows_kernel.  Input gradient: the lanes of a row
+// exchange their gradient entries, and lane j computes elements j, j + 16, ... as sums over the
+// classes in ascending order, masked by the inputs it still holds.
+// The loss: each workgroup adds its rows' terms up in row order, and the workgroup that arrives last
+// adds the workgroups' sums up in a fixed order (thread t sums t, t + BLOCK, ...; a butterfly over each
+// wavefront; the wavefronts in turn), so the result does not depend on which one came last.
+struct HeadParams {
+  const double* h;      // [rows, K] inputs of the Linear (contiguous rows)
+  const double* w;      // [N, K]
+  const double* bias;   // [N]
+  const double* truth;  // [rows, N]
+  double* logits;       // [rows, N]
+  double* grad;         // [rows, N]  -(truth - p)
+  double* dx;           // [rows, K] or NULL
+  double* partial;      // one sum per workgroup
+  unsigned long long* arrivals;  // zero between launches
+  double* loss;
+  int* flags;
+  size_t rows;
+  int N, K;
+  LossMirror mirror;
+};
+
+template <int KI, int NC, bool MASK, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void head_ce_kernel(HeadParams p) {
+  constexpr int ROWS = BLOCK / 16;  // rows per workgroup
+  static_assert(NC == 4 || NC == 8 || NC == 16, "the class sums are exchanged by halving");
+  // the weights, transposed: [16 * KI][P], the NC classes of one input side by side, zero from class N
+  // and from input K on; with P = NC + 2 the 16 lanes of a row, which read 16 consecutive inputs, hit
+  // different banks
+  extern __shared__ __attribute__((aligned(16))) double head_ws[];
+  constexpr int P = NC + 2;
+  __shared__ double wave_sum[BLOCK / 64];
+  __shared__ double row_sum[ROWS];
+  __shared__ int nan_here, last_nan;
+  __shared__ bool is_last;
+  const int t = threadIdx.x;
+  if (t == 0) nan_here = 0;
+  const int K = p.K, N = p.N;
+  const int r = t >> 4, j = t & 15;
+  const size_t row0 = (size_t)blockIdx.x * ROWS;
+  const size_t row = row0 + r;
+  const bool row_ok = row < p.rows;
+
+  // every global load of the workgroup is issued before the first one is waited for
+  double hv[KI];
+  {
+    const double* hr = p.h + row * (size_t)K;
+#pragma unroll
+    for (int i = 0; i < KI; ++i) {
+      const int k = j + 16 * i;
+      hv[i] = (row_ok && k < K) ? hr[k] : 0.0;
+    }
+    for (int k = t; k < 16 * KI; k += BLOCK) {  // (at most two rounds)
+      double v[NC];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) v[c] = (c < N && k < K) ? p.w[(size_t)c * K + k] : 0.0;
+#pragma unroll
+      for (int c = 0; c < NC; c += 2) *reinterpret_cast<v2d*>(head_ws + k * P + c) = v2d{v[c], v[c + 1]};
+    }
+  }
+  const double bias = j < N ? p.bias[j] : 0.0;
+  const double tv = (row_ok && j < N) ? p.truth[row * N + j] : 0.0;
+  __syncthreads();
+
+  // logits.  No branch in the loops (a branch would have every LDS read waited for on its own): an
+  // index past the row is clamped and its product replaced by zero; classes from N on have zero weights.
+  // (inputs and weights past the row's end are zero, so the loops carry no test; the weights of the
+  // next input are on their way while those of this one are used)
+  double acc[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) acc[c] = 0.0;
+  const v2d* const wj = reinterpret_cast<const v2d*>(head_ws + j * P);  // input j + 16 i: wj + i * 8 P
+  {
+    v2d w2[2][NC / 2];
+#pragma unroll
+    for (int c = 0; c < NC / 2; ++c) w2[0][c] = wj[c];
+#pragma unroll
+    for (int i = 0; i < KI; ++i) {
+      if (i + 1 < KI) {
+#pragma unroll
+        for (int c = 0; c < NC / 2; ++c) w2[(i + 1) & 1][c] = wj[(i + 1) * 8 * P + c];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int c = 0; c < NC / 2; ++c) {
+        acc[2 * c] = fma(hv[i], w2[i & 1][c].x, acc[2 * c]);
+        acc[2 * c + 1] = fma(hv[i], w2[i & 1][c].y, acc[2 * c + 1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  // The 16 lanes of a row add their shares up by halving: with offset 8, 4, 2, 1 in turn a lane keeps
+  // the classes whose index has the lane's bit at that position and receives its partner's share of
+  // them, so that lane j ends with the whole sum of class j (lanes from NC on: a class below NC again).
+#pragma unroll
+  for (int off = 8; off > 0; off >>= 1) {
+    if (off < NC) {
+      const bool upper = (j & off) != 0;
+#pragma unroll
+      for (int i = 0; i < off; ++i) {
+        const double lo = acc[i], hi = acc[i + off < NC ? i + off : i];
+        const double got = __shfl_xor(upper ? lo : hi, off);
+        acc[i] = (upper ? hi : lo) + got;
+      }
+    } else {  // fewer classes than 2 * off: every lane keeps all of them
+#pragma unroll
+      for (int c = 0; c < NC; ++c) acc[c] = acc[c] + __shfl_xor(acc[c], off);
+    }
+  }
+  double z = acc[0];
+  const bool col_ok = j < N, ok = row_ok && col_ok;
+  z = z + bias;
+  const bool saw_nan = ok && z != z;
+  double mx = col_ok ? MaxOp::apply(-DBL_MAX, z) : -DBL_MAX;
+  mx = group_reduce<kHeadCols, MaxOp>(mx, nullptr);
+  const double ev = col_ok ? exp(z - mx) : 0.0;
+  const double s = group_reduce<kHeadCols, SumOp>(ev, nullptr);
+  double lsum = 0.0, g = 0.0;
+  if (ok) {
+    const double pr = ev / s;
+    lsum = loss_term(tv, pr);
+    g = -(tv - pr);
+    p.grad[row * N + j] = g;
+    p.logits[row * N + j] = z;
+  }
+  lsum = group_reduce<kHeadCols, SumOp>(lsum, nullptr);
+  if (j == 0) row_sum[r] = row_ok ? lsum : 0.0;
+  if (saw_nan) nan_here = 1;  // (every writer writes the same value)
+  __syncthreads();
+
+  // The loss.  Thread 0 hands this workgroup's sum over with an atomic exchange, which is carried out
+  // where every workgroup of the device sees it, and only then - the exchange's return value is an
+  // operand of the addition - counts the workgroup in at `arrivals` (low word: workgroups, high word:
+  // those that met a NaN logit).  Whoever counts in last therefore finds every other sum in place and
+  // reads them with atomic loads.  No fence is involved: a device-wide release would have every
+  // workgroup write the whole L2 back.  The exchange travels while the input gradient is computed.
+  unsigned long long* const partial = reinterpret_cast<unsigned long long*>(p.partial);
+  unsigned long long old = 0;
+  if (t == 0) {
+    double mine = 0.0;
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) mine += row_sum[i];
+    old = atomicExch(partial + blockIdx.x, (unsigned long long)__double_as_longlong(mine));
+  }
+
+  if (p.dx) {
+    double gc[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) gc[c] = __shfl(g, c, 16);  // (zero from class N on)
+    double* const dr = p.dx + row * (size_t)K;
+    v2d w2[2][NC / 2];
+#pragma unroll
+    for (int c = 0; c < NC / 2; ++c) w2[0][c] = wj[c];
+#pragma unroll
+    for (int i = 0; i < KI; ++i) {
+      const int k = j + 16 * i;
+      if (i + 1 < KI) {
+#pragma unroll
+        for (int c = 0; c < NC / 2; ++c) w2[(i + 1) & 1][c] = wj[(i + 1) * 8 * P + c];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      double a = 0.0;
+#pragma unroll
+      for (int c = 0; c < NC / 2; ++c) {
+        a = fma(gc[2 * c], w2[i & 1][c].x, a);
+        a = fma(gc[2 * c + 1], w2[i & 1][c].y, a);
+      }
+      if (MASK) a = a * (hv[i] > 0.0 ? 1.0 : 0.0);
+      if (row_ok && k < K) dr[k] = a;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+
+  if (t == 0) {
+    asm volatile("" : "+v"(old));  // the addition below waits for the exchange, whatever its value
+    const unsigned long long inc = 1ull + ((unsigned long long)nan_here << 32) + (old & 0ull);
+    const unsigned long long seen = atomicAdd(p.arrivals, inc) + inc;
+    last_nan = (int)((seen >> 32) != 0);
+    is_last = (unsigned)seen == gridDim.x;
+  }
+  __syncthreads();
+  if (!is_last) return;
+  double sum = 0.0;
+  for (unsigned base = t; base < gridDim.x; base += BLOCK * 4) {  // four loads in flight
+    unsigned long long v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const unsigned at = base + BLOCK * i < gridDim.x ? base + BLOCK * i : 0;
+      v[i] = __hip_atomic_load(partial + at, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (base + BLOCK * i < gridDim.x) sum += __longlong_as_double((long long)v[i]);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum = sum + __shfl_xor(sum, off);
+  if ((t & 63) == 0) wave_sum[t >> 6] = sum;
+  __syncthreads();
+  if (t == 0) {
+    double total = wave_sum[0];
+#pragma unroll
+    for (int w = 1; w < BLOCK / 64; ++w) total += wave_sum[w];
+    const double l = -total / (double)p.rows;
+    p.loss[0] = l;
+    p.flags[1] = last_nan;
+    __hip_atomic_store(p.arrivals, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // re-armed for the next launch
+    publish(p.mirror, l, last_nan, false, 0);
+  }
+}
+
 // softmax down the columns (Softmax::with_axis(0), src/module/activation/softmax.rs:23-28):
 // one thread per column walks the rows three times; a rarely used orientation, kept simple.
 __global__ __launch_bounds__(256) void softmax_columns_kernel(const double* __restrict__ z,
@@ -530,6 +755,60 @@ int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* g
     hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(1024), 0, s, row_loss, loss, flags, rows, mirror);
     RST_HIP(hipGetLastError());
   }
+  return RST_OK;
+}
+
+bool head_ce_supported(size_t cols, size_t in_features) {
+  return cols >= 1 && cols <= (size_t)kHeadCols && in_features >= 1 && in_features <= 16 * 18;
+}
+
+int launch_head_ce(hipStream_t s, const double* h, const double* w, const double* bias, const double* truth,
+                   double* logits, double* grad, double* dx, bool mask, double* row_loss, double* loss,
+                   int* flags, size_t rows, size_t cols, size_t in_features, LossMirror mirror) {
+  if (!head_ce_supported(cols, in_features))
+    return fail(RST_ERR_UNSUPPORTED, "fused head: %zu classes on %zu inputs do not fit", cols, in_features);
+  if (rows == 0) return RST_OK;
+  // 16 rows to a workgroup while that leaves every compute unit with work, 32 beyond (each workgroup
+  // pays a round trip to the one arrival counter)
+  const int block_threads = rows <= 16 * 512 / 2 ? 256 : 512;
+  const size_t rows_per_block = block_threads / 16;
+  const size_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+  HeadParams p{};
+  p.h = h; p.w = w; p.bias = bias; p.truth = truth;
+  p.logits = logits; p.grad = grad; p.dx = dx;
+  p.partial = row_loss;  // [rows] holds one word per workgroup
+  p.arrivals = reinterpret_cast<unsigned long long*>(flags + 4);
+  p.loss = loss; p.flags = flags;
+  p.rows = rows; p.N = (int)cols; p.K = (int)in_features;
+  p.mirror = mirror;
+  p.mirror.hits = nullptr;  // the hit count is not taken here
+  const bool masked = mask && dx;
+  const int nc = cols <= 4 ? 4 : cols <= 8 ? 8 : 16;
+  const size_t lds = (size_t)(nc + 2) * 16 * (in_features <= 16 * 8 ? 8 : 18) * sizeof(double);
+  const dim3 grid((unsigned)blocks), block(block_threads);
+#define RST_HEAD_LAUNCH3(KI, NC, M, B) hipLaunchKernelGGL((head_ce_kernel<KI, NC, M, B>), grid, block, lds, s, p)
+#define RST_HEAD_LAUNCH(KI, NC)                                  \
+  do {                                                           \
+    if (block_threads == 256) {                                  \
+      if (masked) RST_HEAD_LAUNCH3(KI, NC, true, 256);           \
+      else RST_HEAD_LAUNCH3(KI, NC, false, 256);                 \
+    } else {                                                     \
+      if (masked) RST_HEAD_LAUNCH3(KI, NC, true, 512);           \
+      else RST_HEAD_LAUNCH3(KI, NC, false, 512);                 \
+    }                                                            \
+  } while (0)
+  if (in_features <= 16 * 8) {
+    if (nc == 4) RST_HEAD_LAUNCH(8, 4);
+    else if (nc == 8) RST_HEAD_LAUNCH(8, 8);
+    else RST_HEAD_LAUNCH(8, 16);
+  } else {
+    if (nc == 4) RST_HEAD_LAUNCH(18, 4);
+    else if (nc == 8) RST_HEAD_LAUNCH(18, 8);
+    else RST_HEAD_LAUNCH(18, 16);
+  }
+#undef RST_HEAD_LAUNCH3
+#undef RST_HEAD_LAUNCH
+  RST_HIP(hipGetLastError());
   return RST_OK;
 }
 

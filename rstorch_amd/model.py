@@ -190,6 +190,11 @@ class DeviceModel:
         """Apply SGD inside the weight-gradient launches of train_step (default) or as a pass."""
         _ffi.check(self.engine.lib.rst_model_fuse_sgd(self.handle, 1 if on else 0))
 
+    def fuse_head(self, on=True):
+        """Run a small classifier head (last Linear, cross entropy, its input gradient) as one
+        launch inside train_step (default) or as the separate launches."""
+        _ffi.check(self.engine.lib.rst_model_fuse_head(self.handle, 1 if on else 0))
+
     def pair_gradients(self, on=True):
         """Launch a layer's weight gradient in one grid with the next layer's input gradient
         when both are large (default), or one after the other."""

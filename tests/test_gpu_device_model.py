@@ -106,6 +106,8 @@ def test_basic_model_from_sequential(engine, oracle):
                                   rs.Linear.new_with_kernel(30, 4, rs.FromArrays(weights[2], weights[3]))])
     loop_model, loss, optim = seq(), rs.CrossEntropyLoss.new(), rs.SGD.new(0.1)
     basic = rs.BasicModel.new(seq(), rs.CrossEntropyLoss.new(), rs.SGD.new(0.1))
+    basic.device.fuse_head(False)
+    fused = rs.BasicModel.new(seq(), rs.CrossEntropyLoss.new(), rs.SGD.new(0.1))  # the head as one launch
     for step in range(5):
         x, y = batch_data(oracle, 16, 20, 4, 3, step, True)
         l1 = loss.forward(loop_model.forward(x), y)
@@ -113,8 +115,11 @@ def test_basic_model_from_sequential(engine, oracle):
         optim.step(loop_model)
         l2 = basic.step(x, y, want_loss=True)
         assert l1 == l2  # same kernels, same order: bit-identical
-    for p, (q, _) in zip(loop_model.parameters(), basic.device.parameters()):
+        l3 = fused.step(x, y, want_loss=True)
+        assert abs(l3 - l1) <= 1e-13 * abs(l1)  # the head's dot products add in another order
+    for p, (q, _), (f, _) in zip(loop_model.parameters(), basic.device.parameters(), fused.device.parameters()):
         np.testing.assert_array_equal(p.parm.to_numpy(), q.to_numpy())
+        assert rel_err(f.to_numpy(), q.to_numpy()) <= 1e-13
     np.testing.assert_array_equal(basic.predict(x).to_numpy(), loop_model.forward(x).to_numpy())
 
 
@@ -151,10 +156,17 @@ def test_profile_records_cover_every_launch(engine, oracle):
     dm.train_step(x, y, 0.01)
     recs = dm.profile_read()
     kinds = [r["kernel"] for r in recs]
-    assert kinds.count("linear_forward") == 3 and kinds.count("grad_weight") == 3
-    assert kinds.count("grad_input") == 2      # the first layer's input gradient is skipped
+    # the last Linear's forward and input gradient run inside the cross-entropy launch (the fused head);
+    # the first layer's input gradient is skipped
+    assert kinds.count("linear_forward") == 2 and kinds.count("grad_weight") == 3
+    assert kinds.count("grad_input") == 1
     # the optimiser rides in the weight-gradient launches unless asked to be a pass of its own
     assert kinds.count("cross_entropy") == 1 and kinds.count("sgd") == 0
+    dm.fuse_head(False)
+    dm.train_step(x, y, 0.01)
+    kinds = [r["kernel"] for r in dm.profile_read()]
+    assert kinds.count("linear_forward") == 3 and kinds.count("grad_input") == 2 and kinds.count("cross_entropy") == 1
+    dm.fuse_head(True)
     assert "relu_forward" not in kinds and "relu_backward" not in kinds  # fused away
     assert all(r["ms"] > 0 for r in recs)
     dm.fuse_sgd(False)
