@@ -48,7 +48,7 @@ PEAK_HBM_GBPS = 8000.0
 # the profile is collected again and the digest updated.
 C4_TRAFFIC_SOURCE = {"profile": "profiles/c4_hbm_traffic.md",
                      "kernel_sources": ["rstorch_amd/csrc/gemm_f64.hip", "rstorch_amd/csrc/gemm_addressing.h"],
-                     "kernel_sources_sha16": "ddc8a362822a16d9"}
+                     "kernel_sources_sha16": "5cfe812563056d9b"}
 
 
 def kernel_sources_digest():
@@ -61,12 +61,12 @@ def kernel_sources_digest():
 
 
 C4_TRAFFIC_BYTES_PER_LAUNCH = {
-    "linear_forward": (8 * 436.4e6 + 3826.0e6) / 9,
-    "grad_weight": (8 * 868.8e6 + 8203.2e6) / 9,
-    "grad_input": (7 * 470.0e6 + 3330.5e6 + 134.3e6) / 8,
+    "linear_forward": (8 * 436.5e6 + 3893.8e6) / 9,
+    "grad_weight": (8 * 867.3e6 + 8443.0e6) / 9,
+    "grad_input": (7 * 470.0e6 + 3338.3e6 + 134.3e6) / 8,
     # a layer's weight gradient + SGD and the next layer's input gradient in one grid (the default):
     # six pairs at the hidden width and the one that carries the head's weight gradient
-    "grad_pair": (6 * 1523.3e6 + 8444.2e6) / 7,
+    "grad_pair": (6 * 1535.2e6 + 8546.4e6) / 7,
 }
 
 C4_SPEC = [("linear", 4096, 4096), ("relu",)] * 8 + [("linear", 4096, 32768)]

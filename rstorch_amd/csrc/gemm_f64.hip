@@ -21,6 +21,7 @@
 // holds B[l/16][l%16], and accumulator register r of lane l holds D[4*r + l/16][l%16].
 #include <cmath>
 #include <cstdlib>
+#include <type_traits>
 
 #include "common.h"
 #include "gemm_addressing.h"
@@ -844,7 +845,6 @@ typedef const __attribute__((address_space(3))) double* lds_cf64_t;
 constexpr int kT64 = 64;
 constexpr int kT64Stage = kT64 * BK;  // doubles per operand and stage
 constexpr int kT64Stages = 4;
-constexpr int kT64Dist = 3;
 
 template <bool KC>
 __device__ __forceinline__ void store_tile_dma64(double* __restrict__ lds, const v2d* __restrict__ reg, int tid) {
@@ -923,16 +923,26 @@ __global__ __launch_bounds__(256, 2) void gemm_f64_mfma_dma64(const GemmParams p
   const int nk = nk_dma + first_dma;
   a_ptr += (long)kt0 * a_step;
   b_ptr += (long)kt0 * b_step;
+  // chunk h of this wavefront's share of a tile, both operands; after the last chunk the pointers move on
+  auto issue_chunk = [&](int stage, int h) {
+    asm volatile("" : "+v"(ao[h]), "+v"(bo[h]));
+    dma16(reinterpret_cast<const double*>(a_ptr + ao[h]), lds_a + stage * kT64Stage + lchunk[h]);
+    dma16(reinterpret_cast<const double*>(b_ptr + bo[h]), lds_b + stage * kT64Stage + lchunk[h]);
+    if (h == CH - 1) {
+      a_ptr += a_step;
+      b_ptr += b_step;
+    }
+  };
   auto issue = [&](int stage) {
 #pragma unroll
-    for (int h = 0; h < CH; ++h) {
-      asm volatile("" : "+v"(ao[h]), "+v"(bo[h]));
-      dma16(reinterpret_cast<const double*>(a_ptr + ao[h]), lds_a + stage * kT64Stage + lchunk[h]);
-      dma16(reinterpret_cast<const double*>(b_ptr + bo[h]), lds_b + stage * kT64Stage + lchunk[h]);
-    }
-    a_ptr += a_step;
-    b_ptr += b_step;
+    for (int h = 0; h < CH; ++h) issue_chunk(stage, h);
   };
+  // prologue: tiles 0 .. kT64Stages-1 on their way.  The remainder tile, if any, is tile 0 and goes
+  // through registers into stage 0; its masked loads are issued behind the tile DMA of the others, so
+  // that all of them are in flight together (one round trip to memory instead of two).
+#pragma unroll
+  for (int t = 0; t < kT64Stages; ++t)
+    if (t >= first_dma && t < nk) issue(t);
   if (k_tail) {
     v2d ra[2], rb[2];
     load_tile<BM, A_KC, true, true, 256>(ra, p.A, p.lda, m0, p.M, nk_all * BK, p.K, tid);
@@ -940,45 +950,92 @@ __global__ __launch_bounds__(256, 2) void gemm_f64_mfma_dma64(const GemmParams p
     store_tile_dma64<A_KC>(lds_a, ra, tid);
     store_tile_dma64<B_KC>(lds_b, rb, tid);
   }
-  // prologue: tiles 0 .. kT64Dist-1 on their way (the remainder tile, if any, is tile 0 and already there)
-#pragma unroll
-  for (int t = 0; t < kT64Dist; ++t)
-    if (t >= first_dma && t < nk) issue(t % kT64Stages);
 
   const uint32_t a_base = (uint32_t)(uintptr_t)lds_a, b_base = (uint32_t)(uintptr_t)lds_b;
   const int a_e = wm * 32 + lr, b_e = wn * 32 + lr;  // fragment 0; fragment 1 is 16 further
+  // A tile's 16 contraction indices are consumed as two pairs of MFMA steps (pair s2: k = 8 s2 + 2 lk in
+  // the first step, 8 s2 + 2 lk + 1 in the second); a fragment of a pair is one 16-byte read per lane.
+  auto read_a = [&](int stage, int s2, int i) {
+    return read_pair64<A_KC>(a_base + (uint32_t)stage * (kT64Stage * 8), a_e + 16 * i, 4 * s2 + lk);
+  };
+  auto read_b = [&](int stage, int s2, int j) {
+    return read_pair64<B_KC>(b_base + (uint32_t)stage * (kT64Stage * 8), b_e + 16 * j, 4 * s2 + lk);
+  };
+  v2d pa[TM], pb[TN];  // the fragments of a tile's first pair
+  v2d qa[TM], qb[TN];  // of its second pair
+  auto mx = [&](const v2d (&fa)[TM], const v2d (&fb)[TN], int i, int j) {
+    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[i].x, fb[j].x, acc[i][j], 0, 0, 0);
+  };
+  auto my = [&](const v2d (&fa)[TM], const v2d (&fb)[TN], int i, int j) {
+    acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[i].y, fb[j].y, acc[i][j], 0, 0, 0);
+  };
+#define RST_FENCE() __builtin_amdgcn_sched_barrier(0)
 
-  for (int kt = 0; kt < nk; ++kt) {
-    // tile kt has landed once at most the younger tiles in flight remain outstanding (4 loads each)
-    const int younger = nk - 1 - kt < kT64Dist - 1 ? nk - 1 - kt : kT64Dist - 1;
+  // One tile.  With one wavefront per SIMD nothing else fills the matrix cores while this one waits,
+  // so everything that is not an MFMA is placed between two of them, one or two instructions at a
+  // time (the fences keep the compiler from gathering them): the reads of the second pair under the
+  // first pair's MFMAs; the wait for tile kt + 1 and the barrier after the fourth MFMA of the second
+  // pair, when all fragments of tile kt are in registers; then, under the last four MFMAs, the reads
+  // of tile kt + 1's first pair and the requests for tile kt + 4, which takes the stage of tile kt.
+  // STEADY: tiles kt + 1 .. kt + 4 all exist (no tests in the instruction stream).
+  auto tile = [&](int kt, auto steady_tag) {
+    constexpr bool STEADY = decltype(steady_tag)::value;
+    const int stage = kt % kT64Stages, next = (kt + 1) % kT64Stages;
+    mx(pa, pb, 0, 0); RST_FENCE();
+    qa[0] = read_a(stage, 1, 0); RST_FENCE();
+    mx(pa, pb, 0, 1); RST_FENCE();
+    qb[0] = read_b(stage, 1, 0); RST_FENCE();
+    mx(pa, pb, 1, 0); RST_FENCE();
+    qb[1] = read_b(stage, 1, 1); RST_FENCE();
+    mx(pa, pb, 1, 1); RST_FENCE();
+    qa[1] = read_a(stage, 1, 1); RST_FENCE();
+    my(pa, pb, 0, 0); my(pa, pb, 0, 1); my(pa, pb, 1, 0); my(pa, pb, 1, 1); RST_FENCE();
+    mx(qa, qb, 0, 0); mx(qa, qb, 0, 1); mx(qa, qb, 1, 0); mx(qa, qb, 1, 1); RST_FENCE();
+    const bool more = STEADY || kt + 1 < nk;
+    if (more) {
+      // tile kt + 1 has landed once at most the younger tiles in flight remain outstanding (4 loads each)
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): this wavefront's reads of tile kt are over
+      if (STEADY) {
+        wait_vmcnt(4 * (kT64Stages - 2));
+      } else {
+        const int younger = nk - 2 - kt < kT64Stages - 2 ? nk - 2 - kt : kT64Stages - 2;
+        wait_vmcnt(4 * younger);
+      }
+      __builtin_amdgcn_s_barrier();  // everybody's share of tile kt + 1 is in LDS; everybody has read tile kt
+    }
+    RST_FENCE();
+    my(qa, qb, 0, 0); RST_FENCE();
+    if (more) {
+      pa[0] = read_a(next, 0, 0);
+      pb[0] = read_b(next, 0, 0);
+    }
+    RST_FENCE();
+    my(qa, qb, 0, 1); RST_FENCE();
+    if (more) {
+      pb[1] = read_b(next, 0, 1);
+      pa[1] = read_a(next, 0, 1);
+    }
+    RST_FENCE();
+    my(qa, qb, 1, 0); RST_FENCE();
+    if (STEADY) issue_chunk(stage, 0);
+    RST_FENCE();
+    my(qa, qb, 1, 1); RST_FENCE();
+    if (STEADY) issue_chunk(stage, 1);
+    RST_FENCE();
+  };
+  {
+    const int younger = nk - 1 < kT64Stages - 1 ? nk - 1 : kT64Stages - 1;
     wait_vmcnt(4 * younger);
-    __syncthreads();  // everybody's share of tile kt is in LDS; everybody is done with tile kt-1
-    if (kt + kT64Dist < nk) issue((kt + kT64Dist) % kT64Stages);
-    const int stage = kt % kT64Stages;
-    const uint32_t sa = a_base + (uint32_t)stage * (kT64Stage * 8), sb = b_base + (uint32_t)stage * (kT64Stage * 8);
-    v2d fa[2][TM], fb[2][TN];
-#pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-      const int pr = 4 * s2 + lk;
-#pragma unroll
-      for (int i = 0; i < TM; ++i) fa[s2][i] = read_pair64<A_KC>(sa, a_e + 16 * i, pr);
-#pragma unroll
-      for (int j = 0; j < TN; ++j) fb[s2][j] = read_pair64<B_KC>(sb, b_e + 16 * j, pr);
-    }
-#pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[s2][i].x, fb[s2][j].x, acc[i][j], 0, 0, 0);
-#pragma unroll
-      for (int i = 0; i < TM; ++i)
-#pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(fa[s2][i].y, fb[s2][j].y, acc[i][j], 0, 0, 0);
-    }
+    __syncthreads();
+    pa[0] = read_a(0, 0, 0);
+    pb[0] = read_b(0, 0, 0);
+    pb[1] = read_b(0, 0, 1);
+    pa[1] = read_a(0, 0, 1);
   }
+  int kt = 0;
+  for (; kt + kT64Stages < nk; ++kt) tile(kt, std::true_type{});
+  for (; kt < nk; ++kt) tile(kt, std::false_type{});
+#undef RST_FENCE
   write_block<TM, TN>(p, &acc[0][0], m0 + wm * 32, n0 + wn * 32, lr, lk, split);
 }
 
