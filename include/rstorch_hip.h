@@ -276,15 +276,23 @@ int rst_model_fuse_sgd(rst_model* model, int enabled);
  * Results are identical either way.  On by default (measured on MI355X at C4's hidden width:
  * 0.946 ms per pair against 0.477 + 0.503 ms for the two launches one after the other). */
 int rst_model_pair_gradients(rst_model* model, int enabled);
-/* enabled != 0 (the default, unless the environment says RSTORCH_HEAD=0): when the model ends in a
- * Linear with at most 16 outputs on at most 288 inputs, rst_model_train_step runs that Linear's forward
- * (src/module/linear.rs:44-58), the cross entropy with its gradient (src/loss/cross_entropy.rs:34-47),
- * the Linear's input gradient (linear.rs:68, masked by a preceding ReLU, relu.rs:25-28) and the final
- * sum of the loss as ONE launch instead of four.  The logits are then plain dot products (16 lanes
- * share a row, each adding every 16th term, then the lanes' sums) instead of matrix-core sums, so
- * results differ from the unfused launches by rounding (1e-15 relative); they are deterministic and
- * do not depend on the number of compute units or on the order in which workgroups finish.  The separate
- * calls (rst_model_forward / _loss / _backward, and the *_to variants) are not affected. */
+/* How much of a small classifier's tail rst_model_train_step runs as ONE launch.
+ * enabled >= 1: when the model ends in a Linear with at most 16 outputs on at most 288 inputs, that
+ * Linear's forward (src/module/linear.rs:44-58), the cross entropy with its gradient
+ * (src/loss/cross_entropy.rs:34-47), the Linear's input gradient (linear.rs:68, masked by a preceding
+ * ReLU, relu.rs:25-28) and the final sum of the loss are one launch instead of four.
+ * enabled >= 2 (the default): when, besides, the Linear in front of it - with nothing but a ReLU
+ * between the two - has at most 112 inputs and 112 outputs, its forward and its input gradient run in
+ * the same launch too (its weights sit in LDS; both products run on the matrix cores), which saves two
+ * more launches.
+ * enabled == 0: the separate launches.  The environment variable RSTORCH_HEAD (0, 1; anything else: 2)
+ * sets the level new models start with.
+ * The fused sums are taken in another order than those of the contraction kernels (the head: 16 lanes
+ * share a row, each adding every 16th term, then the lanes' sums; the hidden layer: four interleaved
+ * partial sums per output), so results differ from the unfused launches by rounding (1e-15 relative);
+ * they are deterministic and do not depend on the number of compute units or on the order in which
+ * workgroups finish.  The separate calls (rst_model_forward / _loss / _backward, and the *_to variants)
+ * are not affected. */
 int rst_model_fuse_head(rst_model* model, int enabled);
 /* rst_model_train_step records its launches into a HIP graph the first time it sees a given
  * (x, truth, batch, lr) and replays the graph afterwards; a different argument re-records (the 64
@@ -299,7 +307,8 @@ int rst_model_graph_enable(rst_model* model, int enabled);
  *   RSTORCH_DMA_GROUP=0  small weight gradients never share the grid of K-sliced 128x128 tiles,
  *                    =1  they do whenever they can (unset: the measured rule);
  *   RSTORCH_DMA64=0      no product goes to the 64x64 direct-to-LDS kernel, =1 every eligible one;
- *   RSTORCH_HEAD=0       new models keep the classifier head as separate launches (rst_model_fuse_head). */
+ *   RSTORCH_HEAD=0 / 1   new models keep the classifier's tail as separate launches / fuse the head alone
+ *                        (rst_model_fuse_head). */
 /* Per-launch timing of the model's kernels: when enabled an event is recorded on the engine's
  * stream after every launch (and one before the first launch of a call); a launch's duration runs
  * from the previous event to its own, so it includes the few microseconds between the previous

@@ -151,9 +151,24 @@ int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* g
 // [rows] scratch).  Only for shapes
 // head_ce_supported accepts: few classes on few inputs, where the weight matrix sits in LDS.
 bool head_ce_supported(size_t cols, size_t in_features);
+// The Linear in front of the head, run by the same launch when it is small enough for its weights to
+// sit in LDS (tail_ce_supported): output = input.weight^T + bias ([rows, in_features] -> the head's
+// input, with the ReLU between the two applied when the head's `mask` says there is one);
+// input_grad = (the head's dx).weight, zeroed where input <= 0 if mask_input_grad, or NULL.
+struct HiddenLayer {
+  const double* input;
+  const double* weight;  // [head in_features, in_features]
+  const double* bias;
+  double* output;        // [rows, head in_features]: written here, and the head's `h` is ignored
+  double* input_grad;    // [rows, in_features] or NULL
+  size_t in_features;
+  bool mask_input_grad;
+};
+bool tail_ce_supported(size_t cols, size_t hidden, size_t in_features, size_t lds_limit);
 int launch_head_ce(hipStream_t s, const double* h, const double* w, const double* bias, const double* truth,
                    double* logits, double* grad, double* dx, bool mask, double* row_loss, double* loss,
-                   int* flags, size_t rows, size_t cols, size_t in_features, LossMirror mirror = LossMirror());
+                   int* flags, size_t rows, size_t cols, size_t in_features, LossMirror mirror = LossMirror(),
+                   const HiddenLayer* hidden = nullptr);
 int launch_softmax_columns(hipStream_t s, const double* z, double* out, int* flags, size_t rows,
                            size_t cols);
 int launch_softmax_jacobian(hipStream_t s, double* jac, size_t cols);
@@ -238,5 +253,6 @@ int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, co
 // the fused classifier head (launch_head_ce) with the engine's loss words, mirror and ticket
 int engine_head_cross_entropy(rst_engine* e, double* row_loss, const double* h, const double* w,
                               const double* bias, const double* truth, double* logits, double* grad,
-                              double* dx, bool mask, size_t rows, size_t cols, size_t in_features);
+                              double* dx, bool mask, size_t rows, size_t cols, size_t in_features,
+                              const rst::HiddenLayer* hidden = nullptr);
 }  // namespace rst

@@ -96,7 +96,8 @@ struct rst_model {
   bool pair_gradients = true;
   // train_step runs a small classifier head (last Linear, cross entropy, that Linear's input
   // gradient) as one launch when the shape allows it
-  bool fuse_head = true;
+  // (0: never; 1: the head alone; 2: together with the Linear in front of it when that one is small too)
+  int fuse_head = 2;
   // profiling
   bool profiling = false;
   bool slot_open = false;
@@ -119,10 +120,13 @@ bool default_graph_enabled() {
   return !(v && v[0] == '0');
 }
 
-// Whether train_step hands a small classifier head to the fused launch: yes, unless RSTORCH_HEAD=0.
-bool default_head_enabled() {
+// What train_step hands to the fused head launch: RSTORCH_HEAD=0 nothing, =1 the head alone, unset or
+// anything else also the Linear in front of it.
+int default_head_mode() {
   const char* v = std::getenv("RSTORCH_HEAD");
-  return !(v && v[0] == '0');
+  if (v && v[0] == '0') return 0;
+  if (v && v[0] == '1') return 1;
+  return 2;
 }
 
 // A graph executable is only destroyed once nothing enqueued on the stream can still be running it.
@@ -219,9 +223,15 @@ int next_non_identity(const rst_model* m, int i) {
 // final_out != NULL: the last layer that computes anything writes there instead of into the model's
 // own buffer (the caller's array that Sequential::forward returns by value; backward reads it again
 // as the mask of a trailing ReLU, so it must stay as it is until then).
-// head >= 0: that layer, the last Linear, is left to the fused head launch (do_head), which also
-// computes the loss: its input is noted, nothing is launched for it.
-int do_forward(rst_model* m, const double* x, size_t batch, double* final_out = nullptr, int head = -1) {
+// The layers that train_step leaves to the fused head launch (do_head): the last Linear and, with
+// it, the Linear in front of it.  -1: none.
+struct Tail {
+  int head = -1, hidden = -1;
+  bool takes(int i) const { return i >= 0 && (i == head || i == hidden); }
+};
+
+// tail: its layers' inputs are noted, nothing is launched for them.
+int do_forward(rst_model* m, const double* x, size_t batch, double* final_out = nullptr, Tail tail = Tail()) {
   rst_engine* e = m->engine;
   if (batch > (size_t)INT_MAX) return fail(RST_ERR_UNSUPPORTED, "batch too large");
   RST_TRY(reserve_activations(m, batch));
@@ -246,23 +256,21 @@ int do_forward(rst_model* m, const double* x, size_t batch, double* final_out = 
       const bool fuse = nx >= 0 && m->layers[nx].kind == RST_LAYER_RELU;
       l.input = cur;  // linear.rs:56 keeps the input for backward
       l.relu_fused = fuse;
-      if (i == head) {
-        cur = dest;
-        continue;
+      if (!tail.takes(i)) {
+        GemmDesc d{};
+        d.A = cur; d.B = l.w; d.C = dest;
+        d.M = (int)batch; d.N = (int)l.out; d.K = (int)l.in;
+        d.lda = (long)l.in; d.ldb = (long)l.in; d.ldc = (long)l.out;
+        d.a_kc = true; d.b_kc = true;
+        d.epilogue = fuse ? EPI_BIAS_RELU : EPI_BIAS;
+        d.bias = l.b;
+        const double flops = 2.0 * (double)batch * (double)l.in * (double)l.out;
+        const double bytes = 8.0 * ((double)batch * l.in + (double)l.in * l.out + (double)batch * l.out);
+        d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
+        RST_TRY(prof_begin(m, RST_KERNEL_LINEAR_FORWARD, i, flops, bytes));
+        RST_TRY(launch_gemm(e->stream, d));
+        RST_TRY(prof_end(m));
       }
-      GemmDesc d{};
-      d.A = cur; d.B = l.w; d.C = dest;
-      d.M = (int)batch; d.N = (int)l.out; d.K = (int)l.in;
-      d.lda = (long)l.in; d.ldb = (long)l.in; d.ldc = (long)l.out;
-      d.a_kc = true; d.b_kc = true;
-      d.epilogue = fuse ? EPI_BIAS_RELU : EPI_BIAS;
-      d.bias = l.b;
-      const double flops = 2.0 * (double)batch * (double)l.in * (double)l.out;
-      const double bytes = 8.0 * ((double)batch * l.in + (double)l.in * l.out + (double)batch * l.out);
-      d.workspace = e->d_gemm_ws; d.workspace_count = e->gemm_ws_count;
-      RST_TRY(prof_begin(m, RST_KERNEL_LINEAR_FORWARD, i, flops, bytes));
-      RST_TRY(launch_gemm(e->stream, d));
-      RST_TRY(prof_end(m));
       cur = dest;
       if (fuse) {
         Layer& r = m->layers[nx];
@@ -300,31 +308,63 @@ int do_loss(rst_model* m, const double* truth, double* host_loss) {
   return RST_OK;
 }
 
-// The layer that train_step can hand to the fused head launch, or -1: the last layer that is not an
-// Identity, if it is a Linear whose shape the head kernel takes.
-int head_layer(const rst_model* m) {
-  if (!m->fuse_head) return -1;
+// The layers that train_step can hand to the fused head launch: the last layer that is not an
+// Identity, if it is a Linear whose shape the head kernel takes; and the Linear in front of it, if
+// nothing but a ReLU stands between the two and both are small enough for the variant that holds the
+// hidden weights in LDS.
+Tail tail_layers(const rst_model* m) {
+  Tail t;
+  if (m->fuse_head == 0) return t;
   const int i = prev_non_identity(m, (int)m->layers.size());
-  if (i < 0 || m->layers[i].kind != RST_LAYER_LINEAR) return -1;
-  return head_ce_supported(m->layers[i].out, m->layers[i].in) ? i : -1;
+  if (i < 0 || m->layers[i].kind != RST_LAYER_LINEAR) return t;
+  if (!head_ce_supported(m->layers[i].out, m->layers[i].in)) return t;
+  t.head = i;
+  if (m->fuse_head < 2) return t;
+  int j = prev_non_identity(m, i);
+  if (j >= 0 && m->layers[j].kind == RST_LAYER_RELU) j = prev_non_identity(m, j);
+  if (j >= 0 && m->layers[j].kind == RST_LAYER_LINEAR &&
+      tail_ce_supported(m->layers[i].out, m->layers[i].in, m->layers[j].in, m->engine->props.sharedMemPerBlock))
+    t.hidden = j;
+  return t;
 }
 
-// Forward of the head Linear, the loss with its gradient and, unless the head is the first Linear
-// (whose input gradient train_step does not need), the head's input gradient: one launch.
-int do_head(rst_model* m, int head, const double* truth) {
+// Forward of the tail's Linear layers, the loss with its gradient and the input gradients of those
+// layers (but not of the model's first Linear, which train_step does not need): one launch.
+int do_head(rst_model* m, Tail tail, const double* truth) {
   rst_engine* e = m->engine;
   if (!truth) return fail(RST_ERR_INVALID_ARGUMENT, "truth is null");
-  Layer& l = m->layers[head];
+  Layer& l = m->layers[tail.head];
   const size_t rows = m->batch;
-  bool wanted = false;
-  for (int i = 0; i < head; ++i) wanted |= m->layers[i].kind == RST_LAYER_LINEAR;
-  const int pv = prev_non_identity(m, head);
-  const bool mask = pv >= 0 && m->layers[pv].kind == RST_LAYER_RELU;
-  const double work = (double)rows * (double)l.in * (double)l.out;
-  RST_TRY(prof_begin(m, RST_KERNEL_CROSS_ENTROPY, head, (wanted ? 4.0 : 2.0) * work,
-                     8.0 * ((double)rows * l.in * (wanted ? 2.0 : 1.0) + 3.0 * (double)rows * l.out)));
+  auto has_linear_before = [&](int i) {
+    for (int k = 0; k < i; ++k)
+      if (m->layers[k].kind == RST_LAYER_LINEAR) return true;
+    return false;
+  };
+  auto relu_before = [&](int i) {
+    const int pv = prev_non_identity(m, i);
+    return pv >= 0 && m->layers[pv].kind == RST_LAYER_RELU;
+  };
+  const bool wanted = has_linear_before(tail.head);
+  double work = (double)rows * (double)l.in * (double)l.out * (wanted ? 4.0 : 2.0);
+  double bytes = 8.0 * ((double)rows * l.in * (wanted ? 2.0 : 1.0) + 3.0 * (double)rows * l.out);
+  HiddenLayer hidden{};
+  if (tail.hidden >= 0) {
+    Layer& hl = m->layers[tail.hidden];
+    const bool wanted1 = has_linear_before(tail.hidden);
+    hidden.input = hl.input;
+    hidden.weight = hl.w;
+    hidden.bias = hl.b;
+    hidden.output = hl.out_buf;
+    hidden.input_grad = wanted1 ? hl.grad_in_buf : nullptr;
+    hidden.in_features = hl.in;
+    hidden.mask_input_grad = relu_before(tail.hidden);
+    work += (double)rows * (double)hl.in * (double)hl.out * (wanted1 ? 4.0 : 2.0);
+    bytes += 8.0 * ((double)rows * hl.in * (wanted1 ? 2.0 : 1.0) + (double)hl.in * hl.out);
+  }
+  RST_TRY(prof_begin(m, RST_KERNEL_CROSS_ENTROPY, tail.head, work, bytes));
   RST_TRY(engine_head_cross_entropy(e, m->row_loss, l.input, l.w, l.b, truth, l.out_buf, m->loss_grad,
-                                    wanted ? l.grad_in_buf : nullptr, mask, rows, l.out, l.in));
+                                    wanted ? l.grad_in_buf : nullptr, relu_before(tail.head), rows, l.out, l.in,
+                                    tail.hidden >= 0 ? &hidden : nullptr));
   RST_TRY(prof_end(m));
   m->loss_grad_valid = true;
   return RST_OK;
@@ -335,9 +375,9 @@ int do_head(rst_model* m, int head, const double* truth) {
 // input_grad_dest != NULL (with need_input_grad): the gradient with respect to the model's input is
 // written there (the caller's array that Sequential::backward returns by value) instead of into the
 // model's own buffer.
-// head >= 0: the input gradient of that Linear (the last one) has been written by do_head already.
+// tail: the input gradients of its layers have been written by do_head already.
 int do_backward(rst_model* m, const double* grad, int need_input_grad, const double** input_grad,
-                const double* fused_lr, double* input_grad_dest = nullptr, int head = -1) {
+                const double* fused_lr, double* input_grad_dest = nullptr, Tail tail = Tail()) {
   rst_engine* e = m->engine;
   if (!m->forward_valid)
     return fail(RST_ERR_STATE, "backward without a forward (the reference panics on a consumed cache)");
@@ -459,8 +499,8 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
       dx_bytes = 8.0 * ((double)batch * l.out + (double)l.in * l.out +
                         (double)batch * l.in * (mask ? 2.0 : 1.0));
     }
-    if (i == head) {
-      // (nothing is pending: the head is the first layer this loop meets)
+    if (tail.takes(i)) {
+      RST_TRY(flush_pending());  // (the head's weight gradient, when this is the layer in front of it)
     } else if (pend.active && wanted && m->pair_gradients && can_pair_gemm(dx, pend.d)) {
       RST_TRY(prof_begin(m, RST_KERNEL_GRAD_PAIR, i, 2.0 * mnk + pend.flops, dx_bytes + pend.bytes));
       RST_TRY(launch_gemm_pair(e->stream, dx, pend.d));
@@ -537,7 +577,7 @@ int rst_model_create(rst_engine* e, const int* kinds, const size_t* in_features,
   if (!m) return fail(RST_ERR_OUT_OF_MEMORY, "host allocation failed");
   m->engine = e;
   m->graph_enabled = default_graph_enabled();
-  m->fuse_head = default_head_enabled();
+  m->fuse_head = default_head_mode();
   m->layers.resize(layer_count);
   size_t offset = 0;
   size_t width = 0;
@@ -725,17 +765,17 @@ int rst_model_sgd_step(rst_model* m, double lr) {
 namespace {
 
 int run_step(rst_model* m, const double* x, const double* truth, size_t batch, double lr) {
-  const int head = head_layer(m);
-  RST_TRY(do_forward(m, x, batch, nullptr, head));
-  if (head >= 0) {
-    RST_TRY(do_head(m, head, truth));
+  const Tail tail = tail_layers(m);
+  RST_TRY(do_forward(m, x, batch, nullptr, tail));
+  if (tail.head >= 0) {
+    RST_TRY(do_head(m, tail, truth));
   } else {
     RST_TRY(do_loss(m, truth, nullptr));
   }
   if (m->fuse_sgd) {  // SGD::step rides in the epilogues of the weight-gradient launches
-    RST_TRY(do_backward(m, nullptr, 0, nullptr, &lr, nullptr, head));
+    RST_TRY(do_backward(m, nullptr, 0, nullptr, &lr, nullptr, tail));
   } else {
-    RST_TRY(do_backward(m, nullptr, 0, nullptr, nullptr, nullptr, head));
+    RST_TRY(do_backward(m, nullptr, 0, nullptr, nullptr, nullptr, tail));
     RST_TRY(do_sgd(m, lr));
   }
   return RST_OK;
@@ -854,7 +894,7 @@ int rst_model_fuse_sgd(rst_model* m, int enabled) {
 
 int rst_model_fuse_head(rst_model* m, int enabled) {
   if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
-  m->fuse_head = enabled != 0;
+  m->fuse_head = enabled <= 0 ? 0 : enabled == 1 ? 1 : 2;
   drop_graph(m);
   return RST_OK;
 }

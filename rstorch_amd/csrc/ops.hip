@@ -57,12 +57,13 @@ int loss_mirror(rst_engine* e, LossMirror* mirror) {
 
 int engine_head_cross_entropy(rst_engine* e, double* row_loss, const double* h, const double* w,
                               const double* bias, const double* truth, double* logits, double* grad,
-                              double* dx, bool mask, size_t rows, size_t cols, size_t in_features) {
+                              double* dx, bool mask, size_t rows, size_t cols, size_t in_features,
+                              const HiddenLayer* hidden) {
   if (rows == 0 || cols == 0) return fail(RST_ERR_SHAPE, "cross entropy of an empty batch");
   LossMirror mirror;
   RST_TRY(loss_mirror(e, &mirror));
   RST_TRY(launch_head_ce(e->stream, h, w, bias, truth, logits, grad, dx, mask, row_loss, e->d_loss, e->d_flags,
-                         rows, cols, in_features, mirror));
+                         rows, cols, in_features, mirror, hidden));
   e->loss_valid = true;
   return RST_OK;
 }

@@ -411,16 +411,22 @@ __global__ __launch_bounds__(1024) void loss_reduce_kernel(const double* __restr
 // workgroup that arrives last.  For heads of at most kHeadCols classes on a few hundred inputs,
 // where the four launches this replaces are each over before the next one has started.
 //
-// A workgroup of BLOCK threads takes BLOCK / 16 rows, 16 lanes to a row.  Lane j of a row keeps inputs j, j + 16, ...
-// of that row in registers (KI of them at most) and the whole weight matrix sits in LDS.  Logits: the
-// lane adds up its share of every class's dot product in ascending k, a butterfly over the 16 lanes
-// completes the sums (every lane then holds all of them), and lane c goes on with class c through
-// the softmax with the arithmetic of softmax_rows_kernel.  Input gradient: the lanes of a row
-// exchange their gradient entries, and lane j computes elements j, j + 16, ... as sums over the
-// classes in ascending order, masked by the inputs it still holds.
+// A workgroup of BLOCK threads takes BLOCK / 16 rows at a time, 16 lanes to a row.  Lane j of a row
+// keeps inputs j, j + 16, ... of that row in registers (KI of them at most) and the whole weight
+// matrix sits in LDS.  Logits: the lane adds up its share of every class's dot product in ascending
+// k, an exchange over the 16 lanes completes the sums, and lane c goes on with class c through the
+// softmax with the arithmetic of softmax_rows_kernel.  Input gradient: the lanes of a row exchange
+// their gradient entries, and lane j computes elements j, j + 16, ... as sums over the classes in
+// ascending order, masked by the inputs it still holds.
 // The loss: each workgroup adds its rows' terms up in row order, and the workgroup that arrives last
 // adds the workgroups' sums up in a fixed order (thread t sums t, t + BLOCK, ...; a butterfly over each
 // wavefront; the wavefronts in turn), so the result does not depend on which one came last.
+//
+// HID: the Linear in front of the head (at most 112 inputs and outputs) runs in the same launch, so
+// that two more launches - its forward and its input gradient - disappear.  Its weights sit in LDS
+// as well; a workgroup (256 threads) takes 16 rows at a time - one MFMA fragment - and walks over
+// the batch with a stride of the grid (the weights are fetched once per workgroup): hidden forward
+// on the matrix cores, the head as above on the result, hidden input gradient on the matrix cores.
 struct HeadParams {
   const double* h;      // [rows, K] inputs of the Linear (contiguous rows)
   const double* w;      // [N, K]
@@ -436,156 +442,334 @@ struct HeadParams {
   size_t rows;
   int N, K;
   LossMirror mirror;
+  // HID
+  const double* h1;     // [rows, K1] inputs of the hidden Linear
+  const double* w2;     // [K, K1] its weights
+  const double* b2;     // [K]
+  double* h_out;        // [rows, K] its outputs (what `h` is otherwise)
+  double* dx1;          // [rows, K1] the gradient with respect to h1, or NULL
+  int K1;
+  int mask1;            // dx1 is zeroed where h1 <= 0
 };
 
-template <int KI, int NC, bool MASK, int BLOCK>
-__global__ __launch_bounds__(BLOCK) void head_ce_kernel(HeadParams p) {
-  constexpr int ROWS = BLOCK / 16;  // rows per workgroup
+typedef double v4d_t __attribute__((ext_vector_type(4)));
+
+// One 16 x 16 MFMA product chain out of LDS: c += sum over steps s of A[.][4 s + lk] x B[4 s + lk][.],
+// a (resp. b) pointing at this lane's element of step 0 and moving by a_step (b_step) doubles per
+// step; `steps` is a multiple of four.  The reads are inline assembly, so that their place in the
+// instruction stream is fixed and the waits can name how many younger reads may still be
+// outstanding: the operands of four steps are in registers or on their way at any time, in two sets
+// of two steps, and a set's four reads go out as soon as the MFMAs that used its registers have been
+// issued.  Each of the four steps of a round adds up in an accumulator of its own (an MFMA that
+// continues the sum of the one issued just before it would wait for its result); they are added
+// together at the end.  After the last step the requests fetch the last operands again; nobody uses them.
+__device__ __forceinline__ void lds_barrier() {
+  // A workgroup barrier for data exchanged through LDS: this wavefront's LDS accesses are over, then
+  // everybody meets.  Unlike __syncthreads() it does not wait for the stores to global memory that
+  // are still on their way (nobody in the workgroup reads those back), which take a microsecond or two.
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+__device__ __forceinline__ double lds_read_f64(uint32_t byte_address) {
+  double v;
+  asm volatile("ds_read_b64 %0, %1" : "=v"(v) : "v"(byte_address) : "memory");
+  return v;
+}
+__device__ __forceinline__ v4d_t mfma_chain(const double* a, int a_step, const double* b, int b_step, int steps) {
+  uint32_t pa = (uint32_t)(uintptr_t)a, pb = (uint32_t)(uintptr_t)b;
+  const uint32_t da = 8u * (uint32_t)a_step, db = 8u * (uint32_t)b_step;
+  double xa0 = lds_read_f64(pa), xb0 = lds_read_f64(pb);
+  double xa1 = lds_read_f64(pa + da), xb1 = lds_read_f64(pb + db);
+  double ya0 = lds_read_f64(pa + 2 * da), yb0 = lds_read_f64(pb + 2 * db);
+  double ya1 = lds_read_f64(pa + 3 * da), yb1 = lds_read_f64(pb + 3 * db);
+  v4d_t c0 = {0.0, 0.0, 0.0, 0.0}, c1 = c0, c2 = c0, c3 = c0;
+  for (int s = 0; s < steps; s += 4) {
+    const bool more = s + 4 < steps;
+    pa += more ? 4 * da : 0;
+    pb += more ? 4 * db : 0;
+    asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(xa0), "+v"(xb0), "+v"(xa1), "+v"(xb1));
+    c0 = __builtin_amdgcn_mfma_f64_16x16x4f64(xa0, xb0, c0, 0, 0, 0);
+    c1 = __builtin_amdgcn_mfma_f64_16x16x4f64(xa1, xb1, c1, 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    xa0 = lds_read_f64(pa);
+    xb0 = lds_read_f64(pb);
+    xa1 = lds_read_f64(pa + da);
+    xb1 = lds_read_f64(pb + db);
+    asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(ya0), "+v"(yb0), "+v"(ya1), "+v"(yb1));
+    c2 = __builtin_amdgcn_mfma_f64_16x16x4f64(ya0, yb0, c2, 0, 0, 0);
+    c3 = __builtin_amdgcn_mfma_f64_16x16x4f64(ya1, yb1, c3, 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    ya0 = lds_read_f64(pa + 2 * da);
+    yb0 = lds_read_f64(pb + 2 * db);
+    ya1 = lds_read_f64(pa + 3 * da);
+    yb1 = lds_read_f64(pb + 3 * db);
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(xa0), "+v"(xb0), "+v"(xa1), "+v"(xb1), "+v"(ya0), "+v"(yb0), "+v"(ya1), "+v"(yb1));
+  return (c0 + c1) + (c2 + c3);
+}
+
+// (two wavefronts per SIMD as the floor of the register budget: with the whole register file to itself
+// the compiler would park the MFMA accumulators in the accumulation registers and copy them back and
+// forth around every instruction of the chain)
+template <int KI, int NC, bool MASK, int BLOCK, bool HID = false>
+__global__ __launch_bounds__(BLOCK, 2) void head_ce_kernel(HeadParams p) {
+  // rows per workgroup and pass (HID: one 16-row MFMA fragment; the wavefronts beyond the first four
+  // only take part in the matrix-core phases and in the copies)
+  constexpr int ROWS = HID ? 16 : BLOCK / 16;
+  constexpr int NW = BLOCK / 64;
   static_assert(NC == 4 || NC == 8 || NC == 16, "the class sums are exchanged by halving");
+  static_assert(!HID || (BLOCK == 512 && KI == 8), "the hidden layer: eight wavefronts, one output fragment each");
   // the weights, transposed: [16 * KI][P], the NC classes of one input side by side, zero from class N
   // and from input K on; with P = NC + 2 the 16 lanes of a row, which read 16 consecutive inputs, hit
   // different banks
   extern __shared__ __attribute__((aligned(16))) double head_ws[];
   constexpr int P = NC + 2;
+  // HID: behind them the hidden layer's weights [n][k] (rows of P1 doubles, zero past its extents), the
+  // 16 input rows [m][k] (P1) and a [16][PH] panel that first holds the hidden layer's output and
+  // then the gradient with respect to it
+  constexpr int PH = 16 * KI + 2;
+  const int K = p.K, N = p.N, K1 = HID ? p.K1 : 0;
+  const int KP1 = (K1 + 15) / 16 * 16, P1 = KP1 + 2;  // (MFMA steps in fours)
+  const int NF2 = HID ? (K + 15) / 16 : 0, NF1 = (K1 + 15) / 16;
+  double* const w2s = head_ws + 16 * KI * P;
+  double* const h1s = w2s + (size_t)NF2 * 16 * P1 + 16;
+  double* const hg = h1s + 16 * P1;
   __shared__ double wave_sum[BLOCK / 64];
   __shared__ double row_sum[ROWS];
   __shared__ int nan_here, last_nan;
   __shared__ bool is_last;
   const int t = threadIdx.x;
   if (t == 0) nan_here = 0;
-  const int K = p.K, N = p.N;
   const int r = t >> 4, j = t & 15;
-  const size_t row0 = (size_t)blockIdx.x * ROWS;
-  const size_t row = row0 + r;
-  const bool row_ok = row < p.rows;
+  const bool head_thread = r < ROWS;
+  const int lane = t & 63, wave = t >> 6, lr = lane & 15, lk = lane >> 4;
+  const size_t passes_all = (p.rows + ROWS - 1) / ROWS;
 
-  // every global load of the workgroup is issued before the first one is waited for
-  double hv[KI];
-  {
-    const double* hr = p.h + row * (size_t)K;
+  // the weights: every global load of a batch is issued before the first one is waited for
+  for (int k = t; k < 16 * KI; k += BLOCK) {  // (at most two rounds)
+    double v[NC];
 #pragma unroll
-    for (int i = 0; i < KI; ++i) {
-      const int k = j + 16 * i;
-      hv[i] = (row_ok && k < K) ? hr[k] : 0.0;
-    }
-    for (int k = t; k < 16 * KI; k += BLOCK) {  // (at most two rounds)
-      double v[NC];
+    for (int c = 0; c < NC; ++c) v[c] = (c < N && k < K) ? p.w[(size_t)c * K + k] : 0.0;
 #pragma unroll
-      for (int c = 0; c < NC; ++c) v[c] = (c < N && k < K) ? p.w[(size_t)c * K + k] : 0.0;
+    for (int c = 0; c < NC; c += 2) *reinterpret_cast<v2d*>(head_ws + k * P + c) = v2d{v[c], v[c + 1]};
+  }
+  if (HID) {
+    // a wavefront takes every eighth row of the padded matrix, a lane one pair of columns
+    constexpr int U = 14;
+    const int kp = 2 * lane;
+    for (int n0 = wave; n0 < NF2 * 16; n0 += NW * U) {
+      double v[U][2];
 #pragma unroll
-      for (int c = 0; c < NC; c += 2) *reinterpret_cast<v2d*>(head_ws + k * P + c) = v2d{v[c], v[c + 1]};
+      for (int u = 0; u < U; ++u) {
+        const int n = n0 + NW * u;
+        const bool row_in = n < K;
+        v[u][0] = (row_in && kp < K1) ? p.w2[(size_t)n * K1 + kp] : 0.0;
+        v[u][1] = (row_in && kp + 1 < K1) ? p.w2[(size_t)n * K1 + kp + 1] : 0.0;
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int n = n0 + NW * u;
+        if (n < NF2 * 16 && kp < P1) *reinterpret_cast<v2d*>(w2s + n * P1 + kp) = v2d{v[u][0], v[u][1]};
+      }
     }
   }
-  const double bias = j < N ? p.bias[j] : 0.0;
-  const double tv = (row_ok && j < N) ? p.truth[row * N + j] : 0.0;
-  __syncthreads();
 
-  // logits.  No branch in the loops (a branch would have every LDS read waited for on its own): an
-  // index past the row is clamped and its product replaced by zero; classes from N on have zero weights.
-  // (inputs and weights past the row's end are zero, so the loops carry no test; the weights of the
-  // next input are on their way while those of this one are used)
-  double acc[NC];
+  // HID: the 16 input rows of a pass travel through registers
+  constexpr int RU = 16 / NW > 0 ? 16 / NW : 1;
+  double h1v[RU][2];
+  auto fetch_inputs = [&](size_t pass) {
+    const size_t first = pass * ROWS;
+    const int kp = 2 * lane;
 #pragma unroll
-  for (int c = 0; c < NC; ++c) acc[c] = 0.0;
-  const v2d* const wj = reinterpret_cast<const v2d*>(head_ws + j * P);  // input j + 16 i: wj + i * 8 P
-  {
-    v2d w2[2][NC / 2];
-#pragma unroll
-    for (int c = 0; c < NC / 2; ++c) w2[0][c] = wj[c];
-#pragma unroll
-    for (int i = 0; i < KI; ++i) {
-      if (i + 1 < KI) {
-#pragma unroll
-        for (int c = 0; c < NC / 2; ++c) w2[(i + 1) & 1][c] = wj[(i + 1) * 8 * P + c];
-      }
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int c = 0; c < NC / 2; ++c) {
-        acc[2 * c] = fma(hv[i], w2[i & 1][c].x, acc[2 * c]);
-        acc[2 * c + 1] = fma(hv[i], w2[i & 1][c].y, acc[2 * c + 1]);
-      }
-      __builtin_amdgcn_sched_barrier(0);
+    for (int u = 0; u < RU; ++u) {
+      const int m = wave + NW * u;
+      const bool in = m < 16 && first + m < p.rows;
+      h1v[u][0] = (in && kp < K1) ? p.h1[(first + m) * (size_t)K1 + kp] : 0.0;
+      h1v[u][1] = (in && kp + 1 < K1) ? p.h1[(first + m) * (size_t)K1 + kp + 1] : 0.0;
     }
-  }
-  // The 16 lanes of a row add their shares up by halving: with offset 8, 4, 2, 1 in turn a lane keeps
-  // the classes whose index has the lane's bit at that position and receives its partner's share of
-  // them, so that lane j ends with the whole sum of class j (lanes from NC on: a class below NC again).
-#pragma unroll
-  for (int off = 8; off > 0; off >>= 1) {
-    if (off < NC) {
-      const bool upper = (j & off) != 0;
-#pragma unroll
-      for (int i = 0; i < off; ++i) {
-        const double lo = acc[i], hi = acc[i + off < NC ? i + off : i];
-        const double got = __shfl_xor(upper ? lo : hi, off);
-        acc[i] = (upper ? hi : lo) + got;
-      }
-    } else {  // fewer classes than 2 * off: every lane keeps all of them
-#pragma unroll
-      for (int c = 0; c < NC; ++c) acc[c] = acc[c] + __shfl_xor(acc[c], off);
-    }
-  }
-  double z = acc[0];
-  const bool col_ok = j < N, ok = row_ok && col_ok;
-  z = z + bias;
-  const bool saw_nan = ok && z != z;
-  double mx = col_ok ? MaxOp::apply(-DBL_MAX, z) : -DBL_MAX;
-  mx = group_reduce<kHeadCols, MaxOp>(mx, nullptr);
-  const double ev = col_ok ? exp(z - mx) : 0.0;
-  const double s = group_reduce<kHeadCols, SumOp>(ev, nullptr);
-  double lsum = 0.0, g = 0.0;
-  if (ok) {
-    const double pr = ev / s;
-    lsum = loss_term(tv, pr);
-    g = -(tv - pr);
-    p.grad[row * N + j] = g;
-    p.logits[row * N + j] = z;
-  }
-  lsum = group_reduce<kHeadCols, SumOp>(lsum, nullptr);
-  if (j == 0) row_sum[r] = row_ok ? lsum : 0.0;
-  if (saw_nan) nan_here = 1;  // (every writer writes the same value)
-  __syncthreads();
+  };
+  if (HID) fetch_inputs(blockIdx.x);
 
-  // The loss.  Thread 0 hands this workgroup's sum over with an atomic exchange, which is carried out
-  // where every workgroup of the device sees it, and only then - the exchange's return value is an
-  // operand of the addition - counts the workgroup in at `arrivals` (low word: workgroups, high word:
-  // those that met a NaN logit).  Whoever counts in last therefore finds every other sum in place and
-  // reads them with atomic loads.  No fence is involved: a device-wide release would have every
-  // workgroup write the whole L2 back.  The exchange travels while the input gradient is computed.
-  unsigned long long* const partial = reinterpret_cast<unsigned long long*>(p.partial);
+  double mine = 0.0;  // (thread 0) the workgroup's loss terms so far
   unsigned long long old = 0;
-  if (t == 0) {
-    double mine = 0.0;
+  unsigned long long* const partial = reinterpret_cast<unsigned long long*>(p.partial);
+  for (size_t pass = blockIdx.x; pass < passes_all; pass += gridDim.x) {
+    const bool last_pass = pass + gridDim.x >= passes_all;
+    const size_t row0 = pass * ROWS;
+    const size_t row = row0 + r;
+    const bool row_ok = row < p.rows;
+    double hv[KI];
+    if (!HID) {
+      const double* hr = p.h + row * (size_t)K;
 #pragma unroll
-    for (int i = 0; i < ROWS; ++i) mine += row_sum[i];
-    old = atomicExch(partial + blockIdx.x, (unsigned long long)__double_as_longlong(mine));
-  }
+      for (int i = 0; i < KI; ++i) {
+        const int k = j + 16 * i;
+        hv[i] = (row_ok && k < K) ? hr[k] : 0.0;
+      }
+    } else {
+      // (the previous pass is done with the input rows and the panel)
+      if (pass != blockIdx.x) lds_barrier();
+      // the 16 input rows, requested during the previous pass: a wavefront takes every eighth row, a
+      // lane a pair of columns
+#pragma unroll
+      for (int u = 0; u < RU; ++u)
+        if (wave + NW * u < 16 && 2 * lane < P1)
+          *reinterpret_cast<v2d*>(h1s + (wave + NW * u) * P1 + 2 * lane) = v2d{h1v[u][0], h1v[u][1]};
+      fetch_inputs(pass + gridDim.x);  // (for the next pass; beyond the batch: zeros, unused)
+    }
+    const double bias = (head_thread && j < N) ? p.bias[j] : 0.0;
+    const double tv = (head_thread && row_ok && j < N) ? p.truth[row * N + j] : 0.0;
+    const double b2v = (HID && wave * 16 + lr < K) ? p.b2[wave * 16 + lr] : 0.0;
+    lds_barrier();
 
-  if (p.dx) {
-    double gc[NC];
+    if (HID) {
+      // The hidden Linear (src/module/linear.rs:44-58) on the 16 rows: wavefront w computes the 16-column
+      // fragment w of the output with FP64 MFMAs, four contraction indices a step, both
+      // operands from LDS; bias and ReLU as in the contraction kernels' epilogue; the result goes to
+      // memory (the head's weight gradient reads it) and into the panel for the head below.
+      if (wave < NF2) {
+        const v4d_t c = mfma_chain(h1s + lr * P1 + lk, 4, w2s + (wave * 16 + lr) * P1 + lk, 4, KP1 / 4);
+        const int col = wave * 16 + lr;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) gc[c] = __shfl(g, c, 16);  // (zero from class N on)
-    double* const dr = p.dx + row * (size_t)K;
-    v2d w2[2][NC / 2];
-#pragma unroll
-    for (int c = 0; c < NC / 2; ++c) w2[0][c] = wj[c];
-#pragma unroll
-    for (int i = 0; i < KI; ++i) {
-      const int k = j + 16 * i;
-      if (i + 1 < KI) {
-#pragma unroll
-        for (int c = 0; c < NC / 2; ++c) w2[(i + 1) & 1][c] = wj[(i + 1) * 8 * P + c];
+        for (int q = 0; q < 4; ++q) {
+          const int m = 4 * q + lk;
+          double v = c[q] + b2v;
+          if (MASK) v = fmax(v, 0.0);
+          if (col >= K) v = 0.0;
+          hg[m * PH + col] = v;
+          if (row0 + m < p.rows && col < K) p.h_out[(row0 + m) * (size_t)K + col] = v;
+        }
       }
-      __builtin_amdgcn_sched_barrier(0);
-      double a = 0.0;
+      lds_barrier();
 #pragma unroll
-      for (int c = 0; c < NC / 2; ++c) {
-        a = fma(gc[2 * c], w2[i & 1][c].x, a);
-        a = fma(gc[2 * c + 1], w2[i & 1][c].y, a);
+      for (int i = 0; i < KI; ++i) {
+        const int k = j + 16 * i;
+        hv[i] = (head_thread && k < NF2 * 16) ? hg[r * PH + k] : 0.0;
       }
-      if (MASK) a = a * (hv[i] > 0.0 ? 1.0 : 0.0);
-      if (row_ok && k < K) dr[k] = a;
-      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // logits.  No branch in the loop (a branch would have every LDS read waited for on its own): inputs
+    // and weights past the row's end are zero; the weights of the next input are on their way while
+    // those of this one are used.
+    const v2d* const wj = reinterpret_cast<const v2d*>(head_ws + j * P);  // input j + 16 i: wj + i * 8 P
+    double g = 0.0;  // this lane's entry of the loss gradient
+    if (head_thread) {
+    double acc[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) acc[c] = 0.0;
+    {
+      v2d w2[2][NC / 2];
+#pragma unroll
+      for (int c = 0; c < NC / 2; ++c) w2[0][c] = wj[c];
+#pragma unroll
+      for (int i = 0; i < KI; ++i) {
+        if (i + 1 < KI) {
+#pragma unroll
+          for (int c = 0; c < NC / 2; ++c) w2[(i + 1) & 1][c] = wj[(i + 1) * 8 * P + c];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int c = 0; c < NC / 2; ++c) {
+          acc[2 * c] = fma(hv[i], w2[i & 1][c].x, acc[2 * c]);
+          acc[2 * c + 1] = fma(hv[i], w2[i & 1][c].y, acc[2 * c + 1]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    // The 16 lanes of a row add their shares up by halving: with offset 8, 4, 2, 1 in turn a lane keeps
+    // the classes whose index has the lane's bit at that position and receives its partner's share of
+    // them, so that lane j ends with the whole sum of class j (lanes from NC on: a class below NC again).
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) {
+      if (off < NC) {
+        const bool upper = (j & off) != 0;
+#pragma unroll
+        for (int i = 0; i < off; ++i) {
+          const double lo = acc[i], hi = acc[i + off < NC ? i + off : i];
+          const double got = __shfl_xor(upper ? lo : hi, off);
+          acc[i] = (upper ? hi : lo) + got;
+        }
+      } else {  // fewer classes than 2 * off: every lane keeps all of them
+#pragma unroll
+        for (int c = 0; c < NC; ++c) acc[c] = acc[c] + __shfl_xor(acc[c], off);
+      }
+    }
+    double z = acc[0];
+    const bool col_ok = j < N, ok = row_ok && col_ok;
+    z = z + bias;
+    const bool saw_nan = ok && z != z;
+    double mx = col_ok ? MaxOp::apply(-DBL_MAX, z) : -DBL_MAX;
+    mx = group_reduce<kHeadCols, MaxOp>(mx, nullptr);
+    const double ev = col_ok ? exp(z - mx) : 0.0;
+    const double s = group_reduce<kHeadCols, SumOp>(ev, nullptr);
+    double lsum = 0.0;
+    if (ok) {
+      const double pr = ev / s;
+      lsum = loss_term(tv, pr);
+      g = -(tv - pr);
+      p.grad[row * N + j] = g;
+      p.logits[row * N + j] = z;
+    }
+    lsum = group_reduce<kHeadCols, SumOp>(lsum, nullptr);
+    if (j == 0) row_sum[r] = row_ok ? lsum : 0.0;
+    if (saw_nan) nan_here = 1;  // (every writer writes the same value)
+    }
+    lds_barrier();
+
+    // The loss.  Thread 0 hands this workgroup's sum over with an atomic exchange, which is carried out
+    // where every workgroup of the device sees it, and only then - the exchange's return value is an
+    // operand of the addition - counts the workgroup in at `arrivals` (low word: workgroups, high word:
+    // those that met a NaN logit).  Whoever counts in last therefore finds every other sum in place and
+    // reads them with atomic loads.  No fence is involved: a device-wide release would have every
+    // workgroup write the whole L2 back.  The exchange travels while the input gradients are computed.
+    if (t == 0) {
+#pragma unroll
+      for (int i = 0; i < ROWS; ++i) mine += row_sum[i];
+      if (last_pass) old = atomicExch(partial + blockIdx.x, (unsigned long long)__double_as_longlong(mine));
+    }
+
+    if (p.dx && head_thread) {
+      double gc[NC];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) gc[c] = __shfl(g, c, 16);  // (zero from class N on)
+      double* const dr = p.dx + row * (size_t)K;
+      v2d w2[2][NC / 2];
+#pragma unroll
+      for (int c = 0; c < NC / 2; ++c) w2[0][c] = wj[c];
+#pragma unroll
+      for (int i = 0; i < KI; ++i) {
+        const int k = j + 16 * i;
+        if (i + 1 < KI) {
+#pragma unroll
+          for (int c = 0; c < NC / 2; ++c) w2[(i + 1) & 1][c] = wj[(i + 1) * 8 * P + c];
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        double a = 0.0;
+#pragma unroll
+        for (int c = 0; c < NC / 2; ++c) {
+          a = fma(gc[2 * c], w2[i & 1][c].x, a);
+          a = fma(gc[2 * c + 1], w2[i & 1][c].y, a);
+        }
+        if (MASK) a = a * (hv[i] > 0.0 ? 1.0 : 0.0);
+        if (row_ok && k < K) dr[k] = a;
+        if (HID) hg[r * PH + k] = k < K ? a : 0.0;  // (every lane took its inputs from the panel before the last barrier)
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    if (HID && p.dx1) {
+      // The hidden Linear's input gradient (linear.rs:68): [16, K] x [K, K1] from the panel and the
+      // weights in LDS, fragment by fragment as above, zeroed where the ReLU in front of it was off.
+      lds_barrier();
+      if (wave < NF1) {
+        const v4d_t c = mfma_chain(hg + lr * PH + lk, 4, w2s + lk * P1 + wave * 16 + lr, 4 * P1, NF2 * 4);
+        const int col = wave * 16 + lr;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int m = 4 * q + lk;
+          double v = c[q];
+          if (p.mask1) v = v * ((col < K1 ? h1s[m * P1 + col] : 0.0) > 0.0 ? 1.0 : 0.0);
+          if (row0 + m < p.rows && col < K1) p.dx1[(row0 + m) * (size_t)K1 + col] = v;
+        }
+      }
     }
   }
 
@@ -762,17 +946,37 @@ bool head_ce_supported(size_t cols, size_t in_features) {
   return cols >= 1 && cols <= (size_t)kHeadCols && in_features >= 1 && in_features <= 16 * 18;
 }
 
+namespace {
+// LDS of the variant that also runs the hidden Linear: the head's weights, the hidden weights padded
+// to whole fragments, 16 input rows and the [16][130] panel
+size_t tail_lds_bytes(size_t cols, size_t hidden, size_t in_features) {
+  const size_t nc = cols <= 4 ? 4 : cols <= 8 ? 8 : 16;
+  const size_t p1 = (in_features + 15) / 16 * 16 + 2, nf2 = (hidden + 15) / 16;
+  return (16 * 8 * (nc + 2) + nf2 * 16 * p1 + 16 + 16 * p1 + 16 * (16 * 8 + 2)) * sizeof(double);
+}
+}  // namespace
+
+bool tail_ce_supported(size_t cols, size_t hidden, size_t in_features, size_t lds_limit) {
+  return head_ce_supported(cols, hidden) && hidden <= 112 && in_features >= 1 && in_features <= 112 &&
+         tail_lds_bytes(cols, hidden, in_features) <= lds_limit;
+}
+
 int launch_head_ce(hipStream_t s, const double* h, const double* w, const double* bias, const double* truth,
                    double* logits, double* grad, double* dx, bool mask, double* row_loss, double* loss,
-                   int* flags, size_t rows, size_t cols, size_t in_features, LossMirror mirror) {
+                   int* flags, size_t rows, size_t cols, size_t in_features, LossMirror mirror,
+                   const HiddenLayer* hidden) {
   if (!head_ce_supported(cols, in_features))
     return fail(RST_ERR_UNSUPPORTED, "fused head: %zu classes on %zu inputs do not fit", cols, in_features);
+  if (hidden && (in_features > 112 || hidden->in_features > 112 || !dx))
+    return fail(RST_ERR_UNSUPPORTED, "fused head with its hidden layer: %zu on %zu inputs do not fit",
+                in_features, hidden->in_features);
   if (rows == 0) return RST_OK;
   // 16 rows to a workgroup while that leaves every compute unit with work, 32 beyond (each workgroup
-  // pays a round trip to the one arrival counter)
-  const int block_threads = rows <= 16 * 512 / 2 ? 256 : 512;
-  const size_t rows_per_block = block_threads / 16;
+  // pays a round trip to the one arrival counter); with the hidden layer 16 (one MFMA fragment) on 512 threads
+  const int block_threads = (hidden || rows > 16 * 512 / 2) ? 512 : 256;
+  const size_t rows_per_block = hidden ? 16 : block_threads / 16;
   const size_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+  if (blocks > 0x7fffffffull) return fail(RST_ERR_UNSUPPORTED, "too many rows for one launch");
   HeadParams p{};
   p.h = h; p.w = w; p.bias = bias; p.truth = truth;
   p.logits = logits; p.grad = grad; p.dx = dx;
@@ -784,8 +988,27 @@ int launch_head_ce(hipStream_t s, const double* h, const double* w, const double
   p.mirror.hits = nullptr;  // the hit count is not taken here
   const bool masked = mask && dx;
   const int nc = cols <= 4 ? 4 : cols <= 8 ? 8 : 16;
+  // (with the hidden layer: one workgroup per compute unit of the part at most - a constant, the grid
+  // fixes the order in which the loss is summed - each walking over the batch)
+  const dim3 grid((unsigned)(hidden && blocks > 256 ? 256 : blocks)), block(block_threads);
+  if (hidden) {
+    p.h1 = hidden->input; p.w2 = hidden->weight; p.b2 = hidden->bias;
+    p.h_out = hidden->output; p.dx1 = hidden->input_grad;
+    p.K1 = (int)hidden->in_features; p.mask1 = hidden->mask_input_grad ? 1 : 0;
+    const size_t lds = tail_lds_bytes(cols, in_features, hidden->in_features);
+#define RST_TAIL_LAUNCH(NC)                                                                          \
+  do {                                                                                               \
+    if (masked) hipLaunchKernelGGL((head_ce_kernel<8, NC, true, 512, true>), grid, block, lds, s, p); \
+    else hipLaunchKernelGGL((head_ce_kernel<8, NC, false, 512, true>), grid, block, lds, s, p);      \
+  } while (0)
+    if (nc == 4) RST_TAIL_LAUNCH(4);
+    else if (nc == 8) RST_TAIL_LAUNCH(8);
+    else RST_TAIL_LAUNCH(16);
+#undef RST_TAIL_LAUNCH
+    RST_HIP(hipGetLastError());
+    return RST_OK;
+  }
   const size_t lds = (size_t)(nc + 2) * 16 * (in_features <= 16 * 8 ? 8 : 18) * sizeof(double);
-  const dim3 grid((unsigned)blocks), block(block_threads);
 #define RST_HEAD_LAUNCH3(KI, NC, M, B) hipLaunchKernelGGL((head_ce_kernel<KI, NC, M, B>), grid, block, lds, s, p)
 #define RST_HEAD_LAUNCH(KI, NC)                                  \
   do {                                                           \

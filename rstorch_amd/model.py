@@ -190,10 +190,12 @@ class DeviceModel:
         """Apply SGD inside the weight-gradient launches of train_step (default) or as a pass."""
         _ffi.check(self.engine.lib.rst_model_fuse_sgd(self.handle, 1 if on else 0))
 
-    def fuse_head(self, on=True):
-        """Run a small classifier head (last Linear, cross entropy, its input gradient) as one
-        launch inside train_step (default) or as the separate launches."""
-        _ffi.check(self.engine.lib.rst_model_fuse_head(self.handle, 1 if on else 0))
+    def fuse_head(self, mode=True):
+        """How much of a small classifier's tail train_step runs as one launch: False / 0 nothing (the
+        separate launches), 1 the last Linear with the cross entropy and its input gradient, True / 2
+        (default) also the Linear in front of it when both are small."""
+        level = 2 if mode is True else 0 if mode is False else int(mode)
+        _ffi.check(self.engine.lib.rst_model_fuse_head(self.handle, level))
 
     def pair_gradients(self, on=True):
         """Launch a layer's weight gradient in one grid with the next layer's input gradient

@@ -156,12 +156,16 @@ def test_profile_records_cover_every_launch(engine, oracle):
     dm.train_step(x, y, 0.01)
     recs = dm.profile_read()
     kinds = [r["kernel"] for r in recs]
-    # the last Linear's forward and input gradient run inside the cross-entropy launch (the fused head);
-    # the first layer's input gradient is skipped
-    assert kinds.count("linear_forward") == 2 and kinds.count("grad_weight") == 3
-    assert kinds.count("grad_input") == 1
+    # the last two Linears' forward and input gradients run inside the cross-entropy launch (the fused
+    # tail of a small classifier); the first layer's input gradient is skipped
+    assert kinds.count("linear_forward") == 1 and kinds.count("grad_weight") == 3
+    assert kinds.count("grad_input") == 0
     # the optimiser rides in the weight-gradient launches unless asked to be a pass of its own
     assert kinds.count("cross_entropy") == 1 and kinds.count("sgd") == 0
+    dm.fuse_head(1)   # the head alone
+    dm.train_step(x, y, 0.01)
+    kinds = [r["kernel"] for r in dm.profile_read()]
+    assert kinds.count("linear_forward") == 2 and kinds.count("grad_input") == 1 and kinds.count("cross_entropy") == 1
     dm.fuse_head(False)
     dm.train_step(x, y, 0.01)
     kinds = [r["kernel"] for r in dm.profile_read()]

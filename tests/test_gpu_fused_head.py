@@ -14,13 +14,17 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-10
 
 SPECS = {
-    "readme": README_MLP,
+    "readme": README_MLP,                                                # hidden 100 x 100 with the head, masks on both sides
     "head_only": [("linear", 20, 10)],                                   # the head is the first Linear: no input gradient
     "identity_then_head": [("identity",), ("linear", 7, 3), ("identity",)],
-    "no_mask": [("linear", 12, 9), ("linear", 9, 16)],                   # a Linear feeds the head: gradient unmasked
+    "no_mask": [("linear", 12, 9), ("linear", 9, 16)],                   # a Linear feeds the head: gradient unmasked; it is the first Linear
     "relu_of_its_own": [("relu",), ("linear", 30, 21), ("identity",), ("relu",), ("linear", 21, 7)],
-    "widest": [("linear", 64, 233), ("relu",), ("linear", 233, 16)],     # 16 classes on 233 inputs: the LDS limit
+    "widest": [("linear", 64, 233), ("relu",), ("linear", 233, 16)],     # 16 classes on 233 inputs: the head alone
     "one_class": [("linear", 5, 8), ("relu",), ("linear", 8, 1)],
+    "linear_in_front": [("linear", 20, 24), ("linear", 24, 18), ("relu",), ("linear", 18, 3)],   # hidden gradient unmasked
+    "odd_extents": [("linear", 50, 111), ("relu",), ("linear", 111, 97), ("relu",), ("linear", 97, 13)],
+    "limit": [("linear", 9, 112), ("relu",), ("linear", 112, 112), ("relu",), ("linear", 112, 16)],
+    "hidden_too_wide": [("linear", 30, 200), ("relu",), ("linear", 200, 100), ("relu",), ("linear", 100, 10)],
 }
 CASES = [("readme", b) for b in (1, 5, 16, 17, 32, 100, 1000, 8192)] + \
         [(name, b) for name in SPECS if name != "readme" for b in (3, 48)]
@@ -33,6 +37,8 @@ def test_fused_head_matches_oracle_and_separate_launches(engine, oracle, name, b
     fused, ref = pair(rs, oracle, spec, 0xC1A55)
     apart, _ = pair(rs, oracle, spec, 0xC1A55)
     apart.fuse_head(False)
+    head_alone, _ = pair(rs, oracle, spec, 0xC1A55)
+    head_alone.fuse_head(1)
     oracle.set_threads(8)
     try:
         n_in, n_out = fused.in_width, fused.out_width
@@ -40,12 +46,16 @@ def test_fused_head_matches_oracle_and_separate_launches(engine, oracle, name, b
             x, y = batch_data(oracle, batch, n_in, n_out, 23, step, True)
             got = fused.train_step(x, y, 0.05)
             other = apart.train_step(x, y, 0.05)
+            middle = head_alone.train_step(x, y, 0.05)
             want = ref.train_step(x, y, 0.05)
             assert abs(got - want) <= TOL * abs(want), "step %d" % step
+            assert abs(middle - want) <= TOL * abs(want), "step %d" % step
             assert abs(got - other) <= 1e-13 * abs(other), "step %d" % step
-            for (p, g), (q, h), (rp, rg) in zip(fused.parameters(), apart.parameters(), ref.parameters()):
+            for (p, g), (q, h), (u, v), (rp, rg) in zip(fused.parameters(), apart.parameters(),
+                                                        head_alone.parameters(), ref.parameters()):
                 assert rel_err(g.to_numpy(), rg) <= TOL
                 assert rel_err(p.to_numpy(), rp) <= TOL
+                assert rel_err(v.to_numpy(), rg) <= TOL
                 assert rel_err(g.to_numpy(), h.to_numpy()) <= 1e-12
     finally:
         oracle.set_threads(1)
