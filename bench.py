@@ -372,7 +372,8 @@ def bench_small(rs, eng, spec, batch, normal, steps, warmup, eager, profile_step
     dm, x, y = make_model(rs, eng, spec, batch, normal)
     if eager:
         dm.graph_enable(False)
-    out = {"batch": batch, "steps": steps, "launch_mode": "plain launches" if eager else "graph replay"}
+    out = {"batch": batch, "steps": steps,
+           "launch_mode": "graph replay" if dm.graph_active() else "plain launches"}
     if fresh_inputs:
         loader = rs.Engine(eng.device)
         wall, loss = time_fresh_steps(rs, eng, loader, dm, batch, normal, steps, warmup, False)

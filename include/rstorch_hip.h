@@ -294,13 +294,21 @@ int rst_model_pair_gradients(rst_model* model, int enabled);
  * workgroups finish.  The separate calls (rst_model_forward / _loss / _backward, and the *_to variants)
  * are not affected. */
 int rst_model_fuse_head(rst_model* model, int enabled);
-/* rst_model_train_step records its launches into a HIP graph the first time it sees a given
- * (x, truth, batch, lr) and replays the graph afterwards; a different argument re-records (the 64
- * most recently used graphs of a model are kept).
- * enabled == 0 switches to plain launches (profiling does so by itself).  Default: enabled,
- * unless the environment says RSTORCH_GRAPH=0. */
+/* How rst_model_train_step launches its kernels.
+ * enabled == 1: it records them into a HIP graph the first time it sees a given (x, truth, batch, lr)
+ * and replays the graph afterwards; a different argument re-records (the 64 most recently used graphs
+ * of a model are kept).  enabled == 0: plain launches (profiling does so by itself).
+ * enabled == 2, the default: the graph for models of eight Linear layers or more, plain launches for
+ * shallower ones - measured on MI355X, a replayed graph of the four or five launches of a shallow
+ * model's step starts later than the first of as many plain launches and costs the host 12 us more
+ * when it reads the loss after every step (the README network at batch 32 with the loss read every
+ * step: 30.0 k steps/s plain, 19.3 k replayed), while from about 25 small launches per step on the
+ * graph is ahead.  The environment variable RSTORCH_GRAPH (0 or 1) fixes the mode new models start
+ * with.  rst_model_graph_active tells whether the model's next step would be replayed. */
 int rst_model_graph_enable(rst_model* model, int enabled);
-/* Environment variables read once per process.  RSTORCH_GRAPH=0: new models launch plainly.
+int rst_model_graph_active(rst_model* model, int* active);
+/* Environment variables read once per process.  RSTORCH_GRAPH=0 / 1: new models launch plainly / replay
+ * a recorded graph, whatever their depth.
  * The next two change which kernel a product runs on and therefore the ORDER of its summation
  * (results stay within rounding, 1e-13 relative, of each other; every setting is deterministic and
  * independent of the number of compute units):

@@ -116,6 +116,7 @@ SIGNATURES = {
     "rst_model_train_step": [_vp, _dp, _dp, _sz, _dbl, c_double_p],
     "rst_model_profile_enable": [_vp, _i32],
     "rst_model_graph_enable": [_vp, _i32],
+    "rst_model_graph_active": [_vp, ctypes.POINTER(ctypes.c_int)],
     "rst_model_fuse_sgd": [_vp, _i32],
     "rst_model_fuse_head": [_vp, _i32],
     "rst_model_pair_gradients": [_vp, _i32],

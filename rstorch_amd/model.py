@@ -203,8 +203,15 @@ class DeviceModel:
         _ffi.check(self.engine.lib.rst_model_pair_gradients(self.handle, 1 if on else 0))
 
     def graph_enable(self, on=True):
-        """Replay the step as a HIP graph (default) or launch its kernels one by one."""
-        _ffi.check(self.engine.lib.rst_model_graph_enable(self.handle, 1 if on else 0))
+        """Replay the step as a HIP graph (True), launch its kernels one by one (False), or let the
+        model's depth decide ("auto", the default: a graph from eight Linear layers on)."""
+        mode = 2 if on == "auto" else 1 if on else 0
+        _ffi.check(self.engine.lib.rst_model_graph_enable(self.handle, mode))
+
+    def graph_active(self):
+        v = ctypes.c_int()
+        _ffi.check(self.engine.lib.rst_model_graph_active(self.handle, ctypes.byref(v)))
+        return bool(v.value)
 
     # -- per-kernel timing -------------------------------------------------------------------
     def profile_enable(self, on=True):

@@ -44,6 +44,7 @@ struct Spec {
 static rst_model* build(rst_engine* e, const Spec& s) {
   rst_model* m = nullptr;
   OK(rst_model_create(e, s.kinds.data(), s.in.data(), s.out.data(), s.kinds.size(), &m));
+  OK(rst_model_graph_enable(m, 1));  // whatever its depth: the graph lifetimes are what is checked here
   return m;
 }
 

@@ -240,7 +240,8 @@ def test_graph_replay_equals_eager_launches(engine, oracle):
     import rstorch_amd as rs
     spec = README_MLP
     weights = make_weights(oracle, spec, 21)
-    g = rs.DeviceModel(spec); g.load_parameters(weights)          # graph replay (default)
+    g = rs.DeviceModel(spec); g.load_parameters(weights); g.graph_enable(True)   # graph replay
+    assert g.graph_active()
     e = rs.DeviceModel(spec); e.load_parameters(weights); e.graph_enable(False)
     other = rs.Linear.new(64, 64)
     x0, y0 = batch_data(oracle, 32, 784, 10, 5, 0)
@@ -367,6 +368,7 @@ def test_recorded_step_survives_other_users_of_the_engine(engine, oracle):
     y = engine.from_numpy(oracle.fill_one_hot(256, 24, 3, 11))
     a, twin = rs.DeviceModel(spec, engine), rs.DeviceModel(spec, engine)
     a.load_parameters(weights); twin.load_parameters(weights)
+    a.graph_enable(True)
     twin.graph_enable(False)
 
     def both():
@@ -484,3 +486,28 @@ def test_train_step_nan_logits(engine, oracle):
     x[4, 7] = 0.5
     with pytest.raises(rs.NanError):
         dm.train_step(x, y, 0.01)
+
+
+def test_launch_mode_follows_the_depth(engine, oracle):
+    """By default the step of a shallow model is launched plainly and that of a model with eight Linear
+    layers or more is replayed from a recorded graph; either can be forced; both give the same bits."""
+    import rstorch_amd as rs
+    shallow = rs.DeviceModel(README_MLP)
+    assert not shallow.graph_active()
+    shallow.graph_enable(True)
+    assert shallow.graph_active()
+    shallow.graph_enable("auto")
+    assert not shallow.graph_active()
+    deep_spec = [("linear", 24, 24), ("relu",)] * 7 + [("linear", 24, 5)]
+    weights = make_weights(oracle, deep_spec, 4)
+    deep = rs.DeviceModel(deep_spec); deep.load_parameters(weights)
+    plain = rs.DeviceModel(deep_spec); plain.load_parameters(weights); plain.graph_enable(False)
+    assert deep.graph_active() and not plain.graph_active()
+    deep.profile_enable(True)
+    assert not deep.graph_active()       # per-launch events need plain launches
+    deep.profile_enable(False)
+    for step in range(4):
+        x, y = batch_data(oracle, 48, 24, 5, 41, step % 2, True)
+        assert deep.train_step(x, y, 0.05) == plain.train_step(x, y, 0.05)
+    for (p, _), (q, _) in zip(deep.parameters(), plain.parameters()):
+        np.testing.assert_array_equal(p.to_numpy(), q.to_numpy())

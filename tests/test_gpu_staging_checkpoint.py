@@ -53,7 +53,7 @@ def test_dense_soft_labels_and_slot_exhaustion(engine):
 def test_training_from_staged_inputs_equals_resident_inputs(engine, oracle):
     import rstorch_amd as rs
     weights = make_weights(oracle, README_MLP, 3)
-    a = rs.DeviceModel(README_MLP); a.load_parameters(weights)
+    a = rs.DeviceModel(README_MLP); a.load_parameters(weights); a.graph_enable(True)   # one graph per slot
     b = rs.DeviceModel(README_MLP); b.load_parameters(weights)
     st = rs.BatchStager(32, 784, 10, depth=2)
     batches = []
