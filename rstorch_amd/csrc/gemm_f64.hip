@@ -1325,15 +1325,16 @@ Route choose_route(const GemmParams& p, bool vec, int* dma_slices, bool is_a_kc 
   // slices of at least eight K steps.  The rule below is fitted to a sweep of 386 mid-size shapes
   // (batch 128..16384, widths 64..4096), each timed with this route forced and with it off:
   //   * never below 192 workgroups, and never against several rounds of long 128x128 slices
-  //     (contractions above 1024) - there the 128x128 kernel is 5-20 % ahead;
+  //     (contractions above 2048) - there the 128x128 kernel is ahead;
   //   * always where a dimension of 64 or less leaves the 128-wide tiles half empty (up to 40 %);
   //   * forward products otherwise whenever the slices are either not needed (four K steps are
   //     enough), or at least four, or at least 24 steps long: 5-28 % ahead of the 32x32 tiles and
   //     of one round of 128x128 slices (two slices of 8-16 steps lose 15-50 %); the rule picks
   //     within 0.6 % (geometric mean) of the better of the two routes, 10 % at worst;
-  //   * input gradients only where they replace one round of 128x128 slices: an input gradient
-  //     on 32x32 tiles shares a grid with its layer's weight gradient in Linear::backward, which
-  //     is worth more than the faster kernel.
+  //   * input gradients of at least 2.5e8 flops with a contraction of up to 4096 on slices of 24 steps
+  //     or more (12 unsliced): 5-24 % ahead on rst_linear_backward as a whole; smaller ones stay on the
+  //     32x32 tiles, where they share a grid with their layer's weight gradient, which is worth more
+  //     than the faster kernel.
   if (dma_ok && dma64_mode() != 0 && is_a_kc) {
     const long long t64 = tiles(64, 64);
     const int nk = p.K / BK;
@@ -1349,10 +1350,10 @@ Route choose_route(const GemmParams& p, bool vec, int* dma_slices, bool is_a_kc 
       const bool half_empty = area128 >= 1.4 * area64 && steps >= 12;
       if (is_b_kc) {
         const bool slices_ok = s == 1 ? steps >= 4 : (steps >= 8 && nk >= 32 && (s >= 4 || steps >= 24));
-        take = half_empty || (multi_round ? nk <= 64 : (slices_ok && (s128 <= 1 || nk <= 64)));
+        take = half_empty || (multi_round ? nk <= 128 : (slices_ok && (s128 <= 1 || nk <= 128)));
       } else {
-        const bool beats_one_round = !multi_round && nk <= 64 && (s == 1 ? steps >= 12 : steps >= 24) && s128 > 1;
-        take = flops >= 2.5e8 && (half_empty || beats_one_round);
+        const bool long_enough = nk <= 256 && (s == 1 ? steps >= 12 : steps >= 24);
+        take = flops >= 2.5e8 && (half_empty || long_enough);
       }
     }
     if (take && fits) {
