@@ -391,6 +391,13 @@ def bench_small(rs, eng, spec, batch, normal, steps, warmup, eager, profile_step
         wall_one, _, loss_one, _ = time_steps(eng, dm, x, y, steps, warmup, False)
         out["one_resident_batch"] = {"ms_per_step": wall_one * 1e3 / steps, "steps_per_s": steps / wall_one,
                                      "final_loss": loss_one}
+        # the same with the scalar loss read back after every step, as the reference's loop does
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            loss_each = dm.train_step(x, y, LR, want_loss=True)
+        wall_each = time.perf_counter() - t0
+        out["one_resident_batch"]["with_loss_read_every_step"] = {
+            "ms_per_step": wall_each * 1e3 / steps, "steps_per_s": steps / wall_each, "final_loss": loss_each}
         loader.close()
     else:
         wall, _, loss, _ = time_steps(eng, dm, x, y, steps, warmup, False)
@@ -722,12 +729,17 @@ def main():
             for name, spec, batch, normal, steps, warmup, psteps, fresh in small.values()}
         result["readme_loop"] = readme_loop
         for config, name in (("C0", "C0_readme_b32"), ("C1", "C1_readme_b8192"), ("C2", "C2_wide_b2048")):
-            # (the single-call step on one resident batch: the README loop also walks a small resident pool)
+            # (the single-call step on one resident batch: the README loop also walks a small resident pool;
+            # where measured, beside it the fraction of that step with the loss read every step, which is
+            # what the loop does as well)
             other = result["other_configs"][name]
-            single = other.get("one_resident_batch", other)["steps_per_s"]
+            resident = other.get("one_resident_batch", other)
             loop = readme_loop.get(config, {}).get("compiled", {})
             if "steps_per_s" in loop:
-                loop["fraction_of_single_call_step"] = loop["steps_per_s"] / single
+                loop["fraction_of_single_call_step"] = loop["steps_per_s"] / resident["steps_per_s"]
+                if "with_loss_read_every_step" in resident:
+                    loop["fraction_of_single_call_step_with_loss_read"] = \
+                        loop["steps_per_s"] / resident["with_loss_read_every_step"]["steps_per_s"]
         if "steps_per_s" in readme_loop.get("C4", {}).get("compiled", {}):
             readme_loop["C4"]["compiled"]["fraction_of_single_call_step"] = \
                 readme_loop["C4"]["compiled"]["steps_per_s"] / (args.steps / wall)
