@@ -5,6 +5,7 @@ multi-step criterion (loss within 1e-8 relative) with fresh inputs every step.
 
 The oracle runs on the host cores the GPU box grants (16 threads; its summation order does not
 depend on the thread count): a C2 step takes about half a second, a C4 step about three."""
+import os
 import time
 
 import numpy as np
@@ -75,6 +76,18 @@ def test_one_default_step_matches_oracle_on_every_tensor(engine, oracle, name, s
     dm.close()
 
 
+def _heartbeat(line):
+    """A long comparison prints nothing a test runner would show before it ends; a line appended to a
+    file under gpurun_out/ (where runs on the GPU box keep their output) shows that it is alive."""
+    try:
+        out_dir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+        os.makedirs(out_dir, exist_ok=True)
+        with open(os.path.join(out_dir, "full_size_steps_progress.txt"), "a") as f:
+            f.write(line + "\n")
+    except OSError:
+        pass
+
+
 def _many_steps(engine, oracle, name, spec, batch, max_steps, min_steps, budget_s):
     import rstorch_amd as rs
     dm = rs.DeviceModel(spec)
@@ -92,6 +105,7 @@ def _many_steps(engine, oracle, name, spec, batch, max_steps, min_steps, budget_
             assert err <= 1e-8, "%s step %d: %.17g vs %.17g" % (name, step, got, want)
             worst = max(worst, err)
             done = step + 1
+            _heartbeat("%s: %d steps, %.0f s, worst loss error %.2e" % (name, done, time.time() - t0, worst))
             if done % 10 == 0:
                 print("%s: %d steps, %.0f s, worst loss error %.2e" % (name, done, time.time() - t0, worst),
                       flush=True)
@@ -114,5 +128,5 @@ def test_hundred_steps_at_c2_full_size(engine, oracle):
 
 def test_many_steps_at_c4_full_size(engine, oracle):
     """The same criterion on the deep MLP at batch 1024 for as many of 100 steps as the oracle
-    finishes in under five minutes (a step is 1.6 TFLOP on the host: about 2.5 s on 16 threads), 25 at least."""
-    _many_steps(engine, oracle, "C4", C4_SPEC, 1024, 100, 25, 280.0)
+    finishes in about two minutes (a step is 1.6 TFLOP on the host: about 2.5 s on 16 threads), 25 at least."""
+    _many_steps(engine, oracle, "C4", C4_SPEC, 1024, 100, 25, 110.0)
