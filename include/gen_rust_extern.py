@@ -1,8 +1,8 @@
 #!/usr/bin/env python3
 """Prints the Rust `extern "C"` block that binds every function declared in rstorch_hip.h.
 
-    python include/gen_rust_extern.py            # the block, as it stands in INTEGRATION.md
-    python include/gen_rust_extern.py --check    # exit 1 if INTEGRATION.md's block is out of date
+    python include/gen_rust_extern.py            # the block, as it stands in the integration notes
+    python include/gen_rust_extern.py --check    # exit 1 if the notes' block is out of date
 
 The reference crate is Rust; this image has no Rust toolchain, so the block is generated from the C
 header (the one source of truth for the ABI) instead of being typed by hand, and tests/test_abi.py

@@ -33,8 +33,9 @@ def test_binding_and_header_agree():
 
 
 def test_rust_extern_block_in_the_integration_notes_matches_the_header():
-    """INTEGRATION.md shows the Rust `extern "C"` block a maintainer of the reference would add; it
-    is generated from the header and must declare every entry point, with the current signatures."""
+    """The integration notes at the repository root show the Rust `extern "C"` block a maintainer of
+    the reference would add; it is generated from the header and must declare every entry point, with
+    the current signatures."""
     gen = os.path.join(ROOT, "include", "gen_rust_extern.py")
     block = subprocess.run([sys.executable, gen], capture_output=True, text=True, check=True).stdout
     assert sorted(re.findall(r"pub fn (rst_[a-z0-9_]+)", block)) == declared_functions()

@@ -78,7 +78,7 @@ def test_one_default_step_matches_oracle_on_every_tensor(engine, oracle, name, s
 
 def _heartbeat(line):
     """A long comparison prints nothing a test runner would show before it ends; a line appended to a
-    file under gpurun_out/ (where runs on the GPU box keep their output) shows that it is alive."""
+    file in the run-output directory beside the tests shows that it is alive."""
     try:
         out_dir = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
         os.makedirs(out_dir, exist_ok=True)
