@@ -774,7 +774,9 @@ __global__ __launch_bounds__(BLOCK, 2) void head_ce_kernel(HeadParams p) {
   }
 
   if (t == 0) {
-    asm volatile("" : "+v"(old));  // the addition below waits for the exchange, whatever its value
+    // the addition below is issued only when the exchange has returned: its result is an input of this
+    // (empty) statement, which no memory access may cross
+    asm volatile("" : "+v"(old) : : "memory");
     const unsigned long long inc = 1ull + ((unsigned long long)nan_here << 32) + (old & 0ull);
     const unsigned long long seen = atomicAdd(p.arrivals, inc) + inc;
     last_nan = (int)((seen >> 32) != 0);
