@@ -424,9 +424,10 @@ __global__ __launch_bounds__(1024) void loss_reduce_kernel(const double* __restr
 //
 // HID: the Linear in front of the head (at most 112 inputs and outputs) runs in the same launch, so
 // that two more launches - its forward and its input gradient - disappear.  Its weights sit in LDS
-// as well; a workgroup (256 threads) takes 16 rows at a time - one MFMA fragment - and walks over
+// as well; a workgroup (512 threads) takes 16 rows at a time - one MFMA fragment - and walks over
 // the batch with a stride of the grid (the weights are fetched once per workgroup): hidden forward
-// on the matrix cores, the head as above on the result, hidden input gradient on the matrix cores.
+// on the matrix cores (wavefront w computes output fragment w), the head as above on the result (the
+// first four wavefronts), hidden input gradient on the matrix cores.
 struct HeadParams {
   const double* h;      // [rows, K] inputs of the Linear (contiguous rows)
   const double* w;      // [N, K]
@@ -454,15 +455,6 @@ struct HeadParams {
 
 typedef double v4d_t __attribute__((ext_vector_type(4)));
 
-// One 16 x 16 MFMA product chain out of LDS: c += sum over steps s of A[.][4 s + lk] x B[4 s + lk][.],
-// a (resp. b) pointing at this lane's element of step 0 and moving by a_step (b_step) doubles per
-// step; `steps` is a multiple of four.  The reads are inline assembly, so that their place in the
-// instruction stream is fixed and the waits can name how many younger reads may still be
-// outstanding: the operands of four steps are in registers or on their way at any time, in two sets
-// of two steps, and a set's four reads go out as soon as the MFMAs that used its registers have been
-// issued.  Each of the four steps of a round adds up in an accumulator of its own (an MFMA that
-// continues the sum of the one issued just before it would wait for its result); they are added
-// together at the end.  After the last step the requests fetch the last operands again; nobody uses them.
 __device__ __forceinline__ void lds_barrier() {
   // A workgroup barrier for data exchanged through LDS: this wavefront's LDS accesses are over, then
   // everybody meets.  Unlike __syncthreads() it does not wait for the stores to global memory that
@@ -474,6 +466,15 @@ __device__ __forceinline__ double lds_read_f64(uint32_t byte_address) {
   asm volatile("ds_read_b64 %0, %1" : "=v"(v) : "v"(byte_address) : "memory");
   return v;
 }
+// One 16 x 16 MFMA product chain out of LDS: c += sum over steps s of A[.][4 s + lk] x B[4 s + lk][.],
+// a (resp. b) pointing at this lane's element of step 0 and moving by a_step (b_step) doubles per
+// step; `steps` is a multiple of four.  The reads are inline assembly, so that their place in the
+// instruction stream is fixed and the waits can name how many younger reads may still be
+// outstanding: the operands of four steps are in registers or on their way at any time, in two sets
+// of two steps, and a set's four reads go out as soon as the MFMAs that used its registers have been
+// issued.  Each of the four steps of a round adds up in an accumulator of its own (an MFMA that
+// continues the sum of the one issued just before it would wait for its result); they are added
+// together at the end.  After the last step the requests fetch the last operands again; nobody uses them.
 __device__ __forceinline__ v4d_t mfma_chain(const double* a, int a_step, const double* b, int b_step, int steps) {
   uint32_t pa = (uint32_t)(uintptr_t)a, pb = (uint32_t)(uintptr_t)b;
   const uint32_t da = 8u * (uint32_t)a_step, db = 8u * (uint32_t)b_step;
