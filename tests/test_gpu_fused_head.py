@@ -111,3 +111,30 @@ def test_nan_logits_are_reported(engine, oracle):
     assert np.isfinite(fresh.train_step(x, y, 0.01))
     with pytest.raises(rs.NanError):
         fresh.train_step(bad, y, 0.0)
+
+
+def test_many_workgroups_and_many_launches(engine, oracle):
+    """The loss hand-over at scale: a head alone on 40 000 rows (1250 workgroups of 32 rows, 18 inputs per
+    lane) against the oracle, and 300 steps of the README network at batch 8192 on two models from the
+    same state - every loss of the run the same bits on both (the arrival word is re-armed by each
+    launch, whichever workgroup came last)."""
+    import rstorch_amd as rs
+    spec = [("linear", 64, 200), ("relu",), ("linear", 200, 10)]     # 200 inputs: too wide for the hidden variant
+    dm, ref = pair(rs, oracle, spec, 12)
+    oracle.set_threads(8)
+    try:
+        x, y = batch_data(oracle, 40000, 64, 10, 43, 0, True)
+        got, want = dm.train_step(x, y, 0.05), ref.train_step(x, y, 0.05)
+        assert abs(got - want) <= TOL * abs(want)
+        for (p, g), (rp, rg) in zip(dm.parameters(), ref.parameters()):
+            assert rel_err(g.to_numpy(), rg) <= TOL and rel_err(p.to_numpy(), rp) <= TOL
+    finally:
+        oracle.set_threads(1)
+    a, _ = pair(rs, oracle, README_MLP, 13)
+    b, _ = pair(rs, oracle, README_MLP, 13)
+    x, y = batch_data(oracle, 8192, 784, 10, 47, 0)
+    dx, dy = engine.from_numpy(x), engine.from_numpy(y)
+    la = [a.train_step(dx, dy, 0.01) for _ in range(300)]
+    lb = [b.train_step(dx, dy, 0.01) for _ in range(300)]
+    assert la == lb
+    assert la[-1] < la[0]
