@@ -48,7 +48,7 @@ PEAK_HBM_GBPS = 8000.0
 # the profile is collected again and the digest updated.
 C4_TRAFFIC_SOURCE = {"profile": "profiles/c4_hbm_traffic.md",
                      "kernel_sources": ["rstorch_amd/csrc/gemm_f64.hip", "rstorch_amd/csrc/gemm_addressing.h"],
-                     "kernel_sources_sha16": "03214f75fb84be34"}
+                     "kernel_sources_sha16": "ad1c4f94c1ed70bf"}
 
 
 def kernel_sources_digest():
@@ -61,12 +61,12 @@ def kernel_sources_digest():
 
 
 C4_TRAFFIC_BYTES_PER_LAUNCH = {
-    "linear_forward": (8 * 436.5e6 + 3877.7e6) / 9,
-    "grad_weight": (8 * 868.3e6 + 7995.7e6) / 9,
-    "grad_input": (7 * 470.0e6 + 3335.1e6 + 134.3e6) / 8,
+    "linear_forward": (8 * 436.4e6 + 3747.9e6) / 9,
+    "grad_weight": (8 * 860.6e6 + 7385.4e6) / 9,
+    "grad_input": (7 * 470.0e6 + 3357.2e6 + 134.3e6) / 8,
     # a layer's weight gradient + SGD and the next layer's input gradient in one grid (the default):
     # six pairs at the hidden width and the one that carries the head's weight gradient
-    "grad_pair": (6 * 1533.1e6 + 8614.3e6) / 7,
+    "grad_pair": (6 * 1501.4e6 + 7758.2e6) / 7,
 }
 
 C4_SPEC = [("linear", 4096, 4096), ("relu",)] * 8 + [("linear", 4096, 32768)]

@@ -55,6 +55,14 @@ struct GemmParams {
   // the first round that sit in the upper wave slots of their CU start this many 10 ns ticks late
   int dephase_ticks;
   int first_round;       // workgroups that fit on the chip at once
+  // Direct-to-LDS kernels on operands that do not promise 16-byte aligned pairs (an odd leading
+  // dimension or extent, a base address that is only 8-byte aligned).  The tile DMA itself takes
+  // 8-byte aligned addresses; what changes is the masked K tail (single loads) and, when an
+  // output-contiguous operand has an odd extent, which K rows travel by DMA: the pair that holds
+  // the operand's last column also fetches the double behind it, which for the operand's very last
+  // K row would lie behind the operand, so that row is kept back for the tail (k_reserve = 1).
+  int unaligned;         // 1 = the K tail is fetched by single loads
+  int k_reserve;         // K rows (0 or 1) kept out of the whole steps that travel by DMA
 };
 
 // Up to kMaxGroup products in one grid: workgroups [first_block[i], first_block[i+1]) belong to
@@ -115,18 +123,20 @@ RST_HD StagedSteps staged_k_steps(int K, int split_k, int steps_per_split, int s
   return s;
 }
 // Direct-to-LDS kernels: whole steps [kt0, kt0 + nk_dma) travel by tile DMA; what is left of K
-// beyond its last whole step (K % BK indices starting at (K / BK) * BK) is an extra first tile of
-// slice 0, copied by masked register loads.
+// beyond the last of them (1 to BK indices starting at dma_whole_steps * BK) is an extra first tile
+// of slice 0, copied by masked register loads.  k_reserve (0 or 1) rows at the end of K never
+// travel by DMA (GemmParams::k_reserve).
+RST_HD int dma_whole_steps(int K, int k_reserve) { return (K - k_reserve) / BK; }
 struct DmaSteps {
   int kt0, nk_dma;
   bool k_tail;
 };
-RST_HD DmaSteps dma_k_steps(int K, int split_k, int steps_per_split, int split) {
+RST_HD DmaSteps dma_k_steps(int K, int split_k, int steps_per_split, int split, int k_reserve) {
   DmaSteps s;
-  const int nk_all = K / BK;
+  const int nk_all = dma_whole_steps(K, k_reserve);
   s.kt0 = split * steps_per_split;
   s.nk_dma = (split_k > 1) ? ((nk_all - s.kt0 < steps_per_split) ? nk_all - s.kt0 : steps_per_split) : nk_all;
-  s.k_tail = (K % BK) != 0 && split == 0;
+  s.k_tail = K > nk_all * BK && split == 0;
   return s;
 }
 
@@ -147,10 +157,15 @@ RST_HD T dma_offset_kc(int chunk, int lane, int o0, int ext, long ld) {
   return (T)8 * (T)((size_t)rr * (size_t)ld + (size_t)(2 * ((lane & 7) ^ (row & 7))));
 }
 // Output-contiguous operand of the 128-wide tiles, chunk = one k row of 128 doubles: lane l fetches
-// columns 2l, 2l+1; a pair that would cross the extent is moved back onto the last whole pair.
+// columns 2l, 2l+1; a pair that begins beyond the extent is moved back onto the last two columns.
+// With an odd extent the pair that begins on the last column stays where it is and also fetches the
+// double behind the row's end (the next row's first one, or padding): it feeds an output that is
+// never stored, and GemmParams::k_reserve keeps the one row where it would leave the operand away
+// from the DMA.
 template <typename T>
 RST_HD T dma_offset_oc128(int chunk, int lane, int o0, int ext, long ld) {
-  const int ge = o0 + 2 * lane + 1 < ext ? 2 * lane : ext - 2 - o0;
+  const int back = ext - 2 - o0 > 0 ? ext - 2 - o0 : 0;  // (0: a tile that holds the one last column of an odd extent)
+  const int ge = o0 + 2 * lane < ext ? 2 * lane : back;
   return (T)8 * (T)((size_t)chunk * (size_t)ld + (size_t)(long)ge);
 }
 // Output-contiguous operand of the 64-wide tiles, chunk = two k rows of 64 doubles (k rows 2*chunk
@@ -160,7 +175,8 @@ template <typename T>
 RST_HD T dma_offset_oc64(int chunk, int lane, int o0, int ext, long ld) {
   const int kr = 2 * chunk + (lane >> 5);
   const int e = 2 * ((lane & 31) ^ (8 * (chunk & 3)));
-  const int ge = o0 + e + 1 < ext ? e : ext - 2 - o0;
+  const int back = ext - 2 - o0 > 0 ? ext - 2 - o0 : 0;
+  const int ge = o0 + e < ext ? e : back;  // as for the 128-wide tiles
   return (T)8 * (T)((size_t)kr * (size_t)ld + (size_t)(long)ge);
 }
 // bytes from one K step of a tile to the next

@@ -13,7 +13,8 @@
 //                      shape and alignment, optional split-K for small outputs;
 //   gemm_f64_mfma_dma  128x128 tiles, eight wavefronts of 64x32, operand tiles moved global -> LDS
 //                      by global_load_lds_dwordx4 and a hand-scheduled inner loop: the path of
-//                      the large aligned products (K a multiple of 16, at least 256 tiles).
+//                      the large products (at least 256 tiles, or fewer on K slices), whatever
+//                      their alignment.
 // K advances in steps of 16 through two LDS stages; the loads of step k+1 are in flight while
 // step k is multiplied.
 //
@@ -502,8 +503,11 @@ __global__ __launch_bounds__(256, (BURST > 0 ? 1 : 2)) void gemm_f64_mfma_mixed_
 }
 
 // ---- 128x128 tiles fed by direct global -> LDS loads ------------------------------------------
-// The main path for large problems with 16-byte aligned operands (even leading dimensions and
-// extents; K need not be a multiple of 16: its remainder is a masked extra tile).
+// The main path for large problems.  K need not be a multiple of 16: its remainder is a masked
+// extra tile.  The operands need no more than their 8-byte alignment: global_load_lds_dwordx4 takes
+// a global address that is only 8-byte aligned at its full rate (measured), so odd leading
+// dimensions and extents travel the same way; for those the K tail is fetched by single loads and
+// GemmParams::k_reserve keeps the operand's last K row for it when a pair could reach behind it.
 // global_load_lds_dwordx4 moves 16 bytes per lane straight into LDS (lane l lands at
 // base + 16*l), so no staging registers and no ds_write instructions are spent on the operand
 // tiles; a wavefront moves one 1 KiB chunk of a tile per instruction:
@@ -642,8 +646,8 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
   // K steps of this workgroup: all whole ones, or slice `split` of a split contraction.  What is
   // left of K beyond its last whole step (K % 16 indices) is an extra first tile of slice 0, copied
   // into stage 0 by ordinary masked loads; the whole steps follow through the DMA pipeline.
-  const DmaSteps ks = dma_k_steps(p.K, p.split_k, p.steps_per_split, split);
-  const int nk_all = p.K / BK;
+  const DmaSteps ks = dma_k_steps(p.K, p.split_k, p.steps_per_split, split, p.k_reserve);
+  const int nk_all = dma_whole_steps(p.K, p.k_reserve);
   const int kt0 = ks.kt0, nk_dma = ks.nk_dma;
   const bool k_tail = ks.k_tail;
   const int nk = nk_dma + (k_tail ? 1 : 0);
@@ -680,8 +684,13 @@ __device__ __forceinline__ void dma_tile(const GemmParams& p, int block, double*
   static_assert(DIST >= 1 && DIST < STAGES && (DIST - 1) * 2 * CH <= 4, "ring of STAGES stages, DIST tiles ahead");
   if (k_tail) {
     v2d ra[(BM * BK / 2) / (NW * 64)], rb[(BN * BK / 2) / (NW * 64)];
-    load_tile<BM, A_KC, true, true, NW * 64>(ra, p.A, p.lda, m0, p.M, nk_all * BK, p.K, tid);
-    load_tile<BN, B_KC, true, true, NW * 64>(rb, p.B, p.ldb, n0, p.N, nk_all * BK, p.K, tid);
+    if (p.unaligned) {  // (uniform over the launch)
+      load_tile<BM, A_KC, false, true, NW * 64>(ra, p.A, p.lda, m0, p.M, nk_all * BK, p.K, tid);
+      load_tile<BN, B_KC, false, true, NW * 64>(rb, p.B, p.ldb, n0, p.N, nk_all * BK, p.K, tid);
+    } else {
+      load_tile<BM, A_KC, true, true, NW * 64>(ra, p.A, p.lda, m0, p.M, nk_all * BK, p.K, tid);
+      load_tile<BN, B_KC, true, true, NW * 64>(rb, p.B, p.ldb, n0, p.N, nk_all * BK, p.K, tid);
+    }
     store_tile_dma<BM, A_KC, NW * 64>(lds_a, ra, tid);
     store_tile_dma<BN, B_KC, NW * 64>(lds_b, rb, tid);
   } else if (nk > 0) {
@@ -915,8 +924,8 @@ __global__ __launch_bounds__(256, 2) void gemm_f64_mfma_dma64(const GemmParams p
     for (int j = 0; j < TN; ++j) acc[i][j] = (v4d){0.0, 0.0, 0.0, 0.0};
 
   // tiles of this workgroup: [the masked remainder of K (slice 0 only)] + the whole steps of its slice
-  const DmaSteps ks = dma_k_steps(p.K, p.split_k, p.steps_per_split, split);
-  const int nk_all = p.K / BK;
+  const DmaSteps ks = dma_k_steps(p.K, p.split_k, p.steps_per_split, split, p.k_reserve);
+  const int nk_all = dma_whole_steps(p.K, p.k_reserve);
   const int kt0 = ks.kt0, nk_dma = ks.nk_dma;
   const bool k_tail = ks.k_tail;
   const int first_dma = k_tail ? 1 : 0;
@@ -945,8 +954,13 @@ __global__ __launch_bounds__(256, 2) void gemm_f64_mfma_dma64(const GemmParams p
     if (t >= first_dma && t < nk) issue(t);
   if (k_tail) {
     v2d ra[2], rb[2];
-    load_tile<BM, A_KC, true, true, 256>(ra, p.A, p.lda, m0, p.M, nk_all * BK, p.K, tid);
-    load_tile<BN, B_KC, true, true, 256>(rb, p.B, p.ldb, n0, p.N, nk_all * BK, p.K, tid);
+    if (p.unaligned) {  // (uniform over the launch)
+      load_tile<BM, A_KC, false, true, 256>(ra, p.A, p.lda, m0, p.M, nk_all * BK, p.K, tid);
+      load_tile<BN, B_KC, false, true, 256>(rb, p.B, p.ldb, n0, p.N, nk_all * BK, p.K, tid);
+    } else {
+      load_tile<BM, A_KC, true, true, 256>(ra, p.A, p.lda, m0, p.M, nk_all * BK, p.K, tid);
+      load_tile<BN, B_KC, true, true, 256>(rb, p.B, p.ldb, n0, p.N, nk_all * BK, p.K, tid);
+    }
     store_tile_dma64<A_KC>(lds_a, ra, tid);
     store_tile_dma64<B_KC>(lds_b, rb, tid);
   }
@@ -1158,7 +1172,7 @@ int launch_dma(hipStream_t stream, GemmParams p, int want_split = 0) {
   p.tiles_m = (p.M + 127) / 128;
   p.tiles_n = (p.N + 127) / 128;
   p.split_k = 1;
-  p.steps_per_split = p.K / BK;
+  p.steps_per_split = dma_whole_steps(p.K, p.k_reserve);
   long long blocks = (long long)p.tiles_m * p.tiles_n;
   // Two independent workgroups per compute unit interleave their barriers and LDS waits: measured
   // on 256 tiles, the K loop runs about 1.5 points of the MFMA peak faster with two than with one.
@@ -1166,7 +1180,7 @@ int launch_dma(hipStream_t stream, GemmParams p, int want_split = 0) {
   // the two partial products are then added (in slice order) by split_reduce_kernel, a fixed cost
   // of about 30 us per launch at 1024 x 4096 outputs: level at K = 16384 (1838 us unsplit, 1847
   // split), 0.5 % ahead at K = 32768.
-  const int nk = p.K / BK;
+  const int nk = dma_whole_steps(p.K, p.k_reserve);
   const size_t need = 2 * ((size_t)p.M * p.N + (size_t)p.M);
   if (want_split > 1) {
     p.steps_per_split = (nk + want_split - 1) / want_split;
@@ -1183,7 +1197,7 @@ int launch_dma(hipStream_t stream, GemmParams p, int want_split = 0) {
   // more than one round of workgroups (two per CU fit): stagger the first round by 0.4 us per K step
   p.first_round = 2 * compute_units();
   p.dephase_ticks = blocks > p.first_round ? (p.steps_per_split < 250 ? 40 * p.steps_per_split : 10000) : 0;
-  RST_OBSERVE_GEMM(GemmKernel::kDma128, 128, 128, 2, 4, A_KC, B_KC, true, 0, blocks, 512, &p, nullptr, 0, nullptr);
+  RST_OBSERVE_GEMM(GemmKernel::kDma128, 128, 128, 2, 4, A_KC, B_KC, p.unaligned == 0, 0, blocks, 512, &p, nullptr, 0, nullptr);
   hipLaunchKernelGGL((gemm_f64_mfma_dma<A_KC, B_KC, 2, 4, 2, 1>), dim3((unsigned)blocks),
                      dim3(512), 0, stream, p);
   RST_HIP(hipGetLastError());
@@ -1196,7 +1210,7 @@ template <bool B_KC>
 int launch_dma64(hipStream_t stream, GemmParams p, int slices) {
   p.tiles_m = (p.M + kT64 - 1) / kT64;
   p.tiles_n = (p.N + kT64 - 1) / kT64;
-  const int nk = p.K / BK;
+  const int nk = dma_whole_steps(p.K, p.k_reserve);
   p.split_k = 1;
   p.steps_per_split = nk;
   long long blocks = (long long)p.tiles_m * p.tiles_n;
@@ -1209,7 +1223,7 @@ int launch_dma64(hipStream_t stream, GemmParams p, int slices) {
     }
   }
   if (blocks > 0x7fffffffLL) return fail(RST_ERR_UNSUPPORTED, "contraction grid too large");
-  RST_OBSERVE_GEMM(GemmKernel::kDma64, 64, 64, 2, 2, true, B_KC, true, 0, blocks, 256, &p, nullptr, 0, nullptr);
+  RST_OBSERVE_GEMM(GemmKernel::kDma64, 64, 64, 2, 2, true, B_KC, p.unaligned == 0, 0, blocks, 256, &p, nullptr, 0, nullptr);
   hipLaunchKernelGGL((gemm_f64_mfma_dma64<B_KC>), dim3((unsigned)blocks), dim3(256), 0, stream, p);
   RST_HIP(hipGetLastError());
   if (p.split_k > 1) RST_TRY(launch_split_reduce(stream, p));
@@ -1288,12 +1302,13 @@ int dma64_mode() {
   return mode;
 }
 
-Route choose_route(const GemmParams& p, bool vec, int* dma_slices, bool is_a_kc = false, bool is_b_kc = false) {
+Route choose_route(const GemmParams& p, int* dma_slices, bool is_a_kc = false, bool is_b_kc = false) {
   auto tiles = [&](int bm, int bn) {
     return (long long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
   };
-  // (leading dimensions below 2^22 doubles keep the 32-bit lane offsets of the tile DMA in range)
-  const bool dma_ok = vec && p.K > 0 && p.M >= 2 && p.N >= 2 && p.lda < (1L << 22) && p.ldb < (1L << 22);
+  // (leading dimensions below 2^22 doubles keep the 32-bit lane offsets of the tile DMA in range;
+  // the tile DMA needs no more than the 8-byte alignment every operand has)
+  const bool dma_ok = p.K > 0 && p.M >= 2 && p.N >= 2 && p.lda < (1L << 22) && p.ldb < (1L << 22);
   const long long t128 = tiles(128, 128);
   *dma_slices = 0;
   if (t128 >= 256) return dma_ok ? Route::kDma : Route::kTile128;
@@ -1304,7 +1319,7 @@ Route choose_route(const GemmParams& p, bool vec, int* dma_slices, bool is_a_kc 
   int s128 = 0;       // its slices, 0 = not taken
   bool multi_round = false;
   if (dma_ok && p.ws != nullptr) {
-    const int nk = p.K / BK;
+    const int nk = dma_whole_steps(p.K, p.k_reserve);
     auto fits = [&](int s) { return p.ws_capacity >= (size_t)s * ((size_t)p.M * p.N + (size_t)p.M); };
     int s = (int)((512 + t128 - 1) / t128);
     if (s > 8) s = 8;
@@ -1337,7 +1352,7 @@ Route choose_route(const GemmParams& p, bool vec, int* dma_slices, bool is_a_kc 
   //     than the faster kernel.
   if (dma_ok && dma64_mode() != 0 && is_a_kc) {
     const long long t64 = tiles(64, 64);
-    const int nk = p.K / BK;
+    const int nk = dma_whole_steps(p.K, p.k_reserve);
     long long s = t64 >= 256 ? 1 : (256 + t64 - 1) / t64;
     if (s > 32) s = 32;
     while (s > 1 && nk / s < 8) --s;
@@ -1372,7 +1387,7 @@ Route choose_route(const GemmParams& p, bool vec, int* dma_slices, bool is_a_kc 
 template <bool A_KC, bool B_KC, bool VEC>
 int launch_layout(hipStream_t stream, const GemmParams& p) {
   int slices = 0;
-  switch (choose_route(p, VEC, &slices, A_KC, B_KC)) {
+  switch (choose_route(p, &slices, A_KC, B_KC)) {
     case Route::kDma: return launch_dma<A_KC, B_KC>(stream, p);
     case Route::kDmaSliced: return launch_dma<A_KC, B_KC>(stream, p, slices);
     case Route::kDma64:
@@ -1387,7 +1402,8 @@ int launch_layout(hipStream_t stream, const GemmParams& p) {
 
 namespace {
 
-// 16-byte loads need both operands aligned with even leading dimensions and extents
+// 16-byte register loads (and the shared-grid kernels) need both operands aligned with even
+// leading dimensions and extents
 bool desc_vec_ok(const GemmDesc& d) {
   auto ok = [](const double* ptr, long ld, int contiguous_extent) {
     return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && (ld % 2 == 0) &&
@@ -1419,6 +1435,8 @@ GemmParams make_params(const GemmDesc& d) {
   p.ws = d.workspace; p.ws_colsum = nullptr; p.ws_capacity = d.workspace ? d.workspace_count : 0;
   p.tiles_m = p.tiles_n = 0;
   p.dephase_ticks = 0; p.first_round = 0;
+  p.unaligned = desc_vec_ok(d) ? 0 : 1;
+  p.k_reserve = ((!d.a_kc && d.M % 2 != 0) || (!d.b_kc && d.N % 2 != 0)) ? 1 : 0;
   return p;
 }
 
@@ -1462,7 +1480,7 @@ bool can_group_gemm(const GemmDesc& d) {
   if (d.M <= 0 || d.N <= 0 || !desc_vec_ok(d)) return false;
   const GemmParams p = make_params(d);
   int slices = 0;
-  return choose_route(p, true, &slices, d.a_kc, d.b_kc) == Route::kTile32;
+  return choose_route(p, &slices, d.a_kc, d.b_kc) == Route::kTile32;
 }
 
 namespace {
@@ -1577,7 +1595,7 @@ bool plan_dma_group(const GemmDesc* d, int count, GemmGroup* g, long long* block
     GemmParams p = make_params(piece[i]);
     p.tiles_m = (p.M + 127) / 128;
     p.tiles_n = (p.N + 127) / 128;
-    const int nk = p.K / BK;
+    const int nk = dma_whole_steps(p.K, p.k_reserve);
     long long s = (long long)(full_slices * (double)cost[i] / (double)cost_max + 0.5);
     if (s > kDmaGroupMaxSlices) s = kDmaGroupMaxSlices;
     if (s > nk / kDmaGroupMinSteps) s = nk / kDmaGroupMinSteps;
@@ -1703,8 +1721,8 @@ int launch_gemm_pair(hipStream_t stream, const GemmDesc& input_grad, const GemmD
   if (!can_pair_gemm(input_grad, weight_grad))
     return fail(RST_ERR_INVALID_ARGUMENT, "these two contractions cannot share a grid");
   GemmParams p1 = make_params(input_grad), p2 = make_params(weight_grad);
-  p1.tiles_m = (p1.M + 127) / 128; p1.tiles_n = (p1.N + 127) / 128; p1.steps_per_split = p1.K / BK;
-  p2.tiles_m = (p2.M + 127) / 128; p2.tiles_n = (p2.N + 127) / 128; p2.steps_per_split = p2.K / BK;
+  p1.tiles_m = (p1.M + 127) / 128; p1.tiles_n = (p1.N + 127) / 128; p1.steps_per_split = dma_whole_steps(p1.K, p1.k_reserve);
+  p2.tiles_m = (p2.M + 127) / 128; p2.tiles_n = (p2.N + 127) / 128; p2.steps_per_split = dma_whole_steps(p2.K, p2.k_reserve);
   const long long b1 = (long long)p1.tiles_m * p1.tiles_n, b2 = (long long)p2.tiles_m * p2.tiles_n;
   RST_OBSERVE_GEMM(GemmKernel::kDma128Pair, 128, 128, 2, 4, true, false, true, 0, b1 + b2, 512, &p1, &p2, (int)b1, nullptr);
   hipLaunchKernelGGL((gemm_f64_mfma_dma_pair<true, false, false, false>), dim3((unsigned)(b1 + b2)), dim3(512),

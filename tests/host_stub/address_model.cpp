@@ -5,7 +5,9 @@
 // and lane of the grid through the SAME index functions the kernels run on the device
 // (rstorch_amd/csrc/gemm_addressing.h) and checks, before anything could reach a GPU:
 //   * every global read lies inside the logical footprint of its operand ((rows-1)*ld + cols doubles)
-//     and every 16-byte access is 16-byte aligned; the 32-bit lane offsets equal their 64-bit values;
+//     and every 16-byte register load is 16-byte aligned (the tile DMA needs 8 bytes only: launches
+//     that promise aligned operands are held to 16, the others to 8 and to never displacing an
+//     element that exists); the 32-bit lane offsets equal their 64-bit values;
 //   * every tile-DMA lane lands inside its LDS stage, every fragment read stays inside the stage, and
 //     the slot a fragment read takes for (row, pair) is the slot the DMA put that (row, pair) in;
 //   * the workgroups of a grid map one-to-one onto (K slice, output tile), the K slices of a tile
@@ -32,6 +34,8 @@ namespace {
 long g_checked[16] = {};       // launches verified, per GemmKernel
 long g_staged_by_tile[2] = {}; // register-staged launches verified: 32x32, 128x128 tiles
 long g_sliced[16] = {};        // of g_checked: launches on K slices
+long g_unaligned[16] = {};     // of g_checked: tile-DMA launches on operands without 16-byte aligned pairs
+long g_reserved[16] = {};      // of g_unaligned: launches that keep the last K row back for the tail
 long g_skipped_repeats = 0;    // launches seen before (same kernel, same parameters)
 long long g_lane_checks = 0;   // individual address checks
 std::set<std::string> g_seen;
@@ -136,10 +140,11 @@ void check_params(const GemmParams& p, bool a_kc, bool b_kc) {
 
 // the slices of a contraction cover its K steps exactly once (DMA kernels: whole steps by DMA + the tail)
 void check_dma_k_cover(const GemmParams& p) {
-  const int nk_all = p.K / BK;
+  if (p.k_reserve != 0 && p.k_reserve != 1) bad("k_reserve = %d", p.k_reserve);
+  const int nk_all = dma_whole_steps(p.K, p.k_reserve);
   int next = 0, tails = 0;
   for (int s = 0; s < p.split_k; ++s) {
-    const DmaSteps ks = dma_k_steps(p.K, p.split_k, p.steps_per_split, s);
+    const DmaSteps ks = dma_k_steps(p.K, p.split_k, p.steps_per_split, s, p.k_reserve);
     if (ks.nk_dma < 0) bad("slice %d has %d K steps", s, ks.nk_dma);
     if (ks.nk_dma > 0 && ks.kt0 != next) bad("slice %d starts at step %d, expected %d", s, ks.kt0, next);
     if (ks.nk_dma > 0) next = ks.kt0 + ks.nk_dma;
@@ -147,7 +152,8 @@ void check_dma_k_cover(const GemmParams& p) {
     tails += ks.k_tail ? 1 : 0;
   }
   if (next != nk_all) bad("the slices cover %d of %d whole K steps", next, nk_all);
-  if (tails != (p.K % BK != 0 ? 1 : 0)) bad("the K remainder is multiplied %d times", tails);
+  if (p.K - nk_all * BK < 0 || p.K - nk_all * BK > BK) bad("a K remainder of %d indices", p.K - nk_all * BK);
+  if (tails != (p.K > nk_all * BK ? 1 : 0)) bad("the K remainder is multiplied %d times", tails);
 }
 void check_staged_k_cover(const GemmParams& p) {
   const int nk_all = (p.K + BK - 1) / BK;
@@ -234,7 +240,7 @@ enum class OcKind { k128, k64 };
 
 // one operand tile of a DMA kernel: every lane of every chunk, first and last K step
 void check_dma_operand(const char* name, const double* base, bool kc, OcKind oc, int ext_tile, int chunks, int o0,
-                       int ext, int K, long ld, int kt0, int nk_dma) {
+                       int ext, int K, long ld, int kt0, int nk_dma, bool aligned) {
   const size_t limit = footprint(kc, ext, K, ld);
   const size_t origin = kc ? (size_t)o0 * (size_t)ld : (size_t)o0;
   const size_t step = (size_t)dma_k_step_bytes(kc, ld) / 8;
@@ -260,15 +266,30 @@ void check_dma_operand(const char* name, const double* base, bool kc, OcKind oc,
         lds = dma_lds_chunk_oc64(c);
       }
       if (o32 != o64) bad("%s DMA lane offset wraps 32 bits: %u vs %" PRIu64, name, o32, o64);
-      if (o64 % 16 != 0) bad("%s DMA lane offset %" PRIu64 " is not a multiple of 16", name, o64);
+      if (o64 % (aligned ? 16 : 8) != 0) bad("%s DMA lane offset %" PRIu64 " is not a multiple of %d", name, o64, aligned ? 16 : 8);
+      {
+        // an element that exists is fetched from its own place: the clamps only move pairs that lie
+        // wholly beyond the extent (rows of a contraction-contiguous tile, columns of the other kind)
+        const uint64_t d = o64 / 8;
+        if (kc) {
+          const int row = 8 * c + (lane >> 3), k = 2 * ((lane & 7) ^ (row & 7));
+          if (o0 + row < ext && d != (uint64_t)row * (uint64_t)ld + (uint64_t)k) bad("%s DMA: row %d pair %d displaced", name, row, k);
+        } else {
+          const int krow = oc == OcKind::k128 ? c : 2 * c + (lane >> 5);
+          const int e = oc == OcKind::k128 ? 2 * lane : 2 * ((lane & 31) ^ (8 * (c & 3)));
+          if (o0 + e < ext && d != (uint64_t)krow * (uint64_t)ld + (uint64_t)e) bad("%s DMA: k row %d column %d displaced", name, krow, e);
+        }
+      }
       if (lds < 0 || lds + 2 * lane + 2 > stage) bad("%s DMA chunk %d lane %d lands outside its LDS stage", name, c, lane);
       if (nk_dma > 0) {
         const size_t first = origin + (size_t)kt0 * step + o64 / 8;
         const size_t last = origin + (size_t)(kt0 + nk_dma - 1) * step + o64 / 8;
         in_range(name, first, 2, limit);
         in_range(name, last, 2, limit);
-        aligned16(name, base, 8 * first);
-        aligned16(name, base, 8 * last);
+        if (aligned) {
+          aligned16(name, base, 8 * first);
+          aligned16(name, base, 8 * last);
+        }
       }
     }
 }
@@ -309,14 +330,30 @@ void check_lds_layout(bool kc, OcKind oc, int ext_tile, int chunks) {
 }
 
 template <int EXT, bool KC>
-void check_tail_tile(const char* name, const double* base, int threads, long ld, int o0, int ext, int K) {
-  // the masked remainder tile: load_tile<EXT, KC, VEC = true, TAIL = true>
+void check_tail_tile(const char* name, const double* base, int threads, long ld, int o0, int ext, int K, int k_reserve,
+                     bool aligned) {
+  // the masked remainder tile: load_tile<EXT, KC, VEC = aligned, TAIL = true>
   const size_t limit = footprint(KC, ext, K, ld);
-  const int k0 = (K / BK) * BK;
+  const int k0 = dma_whole_steps(K, k_reserve) * BK;
   const int pairs = EXT * BK / 2;
   if (pairs % threads != 0) bad("%s: %d pairs do not split over %d threads", name, pairs, threads);
   for (int q = 0; q < pairs; ++q) {
-    const PairSource s = staged_pair_source<EXT, KC, true, true>(q, ld, o0, ext, k0, K);
+    const PairSource s = aligned ? staged_pair_source<EXT, KC, true, true>(q, ld, o0, ext, k0, K)
+                                 : staged_pair_source<EXT, KC, false, true>(q, ld, o0, ext, k0, K);
+    {
+      // what is kept is the element the pair slot stands for
+      const int e = KC ? o0 + (q >> 3) : o0 + 2 * (q % (EXT / 2));
+      const int k = KC ? k0 + 2 * (q & 7) : k0 + q / (EXT / 2);
+      if (KC) {
+        if (e < ext && s.keep_first && s.first != (size_t)e * (size_t)ld + (size_t)k) bad("%s: (%d, %d) displaced", name, e, k);
+        if (e < ext && s.keep_second && s.second != (size_t)e * (size_t)ld + (size_t)k + 1) bad("%s: (%d, %d) displaced", name, e, k + 1);
+        if (s.keep_first != (k < K) || s.keep_second != (k + 1 < K)) bad("%s: the K mask of pair %d is wrong", name, q);
+      } else {
+        if (e < ext && s.keep_first && s.first != (size_t)k * (size_t)ld + (size_t)e) bad("%s: (%d, %d) displaced", name, e, k);
+        if (e + 1 < ext && s.keep_second && s.second != (size_t)k * (size_t)ld + (size_t)e + 1) bad("%s: (%d, %d) displaced", name, e + 1, k);
+        if (s.keep_first != (k < K) || s.keep_second != (k < K)) bad("%s: the K mask of pair %d is wrong", name, q);
+      }
+    }
     in_range(name, s.first, 1, limit);
     in_range(name, s.second, 1, limit);
     if (s.vec) {
@@ -326,15 +363,29 @@ void check_tail_tile(const char* name, const double* base, int threads, long ld,
   }
 }
 
+// what a launch on the tile DMA promises about its operands
+void check_dma_promises(const GemmParams& p, bool a_kc, bool b_kc) {
+  if (p.M < 2 || p.N < 2) bad("the pair clamps need extents of at least 2");
+  if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) % 8) bad("operands are not 8-byte aligned");
+  if (p.unaligned != 0 && p.unaligned != 1) bad("unaligned = %d", p.unaligned);
+  if (!p.unaligned) {
+    if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) % 16) bad("operands promised 16-byte aligned are not");
+    if (p.lda % 2 || p.ldb % 2) bad("odd leading dimension on operands promised aligned");
+    if ((a_kc ? p.K : p.M) % 2 || (b_kc ? p.K : p.N) % 2) bad("odd contiguous extent on operands promised aligned");
+  }
+  // an output-contiguous operand of odd extent: its last K row must not travel by DMA
+  const bool reach_behind = (!a_kc && p.M % 2) || (!b_kc && p.N % 2);
+  if (reach_behind && p.k_reserve != 1) bad("an odd output-contiguous extent without the last K row kept back");
+}
+
 // all workgroups of one problem on 128x128 direct-to-LDS tiles (8 wavefronts of 64x32)
 void check_dma128_problem(const GemmParams& p, bool a_kc, bool b_kc, long long blocks, bool ragged = false) {
   g_context = std::string("dma128 ") + describe(p, a_kc, b_kc);
   check_params(p, a_kc, b_kc);
   if (p.tiles_m != (p.M + 127) / 128 || p.tiles_n != (p.N + 127) / 128) bad("tile counts do not match 128x128 tiles");
   if (blocks != (long long)p.tiles_m * p.tiles_n * p.split_k) bad("%lld workgroups for %d x %d tiles x %d slices", blocks, p.tiles_m, p.tiles_n, p.split_k);
-  if (p.M < 2 || p.N < 2) bad("the pair clamps need extents of at least 2");
-  if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) % 16) bad("operands are not 16-byte aligned");
-  if (p.lda % 2 || p.ldb % 2) bad("odd leading dimension on the 16-byte DMA path");
+  check_dma_promises(p, a_kc, b_kc);
+  const bool aligned = p.unaligned == 0;
   check_dma_k_cover(p);
   check_lds_layout(a_kc, OcKind::k128, 128, 16);
   check_lds_layout(b_kc, OcKind::k128, 128, 16);
@@ -350,14 +401,14 @@ void check_dma128_problem(const GemmParams& p, bool a_kc, bool b_kc, long long b
     if (visited[id]) bad("tile (%d, %d) of slice %d has two workgroups", tc.tile_m, tc.tile_n, tc.split);
     visited[id] = 1;
     const int m0 = tc.tile_m * 128, n0 = tc.tile_n * 128;
-    const DmaSteps ks = dma_k_steps(p.K, p.split_k, p.steps_per_split, tc.split);
-    check_dma_operand("A tile DMA", p.A, a_kc, OcKind::k128, 128, 16, m0, p.M, p.K, p.lda, ks.kt0, ks.nk_dma);
-    check_dma_operand("B tile DMA", p.B, b_kc, OcKind::k128, 128, 16, n0, p.N, p.K, p.ldb, ks.kt0, ks.nk_dma);
+    const DmaSteps ks = dma_k_steps(p.K, p.split_k, p.steps_per_split, tc.split, p.k_reserve);
+    check_dma_operand("A tile DMA", p.A, a_kc, OcKind::k128, 128, 16, m0, p.M, p.K, p.lda, ks.kt0, ks.nk_dma, aligned);
+    check_dma_operand("B tile DMA", p.B, b_kc, OcKind::k128, 128, 16, n0, p.N, p.K, p.ldb, ks.kt0, ks.nk_dma, aligned);
     if (ks.k_tail) {
-      if (a_kc) check_tail_tile<128, true>("A remainder tile", p.A, 512, p.lda, m0, p.M, p.K);
-      else check_tail_tile<128, false>("A remainder tile", p.A, 512, p.lda, m0, p.M, p.K);
-      if (b_kc) check_tail_tile<128, true>("B remainder tile", p.B, 512, p.ldb, n0, p.N, p.K);
-      else check_tail_tile<128, false>("B remainder tile", p.B, 512, p.ldb, n0, p.N, p.K);
+      if (a_kc) check_tail_tile<128, true>("A remainder tile", p.A, 512, p.lda, m0, p.M, p.K, p.k_reserve, aligned);
+      else check_tail_tile<128, false>("A remainder tile", p.A, 512, p.lda, m0, p.M, p.K, p.k_reserve, aligned);
+      if (b_kc) check_tail_tile<128, true>("B remainder tile", p.B, 512, p.ldb, n0, p.N, p.K, p.k_reserve, aligned);
+      else check_tail_tile<128, false>("B remainder tile", p.B, 512, p.ldb, n0, p.N, p.K, p.k_reserve, aligned);
     }
     for (int wave = 0; wave < 8; ++wave) {
       const int wm = wave / 4, wn = wave % 4;
@@ -376,9 +427,8 @@ void check_dma64_problem(const GemmParams& p, bool b_kc, long long blocks) {
   check_params(p, a_kc, b_kc);
   if (p.tiles_m != (p.M + 63) / 64 || p.tiles_n != (p.N + 63) / 64) bad("tile counts do not match 64x64 tiles");
   if (blocks != (long long)p.tiles_m * p.tiles_n * p.split_k) bad("%lld workgroups for %d x %d tiles x %d slices", blocks, p.tiles_m, p.tiles_n, p.split_k);
-  if (p.M < 2 || p.N < 2) bad("the pair clamps need extents of at least 2");
-  if ((reinterpret_cast<uintptr_t>(p.A) | reinterpret_cast<uintptr_t>(p.B)) % 16) bad("operands are not 16-byte aligned");
-  if (p.lda % 2 || p.ldb % 2) bad("odd leading dimension on the 16-byte DMA path");
+  check_dma_promises(p, a_kc, b_kc);
+  const bool aligned = p.unaligned == 0;
   check_dma_k_cover(p);
   check_lds_layout(true, OcKind::k64, 64, 8);
   check_lds_layout(b_kc, OcKind::k64, 64, 8);
@@ -392,13 +442,13 @@ void check_dma64_problem(const GemmParams& p, bool b_kc, long long blocks) {
     if (visited[id]) bad("tile (%d, %d) of slice %d has two workgroups", tc.tile_m, tc.tile_n, tc.split);
     visited[id] = 1;
     const int m0 = tc.tile_m * 64, n0 = tc.tile_n * 64;
-    const DmaSteps ks = dma_k_steps(p.K, p.split_k, p.steps_per_split, tc.split);
-    check_dma_operand("A tile DMA", p.A, true, OcKind::k64, 64, 8, m0, p.M, p.K, p.lda, ks.kt0, ks.nk_dma);
-    check_dma_operand("B tile DMA", p.B, b_kc, OcKind::k64, 64, 8, n0, p.N, p.K, p.ldb, ks.kt0, ks.nk_dma);
+    const DmaSteps ks = dma_k_steps(p.K, p.split_k, p.steps_per_split, tc.split, p.k_reserve);
+    check_dma_operand("A tile DMA", p.A, true, OcKind::k64, 64, 8, m0, p.M, p.K, p.lda, ks.kt0, ks.nk_dma, aligned);
+    check_dma_operand("B tile DMA", p.B, b_kc, OcKind::k64, 64, 8, n0, p.N, p.K, p.ldb, ks.kt0, ks.nk_dma, aligned);
     if (ks.k_tail) {
-      check_tail_tile<64, true>("A remainder tile", p.A, 256, p.lda, m0, p.M, p.K);
-      if (b_kc) check_tail_tile<64, true>("B remainder tile", p.B, 256, p.ldb, n0, p.N, p.K);
-      else check_tail_tile<64, false>("B remainder tile", p.B, 256, p.ldb, n0, p.N, p.K);
+      check_tail_tile<64, true>("A remainder tile", p.A, 256, p.lda, m0, p.M, p.K, p.k_reserve, aligned);
+      if (b_kc) check_tail_tile<64, true>("B remainder tile", p.B, 256, p.ldb, n0, p.N, p.K, p.k_reserve, aligned);
+      else check_tail_tile<64, false>("B remainder tile", p.B, 256, p.ldb, n0, p.N, p.K, p.k_reserve, aligned);
     }
     for (int wave = 0; wave < 4; ++wave) check_write_block(p, 2, 2, m0 + (wave >> 1) * 32, n0 + (wave & 1) * 32, tc.split, cov);
   }
@@ -635,6 +685,10 @@ void observe_gemm_launch(const GemmLaunch& l) {
   }
   ++g_checked[(int)l.kernel];
   if (l.p && l.p->split_k > 1) ++g_sliced[(int)l.kernel];
+  if (l.p && (l.kernel == GemmKernel::kDma128 || l.kernel == GemmKernel::kDma64) && l.p->unaligned) {
+    ++g_unaligned[(int)l.kernel];
+    if (l.p->k_reserve) ++g_reserved[(int)l.kernel];
+  }
 }
 
 }  // namespace rst
@@ -643,6 +697,8 @@ void observe_gemm_launch(const GemmLaunch& l) {
 extern "C" long address_model_checked(int kernel) { return kernel >= 0 && kernel < 16 ? rst::g_checked[kernel] : 0; }
 extern "C" long address_model_staged_checked(int tile) { return rst::g_staged_by_tile[tile == 32 ? 0 : 1]; }
 extern "C" long address_model_sliced(int kernel) { return kernel >= 0 && kernel < 16 ? rst::g_sliced[kernel] : 0; }
+extern "C" long address_model_unaligned(int kernel) { return kernel >= 0 && kernel < 16 ? rst::g_unaligned[kernel] : 0; }
+extern "C" long address_model_reserved(int kernel) { return kernel >= 0 && kernel < 16 ? rst::g_reserved[kernel] : 0; }
 extern "C" long address_model_repeats() { return rst::g_skipped_repeats; }
 extern "C" long long address_model_lane_checks() { return rst::g_lane_checks; }
 extern "C" const char* address_model_kernel_name(int kernel) { return rst::kernel_name((rst::GemmKernel)kernel); }

@@ -13,6 +13,8 @@
 extern "C" long address_model_checked(int kernel);
 extern "C" long address_model_staged_checked(int tile);
 extern "C" long address_model_sliced(int kernel);
+extern "C" long address_model_unaligned(int kernel);
+extern "C" long address_model_reserved(int kernel);
 extern "C" long address_model_repeats();
 extern "C" long long address_model_lane_checks();
 extern "C" const char* address_model_kernel_name(int kernel);
@@ -155,6 +157,26 @@ int main() {
   run(Case{WEIGHT_GRAD, 1000, 4096, 2048, 0, 0, 0, false, false, 6, 1});
   run(Case{FORWARD, 8192, 100, 784, 0, 0, 0, false, false, 1, 1});
   run(Case{INPUT_GRAD, 8192, 100, 100, 0, 0, 0, false, false, 1, 1});
+  // ---- a network with every extent odd (1023-4095-4095-999 at batch 2047) and its neighbours: the tile DMA
+  //      on 8-byte aligned pairs, the last K row kept back where a pair could reach behind the operand ------
+  for (int batch : {2047, 2048, 2049})
+    for (int pad : {0, 1}) {
+      const int w[4] = {1023, 4095, 4095, 999};
+      for (int l = 0; l < 3; ++l) {
+        run(Case{FORWARD, batch, w[l + 1], w[l], pad, pad, 0, pad == 1, false, 1, 1});
+        run(Case{WEIGHT_GRAD, w[l + 1], w[l], batch, pad, 0, pad, false, pad == 1, 6, 1});
+        run(Case{INPUT_GRAD, batch, w[l], w[l + 1], 0, pad, 0, false, false, 1, 1});
+      }
+    }
+  // K a multiple of 16 with an odd output-contiguous extent (the tail is then a whole step), mid sizes on slices
+  run(Case{WEIGHT_GRAD, 4095, 1023, 2048, 0, 0, 0, false, false, 6, 1});
+  run(Case{INPUT_GRAD, 2048, 1023, 4096, 0, 0, 0, false, false, 1, 1});
+  run(Case{INPUT_GRAD, 8192, 101, 785, 0, 0, 0, false, false, 1, 1});
+  run(Case{FORWARD, 8192, 101, 785, 0, 0, 0, false, false, 1, 1});
+  run(Case{WEIGHT_GRAD, 1001, 1535, 4096, 0, 0, 0, false, false, 6, 1});
+  run(Case{WEIGHT_GRAD, 999, 1023, 16, 0, 0, 0, false, false, 6, 1});
+  run(Case{WEIGHT_GRAD, 4095, 4095, 16, 0, 0, 0, false, false, 6, 1});
+  run(Case{WEIGHT_GRAD, 4095, 4095, 17, 0, 0, 0, false, false, 6, 1});
 
   // ---- grouped launches: weight gradients of small layers, short and long batches ----------------------
   long groups = 0, pairs = 0;
@@ -213,6 +235,10 @@ int main() {
   // sliced and unsliced direct-to-LDS launches, sliced register-staged ones
   all = all && address_model_sliced(0) > 0 && address_model_sliced(3) > 0 && address_model_sliced(6) > 0 &&
         address_model_checked(3) > address_model_sliced(3) && address_model_checked(6) > address_model_sliced(6);
+  std::printf("  tile DMA on operands without aligned pairs: %ld + %ld launches (128x128 + 64x64), %ld + %ld with the last K row kept back\n",
+              address_model_unaligned(3), address_model_unaligned(6), address_model_reserved(3), address_model_reserved(6));
+  all = all && address_model_unaligned(3) > 0 && address_model_unaligned(6) > 0 && address_model_reserved(3) > 0 &&
+        address_model_reserved(6) > 0;
   std::printf("address sweep ok: %ld cases, %ld groups, %ld pairs, %ld launches verified (%ld repeats skipped), %lld address checks\n",
               g_cases, groups, pairs, total, address_model_repeats(), address_model_lane_checks());
   if (!all) {

@@ -28,10 +28,22 @@ def test_every_planned_lane_stays_inside_its_operand():
     assert "address sweep ok" in run.stdout
 
 
-def test_the_model_catches_a_wrong_offset(tmp_path):
+MUTANTS = {
+    # the tile DMA's last-row clamp, off by one
+    "last_row_clamp": ("const int rr = o0 + row < ext ? row : ext - 1 - o0;",
+                       "const int rr = o0 + row < ext ? row : ext - o0;"),
+    # the last row of the contraction is not kept away from the tile DMA: the pair on the last column
+    # of an odd, output-contiguous extent then reads one double behind the operand
+    "last_k_row_not_kept_back": ("RST_HD int dma_whole_steps(int K, int k_reserve) { return (K - k_reserve) / BK; }",
+                                 "RST_HD int dma_whole_steps(int K, int k_reserve) { return K / BK; }"),
+}
+
+
+@pytest.mark.parametrize("mutant", sorted(MUTANTS))
+def test_the_model_catches_a_wrong_offset(tmp_path, mutant):
     """The checker is only worth something if it fails when the arithmetic is wrong: rebuild the
-    model and the library's contraction source against a copy of the index header in which one clamp
-    is off by one (the tile DMA's last-row clamp), and the sweep must abort with a bounds message."""
+    model and the library's contraction source against a copy of the index header with one line
+    changed, and the sweep must abort with a bounds message."""
     if shutil.which("hipcc") is None and not os.path.exists("/opt/rocm/bin/hipcc"):
         pytest.skip("needs hipcc")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -43,9 +55,9 @@ def test_the_model_catches_a_wrong_offset(tmp_path):
     shutil.copytree(os.path.join(root, "include"), work / "include", ignore=shutil.ignore_patterns("__pycache__"))
     header = work / "rstorch_amd" / "csrc" / "gemm_addressing.h"
     text = header.read_text()
-    good = "const int rr = o0 + row < ext ? row : ext - 1 - o0;"
+    good, wrong = MUTANTS[mutant]
     assert text.count(good) == 1
-    header.write_text(text.replace(good, "const int rr = o0 + row < ext ? row : ext - o0;"))
+    header.write_text(text.replace(good, wrong))
     build = subprocess.run(["make", "-C", str(work / "tests" / "host_stub"), "-j8", "-s", "build/address_sweep_driver"],
                            capture_output=True, text=True)
     assert build.returncode == 0, build.stderr[-3000:]

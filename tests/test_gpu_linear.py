@@ -41,6 +41,11 @@ SHAPES = [
     (2048, 1000, 512), (1024, 1024, 512), (4096, 64, 2048), (2050, 1022, 510), (16384, 512, 64),
     # small outputs with a long contraction: the split-K path (with and without a K tail)
     (8192, 784, 100), (8192, 100, 10), (32, 4099, 24), (4100, 7, 9), (16384, 33, 65),
+    # odd extents and leading dimensions on the direct-to-LDS kernels (8-byte aligned pairs; where an
+    # output-contiguous operand has an odd extent the last row of the contraction goes with the tail):
+    # 128x128 tiles unsliced and on K slices, a batch that is a multiple of 16 (the tail is then a
+    # whole step), the 64x64 tiles, a single last column in a tile of its own (1025 = 8 x 128 + 1)
+    (2047, 1023, 4095), (2048, 1023, 4095), (2049, 2047, 1025), (8192, 785, 101), (1031, 4097, 515),
 ]
 
 
