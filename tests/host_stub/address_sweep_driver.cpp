@@ -177,6 +177,11 @@ int main() {
   run(Case{WEIGHT_GRAD, 999, 1023, 16, 0, 0, 0, false, false, 6, 1});
   run(Case{WEIGHT_GRAD, 4095, 4095, 16, 0, 0, 0, false, false, 6, 1});
   run(Case{WEIGHT_GRAD, 4095, 4095, 17, 0, 0, 0, false, false, 6, 1});
+  // 256..511 tiles over a very long contraction (two K halves), odd everywhere
+  run(Case{WEIGHT_GRAD, 2047, 2045, 24577, 0, 0, 0, false, false, 6, 1});
+  run(Case{WEIGHT_GRAD, 2047, 2045, 24576, 1, 0, 0, false, false, 6, 1});
+  run(Case{INPUT_GRAD, 2049, 2047, 24593, 0, 0, 0, true, false, 1, 1});
+  run(Case{FORWARD, 2047, 2049, 24577, 0, 0, 0, false, true, 1, 1});
 
   // ---- grouped launches: weight gradients of small layers, short and long batches ----------------------
   long groups = 0, pairs = 0;

@@ -86,7 +86,8 @@ def test_backward_matches_oracle(engine, oracle, batch, k, n):
 
 # 256..511 tiles with a very long contraction (K >= 24576): the direct-to-LDS kernels cut K in two
 # halves - forward, input gradient, and weight gradient (+ bias gradient over slices) in turn
-@pytest.mark.parametrize("batch,k,n", [(2048, 24576, 2046), (2064, 2048, 24576), (24576, 2048, 2046)])
+@pytest.mark.parametrize("batch,k,n", [(2048, 24576, 2046), (2064, 2048, 24576), (24576, 2048, 2046),
+                                       (24577, 2047, 2045)])  # (the last: odd everywhere, 8-byte aligned pairs)
 def test_two_way_k_split_matches_oracle(engine, oracle, batch, k, n):
     import rstorch_amd as rs
     rng = np.random.default_rng(batch + 3 * k + 7 * n)
