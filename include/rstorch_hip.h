@@ -272,7 +272,7 @@ int rst_model_train_step(rst_model* model, const double* x, const double* truth,
 int rst_model_fuse_sgd(rst_model* model, int enabled);
 /* enabled != 0: the backward pass holds each layer's weight gradient back until the next layer's
  * input gradient is due and launches the two, which do not depend on each other, as one grid when
- * both are large aligned products (a 256-tile input gradient alone leaves one workgroup per CU).
+ * both are large products (a 256-tile input gradient alone leaves one workgroup per CU).
  * Results are identical either way.  On by default (measured on MI355X at C4's hidden width:
  * 0.946 ms per pair against 0.477 + 0.503 ms for the two launches one after the other). */
 int rst_model_pair_gradients(rst_model* model, int enabled);

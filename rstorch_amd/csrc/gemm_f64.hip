@@ -483,7 +483,9 @@ __global__ __launch_bounds__(256, (BURST > 0 ? 1 : 2)) void gemm_f64_mfma_group(
   __shared__ __attribute__((aligned(16))) double lds_a[tile_lds_doubles<32, A_KC, 256, BURST>()];
   __shared__ __attribute__((aligned(16))) double lds_b[tile_lds_doubles<32, B_KC, 256, BURST>()];
   const int i = group_member_of_block(g.first_block, g.count, (int)blockIdx.x);
-  gemm_tile<32, 32, 2, 2, A_KC, B_KC, true, BURST>(g.p[i], (int)blockIdx.x - g.first_block[i], lds_a, lds_b);
+  // (uniform over the workgroup: a member whose operands do not promise aligned pairs loads singly)
+  if (g.p[i].unaligned) gemm_tile<32, 32, 2, 2, A_KC, B_KC, false, BURST>(g.p[i], (int)blockIdx.x - g.first_block[i], lds_a, lds_b);
+  else gemm_tile<32, 32, 2, 2, A_KC, B_KC, true, BURST>(g.p[i], (int)blockIdx.x - g.first_block[i], lds_a, lds_b);
 }
 
 // The same with a layout per problem (a layer's input gradient next to its weight gradient).
@@ -494,11 +496,16 @@ __global__ __launch_bounds__(256, (BURST > 0 ? 1 : 2)) void gemm_f64_mfma_mixed_
   __shared__ __attribute__((aligned(16))) double lds_b[tile_lds_doubles<32, false, 256, BURST>()];
   const int i = group_member_of_block(g.first_block, g.count, (int)blockIdx.x);
   const int block = (int)blockIdx.x - g.first_block[i];
-  switch (g.layout[i]) {
+  switch (g.layout[i] | (g.p[i].unaligned ? 4 : 0)) {
     case 0: gemm_tile<32, 32, 2, 2, false, false, true, BURST>(g.p[i], block, lds_a, lds_b); break;
     case 1: gemm_tile<32, 32, 2, 2, true, false, true, BURST>(g.p[i], block, lds_a, lds_b); break;
     case 2: gemm_tile<32, 32, 2, 2, false, true, true, BURST>(g.p[i], block, lds_a, lds_b); break;
-    default: gemm_tile<32, 32, 2, 2, true, true, true, BURST>(g.p[i], block, lds_a, lds_b); break;
+    case 3: gemm_tile<32, 32, 2, 2, true, true, true, BURST>(g.p[i], block, lds_a, lds_b); break;
+    // members whose operands do not promise aligned pairs: single loads
+    case 4: gemm_tile<32, 32, 2, 2, false, false, false, BURST>(g.p[i], block, lds_a, lds_b); break;
+    case 5: gemm_tile<32, 32, 2, 2, true, false, false, BURST>(g.p[i], block, lds_a, lds_b); break;
+    case 6: gemm_tile<32, 32, 2, 2, false, true, false, BURST>(g.p[i], block, lds_a, lds_b); break;
+    default: gemm_tile<32, 32, 2, 2, true, true, false, BURST>(g.p[i], block, lds_a, lds_b); break;
   }
 }
 
@@ -1442,11 +1449,12 @@ GemmParams make_params(const GemmDesc& d) {
 
 // true when launch_gemm would run d as unsplit 128x128 direct-to-LDS tiles
 bool takes_plain_dma(const GemmDesc& d, long long* blocks) {
-  if (d.M < 2 || d.N < 2 || d.K <= 0 || d.K % BK != 0 || !desc_vec_ok(d)) return false;
+  if (d.M < 2 || d.N < 2 || d.K <= 0) return false;
   if (d.lda >= (1L << 22) || d.ldb >= (1L << 22)) return false;
   *blocks = (long long)((d.M + 127) / 128) * ((d.N + 127) / 128);
   if (*blocks < 256) return false;
-  return !(*blocks < 512 && d.K / BK >= kSplitMinSteps && d.workspace != nullptr);
+  const GemmParams p = make_params(d);
+  return !(*blocks < 512 && dma_whole_steps(p.K, p.k_reserve) >= kSplitMinSteps && d.workspace != nullptr);
 }
 
 }  // namespace
@@ -1476,8 +1484,7 @@ void plan_group_member(GemmParams& p) {
 }  // namespace
 
 bool can_group_gemm(const GemmDesc& d) {
-  // the grouped kernels use 16-byte loads
-  if (d.M <= 0 || d.N <= 0 || !desc_vec_ok(d)) return false;
+  if (d.M <= 0 || d.N <= 0) return false;
   const GemmParams p = make_params(d);
   int slices = 0;
   return choose_route(p, &slices, d.a_kc, d.b_kc) == Route::kTile32;
@@ -1507,7 +1514,7 @@ constexpr int kDmaGroupGrid = 256;
 // tiles (more have enough workgroups of their own, and the slices of a larger output would crowd
 // the shared workspace)
 bool dma_group_member(const GemmDesc& d) {
-  return !d.a_kc && !d.b_kc && desc_vec_ok(d) && d.K / BK >= 2 * kDmaGroupMinSteps && d.M >= 2 && d.N >= 2 &&
+  return !d.a_kc && !d.b_kc && d.K / BK >= 2 * kDmaGroupMinSteps && d.M >= 2 && d.N >= 2 &&
          (long long)((d.M + 127) / 128) * ((d.N + 127) / 128) <= 8 && d.lda < (1L << 22) && d.ldb < (1L << 22) &&
          d.workspace != nullptr;
 }

@@ -668,7 +668,8 @@ void observe_gemm_launch(const GemmLaunch& l) {
       for (int i = 0; i < l.group->count; ++i) {
         const bool a_kc = l.kernel == GemmKernel::kStagedMixedGroup ? (l.group->layout[i] & 1) != 0 : l.a_kc;
         const bool b_kc = l.kernel == GemmKernel::kStagedMixedGroup ? (l.group->layout[i] & 2) != 0 : l.b_kc;
-        check_staged_problem(l.group->p[i], 32, 32, 2, 2, a_kc, b_kc, true, l.group->first_block[i + 1] - l.group->first_block[i]);
+        check_staged_problem(l.group->p[i], 32, 32, 2, 2, a_kc, b_kc, l.group->p[i].unaligned == 0,
+                             l.group->first_block[i + 1] - l.group->first_block[i]);
       }
       break;
     }
@@ -685,9 +686,19 @@ void observe_gemm_launch(const GemmLaunch& l) {
   }
   ++g_checked[(int)l.kernel];
   if (l.p && l.p->split_k > 1) ++g_sliced[(int)l.kernel];
-  if (l.p && (l.kernel == GemmKernel::kDma128 || l.kernel == GemmKernel::kDma64) && l.p->unaligned) {
+  if (l.p && (l.kernel == GemmKernel::kDma128 || l.kernel == GemmKernel::kDma64 || l.kernel == GemmKernel::kDma128Pair) &&
+      (l.p->unaligned || (l.p2 && l.p2->unaligned))) {
     ++g_unaligned[(int)l.kernel];
-    if (l.p->k_reserve) ++g_reserved[(int)l.kernel];
+    if (l.p->k_reserve || (l.p2 && l.p2->k_reserve)) ++g_reserved[(int)l.kernel];
+  }
+  if (l.group) {
+    bool any = false, reserved = false;
+    for (int i = 0; i < l.group->count; ++i) {
+      any = any || l.group->p[i].unaligned;
+      reserved = reserved || l.group->p[i].k_reserve;
+    }
+    if (any) ++g_unaligned[(int)l.kernel];
+    if (reserved) ++g_reserved[(int)l.kernel];
   }
 }
 

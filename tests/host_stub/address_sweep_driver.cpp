@@ -191,10 +191,14 @@ int main() {
     std::vector<GemmDesc> ds;
     bool ok = true;
     for (int i = 0; i < count; ++i) {
-      Case c{WEIGHT_GRAD, 2 * (1 + (int)rnd(150)), 2 * (1 + (int)rnd(400)), batch, 0, 0, 0, false, false, 2 + 4 * (int)rnd(2), 1};
+      // every third group has members of odd extents (single loads, 8-byte aligned tile DMA)
+      const int odd = it % 3 == 2 ? 1 : 0;
+      Case c{WEIGHT_GRAD, 2 * (1 + (int)rnd(150)) - odd * (int)rnd(2), 2 * (1 + (int)rnd(400)) - odd * (int)rnd(2), batch - odd * (int)rnd(2),
+             0, 0, 0, false, false, 2 + 4 * (int)rnd(2), 1};
       GemmDesc d = make(c);
       if (it % 5 == 4 && i == count - 1) {  // a layer's input gradient riding along (mixed layouts)
-        Case x{INPUT_GRAD, batch, 2 * (1 + (int)rnd(60)), 2 * (1 + (int)rnd(60)), 0, 0, 0, false, false, (int)rnd(2), 1};
+        Case x{INPUT_GRAD, batch, 2 * (1 + (int)rnd(60)) - odd * (int)rnd(2), 2 * (1 + (int)rnd(60)) - odd * (int)rnd(2), 0, 0, 0, false, false,
+               (int)rnd(2), 1};
         d = make(x);
       }
       ok = ok && can_group_gemm(d);
@@ -208,8 +212,8 @@ int main() {
     ++groups;
   }
   // ---- paired launches: an input gradient with the weight gradient of the layer above ------------------
-  const int widths[] = {2048, 4096, 4224, 8192, 32768};
-  for (int batch : {1024, 2048, 4096})
+  const int widths[] = {2048, 4096, 4224, 8192, 32768, 4095, 2049};
+  for (int batch : {1024, 2048, 4096, 1023, 2047})
     for (int w_in : widths)
       for (int w_out : widths) {
         // (one pair with the 32768-wide head, the others up to 32 Mi outputs)
@@ -242,8 +246,12 @@ int main() {
         address_model_checked(3) > address_model_sliced(3) && address_model_checked(6) > address_model_sliced(6);
   std::printf("  tile DMA on operands without aligned pairs: %ld + %ld launches (128x128 + 64x64), %ld + %ld with the last K row kept back\n",
               address_model_unaligned(3), address_model_unaligned(6), address_model_reserved(3), address_model_reserved(6));
+  std::printf("  shared grids with such members: %ld + %ld + %ld + %ld launches (staged, mixed, 128x128 sliced, pairs)\n",
+              address_model_unaligned(1), address_model_unaligned(2), address_model_unaligned(4), address_model_unaligned(5));
   all = all && address_model_unaligned(3) > 0 && address_model_unaligned(6) > 0 && address_model_reserved(3) > 0 &&
-        address_model_reserved(6) > 0;
+        address_model_reserved(6) > 0 && address_model_unaligned(1) > 0 && address_model_unaligned(2) > 0 &&
+        address_model_unaligned(4) > 0 && address_model_unaligned(5) > 0 && address_model_reserved(4) > 0 &&
+        address_model_reserved(5) > 0;
   std::printf("address sweep ok: %ld cases, %ld groups, %ld pairs, %ld launches verified (%ld repeats skipped), %lld address checks\n",
               g_cases, groups, pairs, total, address_model_repeats(), address_model_lane_checks());
   if (!all) {

@@ -28,6 +28,15 @@ CASES = [
     ("C4_deep_reduced", [("linear", 512, 512), ("relu",)] * 8 + [("linear", 512, 4096)], 128, True, 0.01),
     ("ragged", [("identity",), ("linear", 33, 65), ("relu",), ("identity",), ("linear", 65, 129),
                 ("relu",), ("linear", 129, 7)], 67, True, 0.05),
+    # every extent odd: the shared grids with members that load singly (small batch), the K-sliced
+    # 128x128 grid and the 64x64 tiles on 8-byte aligned pairs (long batch), and wide layers whose
+    # gradients pair up on the tile DMA with the last row of the contraction kept back
+    ("odd_readme_b33", [("identity",), ("linear", 785, 101), ("relu",), ("linear", 101, 101), ("relu",),
+                        ("linear", 101, 11)], 33, False, 0.01),
+    ("odd_readme_b8191", [("identity",), ("linear", 785, 101), ("relu",), ("linear", 101, 101), ("relu",),
+                          ("linear", 101, 11)], 8191, False, 0.01),
+    ("odd_wide_b1023", [("linear", 511, 2049), ("relu",), ("linear", 2049, 4095), ("relu",), ("linear", 4095, 2047),
+                        ("relu",), ("linear", 2047, 999)], 1023, True, 0.01),
 ]
 
 
@@ -193,10 +202,16 @@ GROUP_CASES = [
     # more small layers than one shared grid holds (eight): two grids
     ("twelve_small_layers", [("linear", 20, 34), ("relu",)] + [("linear", 34, 34), ("relu",)] * 10 +
      [("linear", 34, 6)], 16, True),
-    # a layer large enough for the 128x128 kernels between small ones, and an odd width that
-    # rules out 16-byte loads
+    # a layer large enough for the 128x128 kernels between small ones, and an odd width (a member of
+    # the shared grid that loads singly)
     ("mixed", [("linear", 64, 2048), ("relu",), ("linear", 2048, 2048), ("relu",), ("linear", 2048, 33),
                ("relu",), ("linear", 33, 10)], 64, True),
+    # every extent odd: members that load singly (small batch) and the K-sliced 128x128 grid on
+    # 8-byte aligned pairs (long batch)
+    ("odd_readme_b33", [("identity",), ("linear", 785, 101), ("relu",), ("linear", 101, 101), ("relu",),
+                        ("linear", 101, 11)], 33, True),
+    ("odd_readme_b8191", [("identity",), ("linear", 785, 101), ("relu",), ("linear", 101, 101), ("relu",),
+                          ("linear", 101, 11)], 8191, False),
 ]
 
 
@@ -307,6 +322,9 @@ PAIR_CASES = [
     ("paired", [("linear", 2048, 2048), ("relu",)] * 3 + [("linear", 2048, 4096)], 2048),
     ("paired_ragged_edges", [("linear", 2050, 2046), ("relu",), ("linear", 2046, 2064), ("relu",),
                              ("linear", 2064, 2304)], 2064),
+    # every extent odd: both products of a pair on 8-byte aligned tile DMA, the last row of each
+    # contraction with the tail
+    ("paired_odd", [("linear", 2047, 2049), ("relu",), ("linear", 2049, 2047), ("relu",), ("linear", 2047, 4095)], 2047),
     ("never_paired", README_MLP, 64),
 ]
 
