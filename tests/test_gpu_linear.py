@@ -243,6 +243,23 @@ def _sweep_cases():
             b = int(rng.integers(40, 140)) * 128 + int(rng.choice([0, 8]))
             k, n = int(rng.integers(5, 130)) * 2, int(rng.integers(5, 130)) * 2
         cases.append((b, k, n))
+    # odd extents on every direct-to-LDS route (8-byte aligned pairs, the last row of the contraction with
+    # the tail where an output-contiguous operand has an odd extent)
+    rng = np.random.default_rng(777)
+    for _ in range(18):
+        kind = int(rng.integers(0, 3))
+        if kind == 0:    # hundreds of 128x128 tiles
+            b, k, n = (2 * int(rng.integers(700, 1500)) + 1 for _ in range(3))
+        elif kind == 1:  # few tiles and a long contraction: K slices
+            b = int(rng.integers(1, 8)) * 128 + int(rng.choice([-1, 1, 31]))
+            n = int(rng.integers(2, 20)) * 128 - int(rng.choice([1, 3, 101]))
+            k = 2 * int(rng.integers(160, 2400)) + 1
+        else:            # the 64x64 band
+            b = int(rng.integers(16, 130)) * 64 + int(rng.choice([-1, 1, 9]))
+            k, n = 2 * int(rng.integers(96, 560)) + 1, 2 * int(rng.integers(8, 130)) + 1
+            if rng.integers(0, 2):
+                k, n = n + 190, k
+        cases.append((b, k, n))
     return cases
 
 
