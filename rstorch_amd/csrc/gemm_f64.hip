@@ -1309,6 +1309,35 @@ int dma64_mode() {
   return mode;
 }
 
+// K slices (1 = none) for a product of 257..511 tiles of 128x128, by a cost model in microseconds fitted
+// to this part: 512 workgroups in flight (two per CU) advance one K step in 3.65 us, up to 256 (one per
+// CU) in 1.95 us, later workgroups start as earlier ones leave; the reduction of s slices moves
+// (2 s + 1) M N doubles at 4.5 TB/s behind a launch of 8 us.  Constants, not the device's own counts:
+// the number of slices fixes the order of the summation, which must not change from device to device.
+int band_slices(const GemmParams& p, long long t128) {
+  const int nk = dma_whole_steps(p.K, p.k_reserve);
+  auto cost = [&](int s) {
+    const int steps = (nk + s - 1) / s;
+    const long long wgs = t128 * s, full = wgs / 512, rem = wgs % 512;
+    double c = (double)full * 3.65 * steps;
+    if (rem > 256) c += 3.65 * steps;
+    else if (rem > 0) c += 1.95 * steps;
+    if (s > 1) c += 8.0 + (2.0 * s + 1.0) * (double)p.M * (double)p.N * 8.0 / 4.5e6;
+    return c;
+  };
+  int best = 1;
+  double best_cost = cost(1);
+  for (int s = 2; s <= 4; ++s) {
+    if (nk / s < 32 || p.ws_capacity < (size_t)s * ((size_t)p.M * p.N + (size_t)p.M)) break;
+    const double c = cost(s);
+    if (c < 0.95 * best_cost) {  // (a slice more has to pay for itself by a margin)
+      best = s;
+      best_cost = c;
+    }
+  }
+  return best;
+}
+
 Route choose_route(const GemmParams& p, int* dma_slices, bool is_a_kc = false, bool is_b_kc = false) {
   auto tiles = [&](int bm, int bn) {
     return (long long)((p.M + bm - 1) / bm) * ((p.N + bn - 1) / bn);
@@ -1318,7 +1347,21 @@ Route choose_route(const GemmParams& p, int* dma_slices, bool is_a_kc = false, b
   const bool dma_ok = p.K > 0 && p.M >= 2 && p.N >= 2 && p.lda < (1L << 22) && p.ldb < (1L << 22);
   const long long t128 = tiles(128, 128);
   *dma_slices = 0;
-  if (t128 >= 256) return dma_ok ? Route::kDma : Route::kTile128;
+  if (t128 >= 256) {
+    if (!dma_ok) return Route::kTile128;
+    // Forward products of 257..511 tiles: two workgroups fit on a CU, so all tiles start at once, the CUs
+    // that got two finish in twice the time of those that got one, and the launch takes as long as 512
+    // tiles would (1024 x 4608 at K = 4096, 288 tiles: 907 us, 54 % of the MFMA peak).  K slices make the
+    // pieces small enough to even that out, at the price of the partial results and their reduction.
+    if (is_a_kc && is_b_kc && t128 > 256 && t128 < 512 && p.ws != nullptr) {
+      const int s = band_slices(p, t128);
+      if (s > 1) {
+        *dma_slices = s;
+        return Route::kDmaSliced;
+      }
+    }
+    return Route::kDma;
+  }
   // 32..255 tiles of 128x128 with a long contraction: the direct-to-LDS kernel on up to eight K
   // slices (about two workgroups per CU, at least 32 K steps each) plus the ordered reduction
   // beats the smaller register-staged tiles by far (128 tiles, K = 4096: 87 % of the MFMA peak

@@ -177,6 +177,12 @@ int main() {
   run(Case{WEIGHT_GRAD, 999, 1023, 16, 0, 0, 0, false, false, 6, 1});
   run(Case{WEIGHT_GRAD, 4095, 4095, 16, 0, 0, 0, false, false, 6, 1});
   run(Case{WEIGHT_GRAD, 4095, 4095, 17, 0, 0, 0, false, false, 6, 1});
+  // forward products of 257..511 tiles: K slices that even out the compute units (two, three slices; ragged, odd)
+  run(Case{FORWARD, 1024, 4608, 4096, 0, 0, 0, false, false, 1, 1});
+  run(Case{FORWARD, 1024, 4608, 2048, 0, 0, 0, false, false, 0, 1});
+  run(Case{FORWARD, 1030, 4600, 2056, 0, 0, 0, false, false, 1, 1});
+  run(Case{FORWARD, 1535, 4095, 4097, 0, 0, 0, false, false, 1, 1});
+  run(Case{FORWARD, 1024, 4608, 4096, 0, 0, 0, false, false, 1, 0});  // (no workspace: unsliced)
   // 256..511 tiles over a very long contraction (two K halves), odd everywhere
   run(Case{WEIGHT_GRAD, 2047, 2045, 24577, 0, 0, 0, false, false, 6, 1});
   run(Case{WEIGHT_GRAD, 2047, 2045, 24576, 1, 0, 0, false, false, 6, 1});

@@ -46,6 +46,9 @@ SHAPES = [
     # 128x128 tiles unsliced and on K slices, a batch that is a multiple of 16 (the tail is then a
     # whole step), the 64x64 tiles, a single last column in a tile of its own (1025 = 8 x 128 + 1)
     (2047, 1023, 4095), (2048, 1023, 4095), (2049, 2047, 1025), (8192, 785, 101), (1031, 4097, 515),
+    # forward products of 257..511 tiles of 128x128: K slices even out the compute units that would
+    # otherwise get two tiles against one (288 tiles on two slices; 324 ragged tiles with a K remainder)
+    (1024, 2048, 4608), (1030, 2056, 4600),
 ]
 
 
