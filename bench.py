@@ -48,7 +48,7 @@ PEAK_HBM_GBPS = 8000.0
 # the profile is collected again and the digest updated.
 C4_TRAFFIC_SOURCE = {"profile": "profiles/c4_hbm_traffic.md",
                      "kernel_sources": ["rstorch_amd/csrc/gemm_f64.hip", "rstorch_amd/csrc/gemm_addressing.h"],
-                     "kernel_sources_sha16": "77e33a52b9339aa7"}
+                     "kernel_sources_sha16": "237284b084fa9419"}
 
 
 def kernel_sources_digest():
@@ -61,12 +61,12 @@ def kernel_sources_digest():
 
 
 C4_TRAFFIC_BYTES_PER_LAUNCH = {
-    "linear_forward": (8 * 436.4e6 + 3894.9e6) / 9,
-    "grad_weight": (8 * 862.3e6 + 7559.0e6) / 9,
-    "grad_input": (7 * 470.0e6 + 3337.0e6 + 134.3e6) / 8,
+    "linear_forward": (8 * 436.4e6 + 3856.8e6) / 9,
+    "grad_weight": (8 * 862.0e6 + 7544.6e6) / 9,
+    "grad_input": (7 * 470.0e6 + 3336.4e6 + 134.3e6) / 8,
     # a layer's weight gradient + SGD and the next layer's input gradient in one grid (the default):
     # six pairs at the hidden width and the one that carries the head's weight gradient
-    "grad_pair": (6 * 1527.7e6 + 8362.0e6) / 7,
+    "grad_pair": (6 * 1525.6e6 + 8036.9e6) / 7,
 }
 
 C4_SPEC = [("linear", 4096, 4096), ("relu",)] * 8 + [("linear", 4096, 32768)]

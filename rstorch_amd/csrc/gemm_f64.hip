@@ -1452,8 +1452,8 @@ int launch_layout(hipStream_t stream, const GemmParams& p) {
 
 namespace {
 
-// 16-byte register loads (and the shared-grid kernels) need both operands aligned with even
-// leading dimensions and extents
+// 16-byte register loads need both operands aligned with even leading dimensions and extents;
+// launches on other operands load singly (GemmParams::unaligned)
 bool desc_vec_ok(const GemmDesc& d) {
   auto ok = [](const double* ptr, long ld, int contiguous_extent) {
     return (reinterpret_cast<uintptr_t>(ptr) % 16 == 0) && (ld % 2 == 0) &&
