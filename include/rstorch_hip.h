@@ -257,6 +257,23 @@ int rst_model_backward(rst_model* model, const double* grad, int need_input_grad
 int rst_model_forward_to(rst_model* model, const double* x, size_t batch, double* logits_out);
 int rst_model_backward_to(rst_model* model, const double* grad, double* input_grad_out, int apply_sgd,
                           double lr);
+/* The loss and the accuracy of the logits that the model's latest rst_model_forward_to wrote
+ * (pred must be that address), for the loop of README.md:64-74, whose host waits for the loss
+ * between the forward and the backward pass: rst_cross_entropy_accuracy(pred, truth, grad_out, ...)
+ * and, with inputs_ahead != 0, the part of the coming backward pass that changes nothing a caller
+ * can see - the input gradients of every Linear above the first, from grad_out, into the model's own
+ * buffers - launched behind the loss kernels BEFORE the host waits, so that the GPU has work while the
+ * host wakes up and enqueues the rest.  Same kernels on the same operands as rst_model_backward_to
+ * would launch: a following rst_model_backward_to(model, grad_out, ...) skips them and its results
+ * are the same to the bit; with any other grad address it computes everything itself.  The caller
+ * promises that grad_out is not rewritten in between, or calls rst_model_discard_inputs.  Only small
+ * models take part (every weight gradient waits for the shared grid at the end of backward anyway,
+ * every ReLU sits right below a Linear, profiling is off); for the others inputs_ahead is ignored.
+ * host_accuracy may be NULL (the loss alone, as rst_cross_entropy). */
+int rst_model_loss_accuracy_to(rst_model* model, const double* pred, const double* truth,
+                               double* grad_out, int inputs_ahead, double* host_loss,
+                               double* host_accuracy);
+int rst_model_discard_inputs(rst_model* model);
 /* SGD::step over every parameter of the model (one launch over the arena). */
 int rst_model_sgd_step(rst_model* model, double lr);
 /* forward, loss, backward, step: the README loop body (README.md:64-74) without accuracy,

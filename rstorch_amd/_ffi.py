@@ -112,6 +112,8 @@ SIGNATURES = {
     "rst_model_backward": [_vp, _dp, _i32, c_void_pp],
     "rst_model_forward_to": [_vp, _dp, _sz, _dp],
     "rst_model_backward_to": [_vp, _dp, _dp, _i32, _dbl],
+    "rst_model_loss_accuracy_to": [_vp, _dp, _dp, _dp, _i32, _dp, _dp],
+    "rst_model_discard_inputs": [_vp],
     "rst_model_sgd_step": [_vp, _dbl],
     "rst_model_train_step": [_vp, _dp, _dp, _sz, _dbl, c_double_p],
     "rst_model_profile_enable": [_vp, _i32],

@@ -80,6 +80,10 @@ class Array2 {
     std::shared_ptr<void> keepalive;
     std::function<void()> before_access;
     std::function<void(Storage&)> resolver;  // runs once
+    // set on the logits a compiled Sequential returns: CrossEntropyLoss::forward hands its work to the
+    // compiled form, which knows what follows a loss in a training loop (true: loss and accuracy are
+    // there and `grad` is filled)
+    std::function<bool(const Array2& pred, const Array2& truth, Array2& grad, double* loss, double* accuracy)> loss_through;
     double* get() {
       if (resolver) {
         auto r = std::move(resolver);
@@ -481,7 +485,35 @@ class Plan : public std::enable_shared_from_this<Plan> {
     x_ = std::move(input);
     out_ = out;
     live_ = true;
+    // a loss on these logits that the previous step followed up with a backward pass: a training loop
+    training_ = loss_seen_ && backward_followed_;
+    loss_seen_ = backward_followed_ = false;
+    inputs_from_.reset();
+    std::weak_ptr<Plan> self = shared_from_this();
+    out.storage()->loss_through = [self](const Array2& pred, const Array2& truth, Array2& grad, double* loss, double* acc) {
+      auto p = self.lock();
+      return p && p->loss_through(pred, truth, grad, loss, acc);
+    };
     return out;
+  }
+
+  // CrossEntropyLoss::forward on the logits of the latest forward pass.  In a training loop the
+  // input gradients of the layers above the first are launched behind the loss, before the host
+  // waits for it (rst_model_loss_accuracy_to): the GPU works while the host wakes up, calls
+  // model.backward(loss.backward()) and optim.step(model), and that pass then skips them.  They are
+  // only kept if the gradient array reaches backward() without anybody having looked at it.
+  bool loss_through(const Array2& pred, const Array2& truth, Array2& grad, double* loss, double* acc) {
+    if (!live_ || pending_ || pred.storage() != out_.storage() || !pred.same_shape(truth)) return false;
+    check(rst_model_loss_accuracy_to(model_, pred.data(), truth.data(), grad.data(), training_ ? 1 : 0, loss, acc));
+    loss_seen_ = true;
+    if (training_) {
+      inputs_from_ = grad.storage();
+      std::weak_ptr<Plan> self = shared_from_this();
+      grad.storage()->before_access = [self] {
+        if (auto p = self.lock()) p->inputs_touched();
+      };
+    }
+    return true;
   }
 
   Array2 backward(Array2 gradient) {
@@ -495,6 +527,7 @@ class Plan : public std::enable_shared_from_this<Plan> {
     grad_ = std::move(gradient);
     gin_ = gin.storage();
     pending_ = true;
+    backward_followed_ = true;
     for (Linear* l : linears_) l->mark_gradient();
     return gin;
   }
@@ -552,6 +585,12 @@ class Plan : public std::enable_shared_from_this<Plan> {
     }
   }
 
+  // somebody looked at (and may have rewritten) the gradient the input gradients were launched from
+  void inputs_touched() {
+    rst_model_discard_inputs(model_);
+    inputs_from_.reset();
+  }
+
   void resolve_input_gradient(Array2::Storage& s) {
     if (pending_ && gin_.lock().get() == &s) run(false, 0.0);
   }
@@ -565,6 +604,12 @@ class Plan : public std::enable_shared_from_this<Plan> {
       gin->materialise(x_.nrows() * in_width_);
     }
     Array2 g = std::move(grad_);
+    if (auto from = inputs_from_.lock()) {
+      // the gradient the input gradients were launched from, untouched since: our own access keeps them
+      if (from == g.storage()) from->before_access = nullptr;
+      else inputs_touched();
+    }
+    inputs_from_.reset();
     check(rst_model_backward_to(model_, g.data(), gin ? gin->ptr : nullptr, apply_sgd ? 1 : 0, lr));
     x_ = Array2();
     out_ = Array2();  // the caches are consumed
@@ -578,7 +623,9 @@ class Plan : public std::enable_shared_from_this<Plan> {
   size_t in_width_ = 0, out_width_ = 0;
   Array2 x_, out_, grad_;  // the forward pass whose caches are live; the gradient of the owed backward
   std::weak_ptr<Array2::Storage> gin_;  // the input gradient that backward returned, if still held
+  std::weak_ptr<Array2::Storage> inputs_from_;  // the loss gradient that input gradients were launched from
   bool live_ = false, pending_ = false;
+  bool training_ = false, loss_seen_ = false, backward_followed_ = false;
 };
 
 }  // namespace detail
@@ -750,8 +797,10 @@ class CrossEntropyLoss : public Loss {
     if (!pred.same_shape(truth)) throw Panic(RST_ERR_SHAPE, "CrossEntropyLoss: pred/truth shapes");
     Array2 g(pred.nrows(), pred.ncols());
     double loss = 0.0, acc = 0.0;
-    check(rst_cross_entropy_accuracy(pred.engine(), pred.data(), truth.data(), g.data(), pred.nrows(),
-                                     pred.ncols(), &loss, &acc));
+    const auto& through = pred.storage()->loss_through;  // logits of a compiled Sequential
+    if (!(through && through(pred, truth, g, &loss, &acc)))
+      check(rst_cross_entropy_accuracy(pred.engine(), pred.data(), truth.data(), g.data(), pred.nrows(),
+                                       pred.ncols(), &loss, &acc));
     detail::AccuracyMemo& memo = detail::accuracy_memo();
     memo.pred.reset();
     if (!pred.storage()->rewritten_in_place && !truth.storage()->rewritten_in_place) {

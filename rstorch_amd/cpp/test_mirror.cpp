@@ -145,7 +145,10 @@ int main() {
       };
       EXPECT(panics([&] { fast.backward(Array2::ones(4, 6)); }));
       EXPECT(panics([&] { fast.parameters(); }));
-      for (int step = 0; step < 6; ++step) {
+      // (from the second step on the compiled form takes the loop for a training loop and launches the
+      // input gradients of the upper layers behind the loss, before the host has it: steps 5-7 make it
+      // drop or overwrite them)
+      for (int step = 0; step < 9; ++step) {
         Array2 x = Array2::normal(48, 24, 5, 10 + step % 2, 0.0, 1.0), y = Array2::one_hot(48, 6, 5, 20 + step % 2);
         Array2 pf = fast.forward(x), ps = slow.forward(x);
         EXPECT(pf.to_host() == ps.to_host());
@@ -159,6 +162,17 @@ int main() {
           EXPECT(gf.to_host() == gs.to_host());
           EXPECT(same_parameters());
           continue;
+        } else if (step == 5) {  // somebody looks at the loss gradient before it goes into backward
+          Array2 gf = lf.backward(), gs = ls.backward();
+          EXPECT(gf.to_host() == gs.to_host());
+          fast.backward(gf); slow.backward(gs);
+        } else if (step == 6) {  // another gradient than the loss's own goes into backward
+          (void)lf.backward(); (void)ls.backward();
+          Array2 other = Array2::normal(48, 6, 5, 40, 0.0, 1.0);
+          fast.backward(other.clone()); slow.backward(other.clone());
+        } else if (step == 7) {  // the loss is computed twice on the same logits; the second gradient is used
+          EXPECT(lf.forward(pf.clone(), y.clone()) == ls.forward(ps.clone(), y.clone()));
+          fast.backward(lf.backward()); slow.backward(ls.backward());
         } else {
           fast.backward(lf.backward()); slow.backward(ls.backward());
         }

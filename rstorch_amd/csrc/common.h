@@ -250,6 +250,10 @@ int static_scratch_setup(int device, hipStream_t stream);
 int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, const double* truth,
                          double* grad_out, double* prob_out, size_t rows, size_t cols,
                          double* host_loss, bool* hits_done = nullptr);
+// the arg-max agreement count of pred / truth into the engine's pinned hit word: enqueues, runs
+// `ahead` (launches the caller wants on the stream before the host waits), waits
+int engine_accuracy(rst_engine* e, const double* pred, const double* truth, size_t rows, size_t cols,
+                    int (*ahead)(void*) = nullptr, void* ahead_arg = nullptr);
 // the fused classifier head (launch_head_ce) with the engine's loss words, mirror and ticket
 int engine_head_cross_entropy(rst_engine* e, double* row_loss, const double* h, const double* w,
                               const double* bias, const double* truth, double* logits, double* grad,

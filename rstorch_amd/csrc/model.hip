@@ -71,6 +71,10 @@ struct rst_model {
   bool forward_valid = false;
   bool loss_grad_valid = false;
   bool grads_valid = false;
+  // rst_model_loss_accuracy_to has launched the input gradients of every Linear above the first from
+  // the gradient at this address; a backward pass from the same address only launches the rest
+  bool inputs_done = false;
+  const double* inputs_grad = nullptr;
   // the captured training step (one graph launch instead of ~10 kernel launches)
   // (a few graphs are kept: a staged input pipeline alternates between its slots' buffers)
   // 0: plain launches; 1: replay; 2: replay when the step has many launches (deep_enough)
@@ -237,7 +241,10 @@ int next_non_identity(const rst_model* m, int i) {
 // it, the Linear in front of it.  -1: none.
 struct Tail {
   int head = -1, hidden = -1;
-  bool takes(int i) const { return i >= 0 && (i == head || i == hidden); }
+  // every Linear but `first` (whose input gradient is the model's): launched ahead of the backward pass
+  bool above_first = false;
+  int first = -1;
+  bool takes(int i) const { return i >= 0 && (i == head || i == hidden || (above_first && i != first)); }
 };
 
 // tail: its layers' inputs are noted, nothing is launched for them.
@@ -302,6 +309,7 @@ int do_forward(rst_model* m, const double* x, size_t batch, double* final_out = 
   m->logits = cur;
   m->forward_valid = true;
   m->loss_grad_valid = false;
+  m->inputs_done = false;
   return RST_OK;
 }
 
@@ -378,6 +386,20 @@ int do_head(rst_model* m, Tail tail, const double* truth) {
   RST_TRY(prof_end(m));
   m->loss_grad_valid = true;
   return RST_OK;
+}
+
+// grad_input[batch, in] = grad . weight (linear.rs:68), under the mask of a preceding ReLU
+GemmDesc input_gradient_desc(rst_model* m, const Layer& l, const double* grad, double* dest, bool mask) {
+  GemmDesc dx{};
+  dx.A = grad; dx.B = l.w; dx.C = dest;
+  dx.M = (int)m->batch; dx.N = (int)l.in; dx.K = (int)l.out;
+  dx.lda = (long)l.out; dx.ldb = (long)l.in; dx.ldc = (long)l.in;
+  dx.a_kc = true; dx.b_kc = false;
+  dx.epilogue = mask ? EPI_MASK : EPI_NONE;
+  dx.mask = mask ? l.input : nullptr;  // the ReLU's output is this layer's input
+  dx.ldmask = (long)l.in;
+  dx.workspace = m->engine->d_gemm_ws; dx.workspace_count = m->engine->gemm_ws_count;
+  return dx;
 }
 
 // fused_lr != NULL: every weight-gradient launch also applies the SGD update to its layer
@@ -498,14 +520,7 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
     GemmDesc dx{};
     double dx_bytes = 0.0;
     if (wanted) {
-      dx.A = cur; dx.B = l.w; dx.C = gin;
-      dx.M = (int)batch; dx.N = (int)l.in; dx.K = (int)l.out;
-      dx.lda = (long)l.out; dx.ldb = (long)l.in; dx.ldc = (long)l.in;
-      dx.a_kc = true; dx.b_kc = false;
-      dx.epilogue = mask ? EPI_MASK : EPI_NONE;
-      dx.mask = mask ? l.input : nullptr;  // the ReLU's output is this layer's input
-      dx.ldmask = (long)l.in;
-      dx.workspace = e->d_gemm_ws; dx.workspace_count = e->gemm_ws_count;
+      dx = input_gradient_desc(m, l, cur, gin, mask);
       dx_bytes = 8.0 * ((double)batch * l.out + (double)l.in * l.out +
                         (double)batch * l.in * (mask ? 2.0 : 1.0));
     }
@@ -560,6 +575,56 @@ int do_backward(rst_model* m, const double* grad, int need_input_grad, const dou
   m->forward_valid = false;
   m->loss_grad_valid = false;
   m->grads_valid = true;
+  m->inputs_done = false;
+  return RST_OK;
+}
+
+// The part of a backward pass that changes nothing a caller can see: the input gradients of every
+// Linear above the first, from `grad`, into the model's own buffers.  For small models only - every
+// weight gradient waits for the shared grid at the end of backward anyway, so launching these first
+// leaves the order of the launches as it is - whose ReLU layers all sit right below a Linear.
+bool inputs_ahead_possible(rst_model* m) {
+  if (!m->forward_valid || m->profiling || m->batch == 0) return false;
+  const int n = (int)m->layers.size();
+  int linears = 0;
+  for (int i = 0; i < n; ++i) {
+    const Layer& l = m->layers[i];
+    if (l.kind == RST_LAYER_RELU) {
+      const int nx = next_non_identity(m, i);
+      if (nx < 0 || m->layers[nx].kind != RST_LAYER_LINEAR) return false;  // (a launch of its own in backward)
+    }
+    if (l.kind != RST_LAYER_LINEAR) continue;
+    ++linears;
+    GemmDesc d{};
+    d.A = m->loss_grad; d.B = l.input; d.C = l.gw;
+    d.M = (int)l.out; d.N = (int)l.in; d.K = (int)m->batch;
+    d.lda = (long)l.out; d.ldb = (long)l.in; d.ldc = (long)l.in;
+    d.a_kc = false; d.b_kc = false;
+    d.epilogue = EPI_DIVIDE; d.divisor = (double)m->batch;
+    d.workspace = m->engine->d_gemm_ws; d.workspace_count = m->engine->gemm_ws_count;
+    if (l.in == 0 || !can_group_gemm(d)) return false;
+  }
+  return linears >= 2;
+}
+
+int do_backward_inputs(rst_model* m, const double* grad) {
+  rst_engine* e = m->engine;
+  const int n = (int)m->layers.size();
+  int first_linear = -1;
+  for (int i = 0; i < n; ++i)
+    if (m->layers[i].kind == RST_LAYER_LINEAR) { first_linear = i; break; }
+  const double* cur = grad;
+  for (int i = n - 1; i > first_linear; --i) {
+    Layer& l = m->layers[i];
+    if (l.kind != RST_LAYER_LINEAR) continue;  // (every ReLU is taken by the Linear above it)
+    const int pv = prev_non_identity(m, i);
+    const bool mask = pv >= 0 && m->layers[pv].kind == RST_LAYER_RELU;
+    RST_TRY(launch_gemm(e->stream, input_gradient_desc(m, l, cur, l.grad_in_buf, mask)));
+    if (mask) m->layers[pv].backward_absorbed = true;
+    cur = l.grad_in_buf;
+  }
+  m->inputs_done = true;
+  m->inputs_grad = grad;
   return RST_OK;
 }
 
@@ -893,8 +958,52 @@ int rst_model_backward_to(rst_model* m, const double* grad, double* input_grad_o
   if (!grad) return fail(RST_ERR_INVALID_ARGUMENT, "grad is null");
   const int need = input_grad_out != nullptr;
   const bool fused = apply_sgd != 0 && m->fuse_sgd;
-  RST_TRY(do_backward(m, grad, need, nullptr, fused ? &lr : nullptr, input_grad_out));
+  Tail done;
+  if (m->inputs_done && m->inputs_grad == grad && m->forward_valid && !m->profiling) {
+    // the input gradients above the first Linear are in their buffers already
+    done.above_first = true;
+    for (int i = 0; i < (int)m->layers.size() && done.first < 0; ++i)
+      if (m->layers[i].kind == RST_LAYER_LINEAR) done.first = i;
+  }
+  RST_TRY(do_backward(m, grad, need, nullptr, fused ? &lr : nullptr, input_grad_out, done));
   if (apply_sgd && !fused) RST_TRY(do_sgd(m, lr));
+  return RST_OK;
+}
+
+int rst_model_loss_accuracy_to(rst_model* m, const double* pred, const double* truth, double* grad_out,
+                               int inputs_ahead, double* host_loss, double* host_accuracy) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  rst_engine* e = m->engine;
+  RST_TRY(engine_activate(e));
+  if (!pred || !truth || !grad_out || !host_loss)
+    return fail(RST_ERR_INVALID_ARGUMENT, "loss_accuracy_to: null operand");
+  if (!m->forward_valid || pred != m->logits)
+    return fail(RST_ERR_STATE, "pred is not what the model's latest forward pass wrote");
+  const size_t rows = m->batch, cols = m->out_width;
+  bool hits_done = false;
+  RST_TRY(engine_cross_entropy(e, nullptr, pred, truth, grad_out, nullptr, rows, cols, nullptr,
+                               host_accuracy ? &hits_done : nullptr));
+  m->inputs_done = false;
+  // behind the loss on the stream, ahead of the host's wait for it
+  struct Ahead {
+    rst_model* m;
+    const double* grad;
+    static int run(void* p) {
+      Ahead* a = static_cast<Ahead*>(p);
+      return do_backward_inputs(a->m, a->grad);
+    }
+  } ahead{m, grad_out};
+  const bool go = inputs_ahead != 0 && inputs_ahead_possible(m);
+  if (host_accuracy && !hits_done) RST_TRY(engine_accuracy(e, pred, truth, rows, cols, go ? &Ahead::run : nullptr, &ahead));
+  else if (go) RST_TRY(do_backward_inputs(m, grad_out));
+  const int status = rst_loss_value(e, host_loss);
+  if (host_accuracy) *host_accuracy = (double)(*static_cast<volatile unsigned long long*>(e->h_hits)) / (double)rows;
+  return status;
+}
+
+int rst_model_discard_inputs(rst_model* m) {
+  if (!m) return fail(RST_ERR_INVALID_ARGUMENT, "model is null");
+  m->inputs_done = false;
   return RST_OK;
 }
 

@@ -8,16 +8,16 @@
 using namespace rst;
 
 namespace rst {
-namespace {
 
-__global__ void reset_softmax_flag_kernel(int* flags) { flags[2] = 0; }
-
-// enqueues the arg-max agreement count of pred / truth and waits until it is in the pinned hit word
-int engine_accuracy(rst_engine* e, const double* pred, const double* truth, size_t rows, size_t cols) {
+// enqueues the arg-max agreement count of pred / truth and waits until it is in the pinned hit word;
+// `ahead` (if any) runs between the two: launches that the caller wants on the stream before the wait
+int engine_accuracy(rst_engine* e, const double* pred, const double* truth, size_t rows, size_t cols,
+                    int (*ahead)(void*), void* ahead_arg) {
   bool mirrored = false;
   const unsigned ticket = engine_next_ticket(e);
   RST_TRY(launch_accuracy(e->stream, pred, truth, rows, cols, e->d_hits, e->hd_hits, &mirrored, e->hd_slots,
                           ticket));
+  if (ahead) RST_TRY(ahead(ahead_arg));
   if (mirrored) {
     RST_TRY(engine_wait_ticket(e, ticket, 2));
     *e->h_hits = e->h_slots[1].count;  // (the record and the plain word hold the same count; only the record is certain to be there)
@@ -28,6 +28,10 @@ int engine_accuracy(rst_engine* e, const double* pred, const double* truth, size
   RST_HIP(hipStreamSynchronize(e->stream));
   return RST_OK;
 }
+
+namespace {
+
+__global__ void reset_softmax_flag_kernel(int* flags) { flags[2] = 0; }
 
 int check_dim(size_t v, const char* what) {
   if (v > (size_t)INT_MAX) return fail(RST_ERR_UNSUPPORTED, "%s = %zu exceeds 2^31-1", what, v);

@@ -288,6 +288,9 @@ class _Plan:
         self.in_width, self.out_width = self.device.in_width, self.device.out_width
         self.x = self.out = None      # the forward pass whose caches are live (kept alive until backward)
         self.pending = None           # (gradient, weak reference to the deferred input gradient)
+        # a loss on the logits that a backward pass followed: the next step is taken for one of a training loop
+        self._training = self._loss_seen = self._backward_followed = False
+        self._inputs_from = None      # weak reference to the loss gradient that input gradients were launched from
 
     def valid_for(self, layers):
         return self.key == tuple(id(l) for l in layers) and all(l._home is self for l in self.linears)
@@ -301,7 +304,33 @@ class _Plan:
         out = self.engine.empty(x.rows, self.out_width)
         _ffi.check(self.engine.lib.rst_model_forward_to(self.device.handle, x.ptr, x.rows, out.ptr))
         self.x, self.out = x, out
+        self._training = self._loss_seen and self._backward_followed
+        self._loss_seen = self._backward_followed = False
+        self._inputs_from = None
+        out._loss_through = weakref.WeakMethod(self._loss_through)
         return out
+
+    def _loss_through(self, pred, truth, grad):
+        """CrossEntropyLoss.forward on the logits of the latest forward pass: the loss, or None when
+        this is not the array forward() returned.  In a training loop the input gradients of the
+        layers above the first are launched behind the loss before the host waits for it
+        (rst_model_loss_accuracy_to), and the backward pass skips them if the gradient array reaches
+        backward() without anybody having looked at it."""
+        if self.x is None or self.pending is not None or pred is not self.out or pred.shape != truth.shape:
+            return None
+        loss = ctypes.c_double()
+        _ffi.check(self.engine.lib.rst_model_loss_accuracy_to(
+            self.device.handle, pred.ptr, truth.ptr, grad.ptr, 1 if self._training else 0, ctypes.byref(loss), None))
+        self._loss_seen = True
+        if self._training:
+            self._inputs_from = weakref.ref(grad)
+            grad._before_access = self._inputs_touched
+        return loss.value
+
+    def _inputs_touched(self):
+        """Somebody looked at (and may have rewritten) the gradient the input gradients were launched from."""
+        _ffi.check(self.engine.lib.rst_model_discard_inputs(self.device.handle))
+        self._inputs_from = None
 
     def backward(self, gradient):
         if self.x is None or self.pending is not None:  # no forward yet, or its caches are taken
@@ -312,6 +341,7 @@ class _Plan:
                                   % (g.shape, (self.x.rows, self.out_width)))
         gin = Array2(self.engine, self.x.rows, self.in_width, resolver=self._resolve_input_grad)
         self.pending = (g, weakref.ref(gin))
+        self._backward_followed = True
         for l in self.linears:
             l._has_grad = True
         return gin
@@ -330,6 +360,12 @@ class _Plan:
         if gin is not None:
             gin._resolver = None
             gin._materialise()
+        if self._inputs_from is not None:
+            if self._inputs_from() is g:   # untouched since: our own access keeps the launched gradients
+                g._before_access = None
+            else:
+                self._inputs_touched()
+            self._inputs_from = None
         _ffi.check(self.engine.lib.rst_model_backward_to(
             self.device.handle, g.ptr, gin._ptr if gin is not None else None, 1 if apply_sgd else 0, float(lr)))
         self.x = self.out = None  # the caches are consumed

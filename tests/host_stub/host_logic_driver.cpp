@@ -125,6 +125,36 @@ int main() {
     OK(rst_free(e, t));
   }
 
+  // ---- the README loop's calls: forward, loss + accuracy with the upper layers' input gradients launched
+  //      ahead of the wait, backward with the update; and every way of not following that up -----------------
+  for (size_t batch : {(size_t)32, (size_t)8192}) {
+    rst_model* m = build(e, readme);
+    double* x = dev(e, batch * 784);
+    double* t = dev(e, batch * 10);
+    double* logits = dev(e, batch * 10);
+    double* g = dev(e, batch * 10);
+    double* g2 = dev(e, batch * 10);
+    double* gin = dev(e, batch * 784);
+    double loss = 0.0, acc = 0.0;
+    EXPECT(rst_model_loss_accuracy_to(m, logits, t, g, 1, &loss, &acc), RST_ERR_STATE);  // no forward pass yet
+    for (int step = 0; step < 6; ++step) {
+      OK(rst_model_forward_to(m, x, batch, logits));
+      if (step == 0) EXPECT(rst_model_loss_accuracy_to(m, g2, t, g, 1, &loss, &acc), RST_ERR_STATE);  // not its logits
+      if (step == 0) EXPECT(rst_model_loss_accuracy_to(m, logits, t, g, 1, nullptr, &acc), RST_ERR_INVALID_ARGUMENT);
+      OK(rst_model_loss_accuracy_to(m, logits, t, g, step != 1, &loss, step == 2 ? nullptr : &acc));
+      if (step == 3) OK(rst_model_discard_inputs(m));
+      if (step == 4) OK(rst_model_loss_accuracy_to(m, logits, t, g2, 1, &loss, &acc));  // the loss taken twice
+      OK(rst_model_backward_to(m, step == 4 ? g2 : step == 5 ? g2 : g, step % 2 ? gin : nullptr, 1, 0.01));
+      EXPECT(rst_model_backward_to(m, g, nullptr, 1, 0.01), RST_ERR_STATE);  // the caches are consumed
+    }
+    OK(rst_model_forward_to(m, x, batch, logits));  // a forward pass that nothing follows
+    OK(rst_model_loss_accuracy_to(m, logits, t, g, 1, &loss, &acc));
+    OK(rst_model_forward_to(m, x, batch, logits));
+    OK(rst_model_backward_to(m, g, nullptr, 0, 0.0));  // (the same address, after another forward: all of it runs)
+    OK(rst_model_destroy(m));
+    for (double* p : {x, t, logits, g, g2, gin}) OK(rst_free(e, p));
+  }
+
   // ---- two models and an operator-level cross entropy sharing one engine -------------------------
   {
     rst_model* a = build(e, readme);

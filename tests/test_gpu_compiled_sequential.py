@@ -71,6 +71,45 @@ def test_readme_loop_compiled_equals_layer_by_layer(engine, oracle, name, spec, 
         assert rel_err(wf, rp) <= 1e-10
 
 
+@pytest.mark.parametrize("name,spec,batch", [("readme_b32", README_MLP, 32), ("readme_b257", README_MLP, 257),
+                                             ("ragged", [("linear", 13, 37), ("relu",), ("linear", 37, 5)], 19)])
+def test_training_loop_on_the_logits_themselves(engine, oracle, name, spec, batch):
+    """loss.forward(pred, y) on the very array forward() returned: from the second step on the compiled
+    form launches the upper layers' input gradients behind the loss, before the host has it.  Nothing
+    observable changes - also when the gradient is looked at, replaced or rewritten on its way into
+    backward(), or the loss is taken twice."""
+    import rstorch_amd as rs
+    fast, slow, _ = twins(rs, oracle, spec, 0xA11)
+    n_in = [l for l in spec if l[0] == "linear"][0][1]
+    n_out = [l for l in spec if l[0] == "linear"][-1][2]
+    loss_f, loss_s = rs.CrossEntropyLoss.new(), rs.CrossEntropyLoss.new()
+    opt_f, opt_s = rs.SGD.new(0.05), rs.SGD.new(0.05)
+    for step in range(8):
+        x, y = batch_data(oracle, batch, n_in, n_out, 9, step % 3, False)
+        pf, ps = fast.forward(x), slow.forward(x)
+        assert loss_f.forward(pf, y) == loss_s.forward(ps, y), step
+        gf, gs = loss_f.backward(), loss_s.backward()
+        if step == 3:    # somebody looks at the gradient
+            assert np.array_equal(gf.to_numpy(), gs.to_numpy())
+        if step == 4:    # somebody rewrites it in place
+            half = 0.5 * gs.to_numpy()
+            gf.assign(half)
+            gs.assign(half)
+        if step == 5:    # another array goes into backward
+            gf = gs = engine.from_numpy(np.ones((batch, n_out)))
+        if step == 6:    # the loss is taken a second time; its gradient is the one used
+            assert loss_f.forward(pf, y) == loss_s.forward(ps, y)
+            gf, gs = loss_f.backward(), loss_s.backward()
+        kept_f, kept_s = fast.backward(gf), slow.backward(gs)
+        if step == 7:    # the gradient with respect to the input is kept and read
+            assert np.array_equal(kept_f.to_numpy(), kept_s.to_numpy())
+        opt_f.step(fast)
+        opt_s.step(slow)
+        for i, ((wf, g1), (ws, g2)) in enumerate(zip(params_np(fast), params_np(slow))):
+            assert np.array_equal(g1, g2), "gradient %d, step %d" % (i, step)
+            assert np.array_equal(wf, ws), "parameter %d, step %d" % (i, step)
+
+
 def test_the_input_gradient_is_computed_only_if_somebody_keeps_it(engine, oracle):
     import rstorch_amd as rs
     spec = [("linear", 24, 40), ("relu",), ("linear", 40, 6)]
