@@ -442,7 +442,9 @@ def readme_loops():
                     "model.backward(loss.backward()) -> optim.step(model) through the module interface of the C++ "
                     "mirror; the loss and the accuracy are read back every step.  compiled: the Sequential runs "
                     "as a device model (backward deferred to the optimiser step, SGD inside the weight-gradient "
-                    "launches, the first layer's input gradient skipped because the loop drops it); "
+                    "launches, the first layer's input gradient skipped because the loop drops it; on small "
+                    "networks the upper layers' input gradients are launched behind the loss before the host "
+                    "waits for it); "
                     "layer_by_layer: one call per layer, SGD as a pass of its own"}
     for config in ("C0", "C1", "C2", "C4"):
         log("README loop, %s ..." % config)
