@@ -564,6 +564,9 @@ class Plan : public std::enable_shared_from_this<Plan> {
     std::shared_ptr<Plan> self = shared_from_this();
     std::weak_ptr<Plan> weak = self;
     auto owed = [weak] { if (auto p = weak.lock()) p->flush(); };
+    // a look at (or a write into) a parameter between the loss and the backward pass: input gradients
+    // launched ahead were computed with the weights of before
+    auto touched = [weak] { if (auto p = weak.lock()) p->parameters_touched(); };
     for (size_t i = 0; i < linears_.size(); ++i) {
       Linear* l = linears_[i];
       double *w, *gw, *b, *gb;
@@ -578,8 +581,8 @@ class Plan : public std::enable_shared_from_this<Plan> {
         check(rst_copy(engine_->handle(), gw, l->grad_weight().data(), nw));
         check(rst_copy(engine_->handle(), gb, l->grad_bias().data(), nb));
       }
-      l->rehome(self, Array2::view(engine_, w, l->output_size(), l->input_size(), self),
-                Array2::view(engine_, b, 1, l->output_size(), self),
+      l->rehome(self, Array2::view(engine_, w, l->output_size(), l->input_size(), self, touched),
+                Array2::view(engine_, b, 1, l->output_size(), self, touched),
                 Array2::view(engine_, gw, l->output_size(), l->input_size(), self, owed),
                 Array2::view(engine_, gb, 1, l->output_size(), self, owed));
     }
@@ -589,6 +592,10 @@ class Plan : public std::enable_shared_from_this<Plan> {
   void inputs_touched() {
     rst_model_discard_inputs(model_);
     inputs_from_.reset();
+  }
+
+  void parameters_touched() {
+    if (!inputs_from_.expired()) inputs_touched();
   }
 
   void resolve_input_gradient(Array2::Storage& s) {

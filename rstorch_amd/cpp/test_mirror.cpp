@@ -170,6 +170,15 @@ int main() {
           (void)lf.backward(); (void)ls.backward();
           Array2 other = Array2::normal(48, 6, 5, 40, 0.0, 1.0);
           fast.backward(other.clone()); slow.backward(other.clone());
+        } else if (step == 8) {  // a parameter is rewritten between the loss and the backward pass
+          for (Sequential* m : {&fast, &slow}) {
+            Parameters ps = m->parameters();
+            Array2& w = *ps.iter()[4].parm;  // the last Linear's weight: its input gradient must see the new one
+            std::vector<double> h = w.to_host();
+            for (double& v : h) v *= 0.5;
+            check(rst_upload(w.engine(), w.data(), h.data(), h.size()));
+          }
+          fast.backward(lf.backward()); slow.backward(ls.backward());
         } else if (step == 7) {  // the loss is computed twice on the same logits; the second gradient is used
           EXPECT(lf.forward(pf.clone(), y.clone()) == ls.forward(ps.clone(), y.clone()));
           fast.backward(lf.backward()); slow.backward(ls.backward());

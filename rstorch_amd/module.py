@@ -281,6 +281,9 @@ class _Plan:
                 _ffi.check(eng.lib.rst_copy(eng.handle, gw._ptr, l.grad_weight.ptr, gw.size))
                 _ffi.check(eng.lib.rst_copy(eng.handle, gb._ptr, l.grad_bias.ptr, gb.size))
             l.weight, l.bias = w, b
+            # a look at (or a write into) a parameter between the loss and the backward pass: input
+            # gradients launched ahead were computed with the weights of before
+            w._before_access = b._before_access = self._parameters_touched
             # reading a gradient first runs the backward pass that is still owed
             gw._before_access = gb._before_access = self.flush
             l.grad_weight, l.grad_bias = gw, gb
@@ -326,6 +329,10 @@ class _Plan:
             self._inputs_from = weakref.ref(grad)
             grad._before_access = self._inputs_touched
         return loss.value
+
+    def _parameters_touched(self):
+        if self._inputs_from is not None:
+            self._inputs_touched()
 
     def _inputs_touched(self):
         """Somebody looked at (and may have rewritten) the gradient the input gradients were launched from."""

@@ -84,11 +84,15 @@ def test_training_loop_on_the_logits_themselves(engine, oracle, name, spec, batc
     n_out = [l for l in spec if l[0] == "linear"][-1][2]
     loss_f, loss_s = rs.CrossEntropyLoss.new(), rs.CrossEntropyLoss.new()
     opt_f, opt_s = rs.SGD.new(0.05), rs.SGD.new(0.05)
-    for step in range(8):
+    for step in range(9):
         x, y = batch_data(oracle, batch, n_in, n_out, 9, step % 3, False)
         pf, ps = fast.forward(x), slow.forward(x)
         assert loss_f.forward(pf, y) == loss_s.forward(ps, y), step
         gf, gs = loss_f.backward(), loss_s.backward()
+        if step == 8:    # a parameter is rewritten between the loss and the backward pass
+            for m in (fast, slow):
+                w = list(m.parameters())[-2].parm  # the last Linear's weight: its input gradient must see the new one
+                w.assign(0.5 * w.to_numpy())
         if step == 3:    # somebody looks at the gradient
             assert np.array_equal(gf.to_numpy(), gs.to_numpy())
         if step == 4:    # somebody rewrites it in place
