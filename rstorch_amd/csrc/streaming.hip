@@ -347,6 +347,17 @@ __global__ __launch_bounds__(1024) void accuracy_small_kernel(const double* __re
   }
 }
 
+// The count of a multi-workgroup accuracy launch, from the device word into its host mirror and the
+// pinned result record (with the launch's ticket): the host then waits for exactly this result by
+// polling instead of copying it back and synchronising the stream - work that a caller has put on the
+// stream behind the accuracy (the input gradients of a coming backward pass) is not waited for.
+__global__ void publish_hits_kernel(const unsigned long long* __restrict__ hits, unsigned long long* hits_mirror,
+                                    ResultSlot* slots, unsigned ticket) {
+  const unsigned long long total = hits[0];
+  hits_mirror[0] = total;
+  store_result_slot(slots + 1, 0.0, total, true, 0u, ticket);
+}
+
 int launch_accuracy(hipStream_t s, const double* pred, const double* truth, size_t rows,
                     size_t cols, unsigned long long* hits, unsigned long long* hits_mirror,
                     bool* mirrored, ResultSlot* slots, unsigned ticket) {
@@ -367,6 +378,11 @@ int launch_accuracy(hipStream_t s, const double* pred, const double* truth, size
                          truth, rows, cols, hits);
   }
   RST_HIP(hipGetLastError());
+  if (hits_mirror && mirrored && slots) {
+    hipLaunchKernelGGL(publish_hits_kernel, dim3(1), dim3(1), 0, s, hits, hits_mirror, slots, ticket);
+    RST_HIP(hipGetLastError());
+    *mirrored = true;
+  }
   return RST_OK;
 }
 
