@@ -284,8 +284,10 @@ def test_cross_entropy_nan_logits_is_an_error(engine):
 def test_accuracy_first_maximum_wins(engine, oracle):
     import rstorch_amd as rs
     rng = np.random.default_rng(8)
-    # (the last three shapes take the one-workgroup-per-row kernel for wide rows)
-    for rows, cols in [(32, 10), (100, 1000), (5, 70), (9, 4096), (40, 4100), (12, 32768), (3, 4097)]:
+    # (the three shapes from (9, 4096) on take the one-workgroup-per-row kernel for wide rows, the last three
+    # the thread-per-row kernel for long batches of narrow rows)
+    for rows, cols in [(32, 10), (100, 1000), (5, 70), (9, 4096), (40, 4100), (12, 32768), (3, 4097),
+                       (9000, 10), (5000, 32), (4097, 17)]:
         pred = rng.integers(0, 4, size=(rows, cols)).astype(np.float64)  # many ties
         truth = np.zeros((rows, cols)); truth[np.arange(rows), rng.integers(0, cols, rows)] = 1.0
         truth[0, :] = 0.0
