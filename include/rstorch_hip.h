@@ -128,10 +128,10 @@ int rst_cross_entropy(rst_engine* engine, const double* pred, const double* trut
                       double* grad_out, double* prob_out, size_t rows, size_t cols,
                       double* host_loss);
 /* rst_cross_entropy with host_loss, and rst_accuracy(pred, truth) (src/utils.rs:55-65) with it: what
- * the README loop asks for back to back (README.md:66-67), answered after ONE wait.  A batch that a
- * single workgroup handles (up to 64 rows of up to 64 logits, 16 rows of up to 512) is counted by
- * the cross-entropy launch itself; otherwise the arg-max launch follows on the stream.  Same loss
- * bits as rst_cross_entropy, same count as rst_accuracy. */
+ * the README loop asks for back to back (README.md:66-67), answered after ONE wait.  Rows of up to
+ * 512 logits (256 when the arrays are not 16-byte aligned or the width is odd) are counted by the
+ * cross-entropy launches themselves; for wider rows the arg-max launch follows on the stream.  Same
+ * loss bits as rst_cross_entropy, same count as rst_accuracy. */
 int rst_cross_entropy_accuracy(rst_engine* engine, const double* pred, const double* truth,
                                double* grad_out, size_t rows, size_t cols, double* host_loss,
                                double* host_accuracy);

@@ -139,6 +139,9 @@ struct LossMirror {
   ResultSlot* slots = nullptr;
   unsigned ticket = 0;
   unsigned long long* hits = nullptr;
+  // device scratch, one word per workgroup of the row kernel, for the hit counts of a cross entropy
+  // on several workgroups (added up by the reduction launch); NULL: such a launch does not count
+  unsigned* group_hits = nullptr;
 };
 int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* grad_out,
                       double* prob_out, double* row_loss, double* loss, int* flags, size_t rows,

@@ -76,13 +76,19 @@ int engine_cross_entropy(rst_engine* e, double* row_loss, const double* pred, co
                          double* grad_out, double* prob_out, size_t rows, size_t cols,
                          double* host_loss, bool* hits_done) {
   if (rows == 0 || cols == 0) return fail(RST_ERR_SHAPE, "cross entropy of an empty batch");
+  unsigned* group_hits = nullptr;
   if (!row_loss) {  // the engine's own scratch; it moves when it grows, so nothing may keep its address
-    RST_TRY(engine_reserve_row_loss(e, rows));
+    // (with the hit count: a second stretch of the same scratch for the workgroups' counts)
+    RST_TRY(engine_reserve_row_loss(e, hits_done ? 2 * rows : rows));
     row_loss = e->d_row_loss;
+    if (hits_done) group_hits = reinterpret_cast<unsigned*>(e->d_row_loss + rows);
   }
   LossMirror mirror;
   RST_TRY(loss_mirror(e, &mirror));
-  if (hits_done) mirror.hits = e->hd_hits;
+  if (hits_done) {
+    mirror.hits = e->hd_hits;
+    mirror.group_hits = group_hits;
+  }
   RST_TRY(launch_softmax_ce(e->stream, pred, truth, grad_out, prob_out, row_loss, e->d_loss,
                             e->d_flags, rows, cols, mirror, hits_done));
   e->loss_with_hits = hits_done && *hits_done;

@@ -75,16 +75,18 @@ __device__ __forceinline__ double loss_term(double truth, double p) {
 // rows per workgroup.  SOLO: the whole batch (at most 64 rows) sits in one workgroup of 1024
 // threads, which then also finishes the loss the way loss_reduce_kernel would (same order of
 // additions, same bits), so that a small batch needs one launch instead of two.
-// ACC (with SOLO): the kernel also counts the rows whose first arg-max agrees between logits and truth
-// (utils.rs:44-65), which a training loop asks for right after the loss - one launch and one
-// round trip instead of two.
+// ACC (rows of at most 64 threads): the kernel also counts the rows whose first arg-max agrees between
+// logits and truth (utils.rs:44-65), which a training loop asks for right after the loss - one launch
+// and one round trip instead of two.  With SOLO the count goes out with the loss; otherwise every
+// workgroup leaves its count in mirror.group_hits[its number] and loss_reduce_kernel adds them up
+// (one word per workgroup: thousands of additions to one word would queue up behind each other).
 template <int TPR, int IPT, int VEC, bool CE, int BLOCK = 256, bool SOLO = false, bool ACC = false>
 __global__ __launch_bounds__(BLOCK) void softmax_rows_kernel(
     const double* __restrict__ z, const double* __restrict__ truth, double* __restrict__ grad,
     double* __restrict__ prob, double* __restrict__ row_loss, double* __restrict__ loss,
     int* __restrict__ flags, size_t rows, size_t cols, LossMirror mirror) {
   static_assert(BLOCK % TPR == 0 && (TPR <= 64 || BLOCK == TPR) && (!SOLO || (CE && BLOCK == 1024)) &&
-                (!ACC || (SOLO && TPR <= 64)), "unsupported shape");
+                (!ACC || (CE && TPR <= 64)), "unsupported shape");
   constexpr int RPB = BLOCK / TPR;
   __shared__ double red[3][TPR > 64 ? TPR / 64 : 1];
 
@@ -215,6 +217,21 @@ __global__ __launch_bounds__(BLOCK) void softmax_rows_kernel(
     lsum = group_reduce<TPR, SumOp>(lsum, red[2]);
     if (sub == 0 && row_ok) row_loss[row] = lsum;
     if (saw_nan) atomicOr(&flags[0], 1);
+    if (ACC) {
+      constexpr int W = TPR < 64 ? TPR : 64;
+#pragma unroll
+      for (int off = W / 2; off > 0; off >>= 1) {
+        argmax_combine(best_z, arg_z, __shfl_xor(best_z, off), __shfl_xor(arg_z, off));
+        argmax_combine(best_t, arg_t, __shfl_xor(best_t, off), __shfl_xor(arg_t, off));
+      }
+      __shared__ unsigned group_count;
+      if (threadIdx.x == 0) group_count = 0;
+      __syncthreads();
+      const unsigned long long agreeing = __ballot(sub == 0 && row_ok && arg_z == arg_t);
+      if ((threadIdx.x & 63) == 0 && agreeing != 0ull) atomicAdd(&group_count, (unsigned)__popcll(agreeing));
+      __syncthreads();
+      if (threadIdx.x == 0) mirror.group_hits[blockIdx.x] = group_count;
+    }
   } else {
     if (saw_nan) atomicOr(&flags[2], 1);
   }
@@ -385,12 +402,21 @@ __global__ __launch_bounds__(BLOCK) __attribute__((amdgpu_waves_per_eu(4, 4))) v
 
 // Second (tiny) launch of a cross entropy: loss = -(sum of the per-row sums) / rows in a fixed
 // order, one workgroup.  It also latches the NaN flag of the launch into flags[1] and re-arms
-// flags[0], so no reset launch is needed.
+// flags[0], so no reset launch is needed.  hit_groups > 0: the row kernel left the arg-max agreements of
+// its workgroups in mirror.group_hits[0 .. hit_groups); their sum goes out with the loss.
 __global__ __launch_bounds__(1024) void loss_reduce_kernel(const double* __restrict__ row_loss,
                                                           double* __restrict__ loss,
                                                           int* __restrict__ flags, size_t rows,
-                                                          LossMirror mirror) {
+                                                          LossMirror mirror, unsigned hit_groups) {
   __shared__ double red[1024 / 64];
+  __shared__ unsigned hit_total;
+  if (hit_groups > 0) {
+    if (threadIdx.x == 0) hit_total = 0;
+    __syncthreads();
+    unsigned mine = 0;
+    for (unsigned g = threadIdx.x; g < hit_groups; g += 1024) mine += mirror.group_hits[g];
+    if (mine != 0) atomicAdd(&hit_total, mine);  // (an integer count: any order)
+  }
   double s = 0.0;
   for (size_t r = threadIdx.x; r < rows; r += 1024) s += row_loss[r];
   s = group_reduce<1024, SumOp>(s, red);
@@ -400,7 +426,8 @@ __global__ __launch_bounds__(1024) void loss_reduce_kernel(const double* __restr
     loss[0] = l;
     flags[1] = nan_seen;
     flags[0] = 0;
-    publish(mirror, l, nan_seen, false, 0);
+    // (group_reduce above ends in a barrier of the whole workgroup: every addition to hit_total is in)
+    publish(mirror, l, nan_seen, hit_groups > 0, hit_groups > 0 ? (unsigned long long)hit_total : 0ull);
   }
 }
 
@@ -851,7 +878,7 @@ __global__ __launch_bounds__(256) void softmax_jacobian_kernel(double* __restric
 template <int TPR, int IPT, int VEC>
 int launch_rows(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
                 double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce,
-                LossMirror mirror, bool* loss_done, bool* hits_done) {
+                LossMirror mirror, bool* loss_done, bool* hits_done, unsigned* hit_groups) {
   constexpr int BLOCK = 256;
   constexpr int RPB = BLOCK / TPR;
   size_t blocks = (rows + RPB - 1) / RPB;
@@ -868,6 +895,16 @@ int launch_rows(hipStream_t s, const double* z, const double* t, double* grad, d
                            z, t, grad, prob, row_loss, loss, flags, rows, cols, mirror);
       }
       *loss_done = true;
+      RST_HIP(hipGetLastError());
+      return RST_OK;
+    }
+  }
+  if constexpr (TPR <= 64) {
+    if (ce && mirror.hits && mirror.group_hits) {  // counted per workgroup; the reduction launch publishes the sum with the loss
+      hipLaunchKernelGGL((softmax_rows_kernel<TPR, IPT, VEC, true, BLOCK, false, true>), dim3((unsigned)blocks),
+                         dim3(BLOCK), 0, s, z, t, grad, prob, row_loss, loss, flags, rows, cols, mirror);
+      *hits_done = true;
+      *hit_groups = (unsigned)blocks;
       RST_HIP(hipGetLastError());
       return RST_OK;
     }
@@ -899,11 +936,11 @@ int launch_wide(hipStream_t s, const double* z, const double* t, double* grad, d
 template <int VEC>
 int dispatch(hipStream_t s, const double* z, const double* t, double* grad, double* prob,
              double* row_loss, double* loss, int* flags, size_t rows, size_t cols, bool ce,
-             LossMirror mirror, bool* loss_done, bool* hits_done) {
+             LossMirror mirror, bool* loss_done, bool* hits_done, unsigned* hit_groups) {
   const size_t units = cols / VEC;  // vectors per row
-  if (units <= 16 * 2) return launch_rows<16, 2, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done);
-  if (units <= 64 * 4) return launch_rows<64, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done);
-  if (units <= 256 * 4) return launch_rows<256, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done);
+  if (units <= 16 * 2) return launch_rows<16, 2, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done, hit_groups);
+  if (units <= 64 * 4) return launch_rows<64, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done, hit_groups);
+  if (units <= 256 * 4) return launch_rows<256, 4, VEC>(s, z, t, grad, prob, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done, hit_groups);
   // measured on 32 Mi logits: 256 threads per row are ahead below about 12 Ki columns, 512 above
   if (cols < 12288) return launch_wide<256, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
   return launch_wide<512, VEC>(s, z, t, grad, prob, row_loss, flags, rows, cols, ce);
@@ -914,13 +951,13 @@ inline bool aligned16(const void* p) { return reinterpret_cast<uintptr_t>(p) % 1
 // The row kernel of a softmax or cross entropy; *loss_done tells whether it finished the loss too.
 int launch_row_kernel(hipStream_t s, const double* z, const double* t, double* grad_out, double* prob_out,
                       double* row_loss, double* loss, int* flags, size_t rows, size_t cols,
-                      LossMirror mirror, bool* loss_done, bool* hits_done) {
+                      LossMirror mirror, bool* loss_done, bool* hits_done, unsigned* hit_groups) {
   const bool ce = grad_out != nullptr;
   const bool vec = cols % 2 == 0 && aligned16(z) && (!ce || (aligned16(t) && aligned16(grad_out))) &&
                    (!prob_out || aligned16(prob_out));
   *loss_done = false;
-  if (vec) return dispatch<2>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done);
-  return dispatch<1>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done);
+  if (vec) return dispatch<2>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done, hit_groups);
+  return dispatch<1>(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, ce, mirror, loss_done, hits_done, hit_groups);
 }
 
 }  // namespace
@@ -937,9 +974,10 @@ int launch_softmax_ce(hipStream_t s, const double* z, const double* t, double* g
   if (rows == 0 || cols == 0) return RST_OK;
   const bool ce = grad_out != nullptr;
   bool loss_done = false;
-  RST_TRY(launch_row_kernel(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, mirror, &loss_done, hits_done));
+  unsigned hit_groups = 0;  // workgroups of the row kernel that left a hit count for the reduction launch
+  RST_TRY(launch_row_kernel(s, z, t, grad_out, prob_out, row_loss, loss, flags, rows, cols, mirror, &loss_done, hits_done, &hit_groups));
   if (ce && !loss_done) {
-    hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(1024), 0, s, row_loss, loss, flags, rows, mirror);
+    hipLaunchKernelGGL(loss_reduce_kernel, dim3(1), dim3(1024), 0, s, row_loss, loss, flags, rows, mirror, hit_groups);
     RST_HIP(hipGetLastError());
   }
   return RST_OK;

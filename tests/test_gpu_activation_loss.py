@@ -308,7 +308,10 @@ def test_accuracy_first_maximum_wins(engine, oracle):
 # wait.  One workgroup's worth of rows is counted inside the cross-entropy launch (first shapes), the
 # others by the arg-max kernels that follow it on the stream.
 @pytest.mark.parametrize("rows,cols", [(32, 10), (1, 2), (64, 64), (16, 512), (7, 33), (65, 10), (3000, 1000),
-                                       (8192, 10), (40, 4100), (8, 32768)])
+                                       (8192, 10), (40, 4100), (8, 32768),
+                                       # several workgroups of rows of at most 64 threads: counted by the row
+                                       # kernel, published by the reduction launch
+                                       (300, 100), (5000, 64), (2000, 512), (1000, 33), (70, 257)])
 def test_cross_entropy_with_accuracy_in_one_wait(engine, oracle, rows, cols):
     import ctypes
     from rstorch_amd import _ffi
