@@ -343,7 +343,7 @@ int rst_cross_entropy_accuracy(rst_engine* e, const double* pred, const double* 
     return fail(RST_ERR_INVALID_ARGUMENT, "cross_entropy_accuracy: null operand");
   bool hits_done = false;
   RST_TRY(engine_cross_entropy(e, nullptr, pred, truth, grad_out, nullptr, rows, cols, nullptr, &hits_done));
-  // a batch that one workgroup handles is counted by the cross-entropy launch itself; otherwise
+  // rows of at most 64 threads are counted by the cross-entropy launches themselves; for wider rows
   // the arg-max kernels follow on the stream, and either way the host waits once
   if (!hits_done) RST_TRY(engine_accuracy(e, pred, truth, rows, cols));
   const int status = rst_loss_value(e, host_loss);
