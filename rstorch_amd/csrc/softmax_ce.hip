@@ -417,8 +417,18 @@ __global__ __launch_bounds__(1024) void loss_reduce_kernel(const double* __restr
     for (unsigned g = threadIdx.x; g < hit_groups; g += 1024) mine += mirror.group_hits[g];
     if (mine != 0) atomicAdd(&hit_total, mine);  // (an integer count: any order)
   }
+  // thread t adds rows t, t + 1024, ... in that order; eight of its loads are in flight at a time (the
+  // row sums were written by other XCDs: every load is a trip to memory)
   double s = 0.0;
-  for (size_t r = threadIdx.x; r < rows; r += 1024) s += row_loss[r];
+  size_t r = threadIdx.x;
+  for (; r + 7 * 1024 < rows; r += 8 * 1024) {
+    double t[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t[j] = row_loss[r + (size_t)j * 1024];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) s += t[j];
+  }
+  for (; r < rows; r += 1024) s += row_loss[r];
   s = group_reduce<1024, SumOp>(s, red);
   if (threadIdx.x == 0) {
     const double l = -s / (double)rows;
